@@ -1,0 +1,89 @@
+"""Device side of the cache: the pools of pages and the state slots."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .manager import CacheManager, PagedNeed, StateNeed
+
+
+@dataclass
+class CacheLayout:
+    """Which cache (one per writing call of the model's schedule) lives where.
+
+    ``paged_groups[g]`` is the need shared by the caches ``group_caches[g]`` (their order is the
+    order of planes in the group's pool); ``state_caches`` maps a cache id to its state need."""
+
+    paged_groups: List[PagedNeed]
+    group_caches: List[List[int]]
+    state_caches: Dict[int, StateNeed]
+
+    def locate(self, cache_id: int) -> Tuple[int, int]:
+        for g, ids in enumerate(self.group_caches):
+            if cache_id in ids:
+                return g, ids.index(cache_id)
+        raise KeyError(f"cache {cache_id} is not paged")
+
+
+class LayerCache:
+    """What a mixer sees of the cache in one step.
+
+    Paged: ``k_pool``/``v_pool`` [pages, kv_heads, page_size, head_dim] of this layer,
+    ``block_tables`` int32 [requests in the step, pages] (-1 = no page), ``slots`` int32 [tokens]
+    (where each token's entry goes), ``page_size``, and ``writes`` (False when this call only
+    reads a cache that another call fills).
+    State: ``state`` [max_requests, *shape]; the step's ``ctx.seq_slots`` index it."""
+
+    __slots__ = ("k_pool", "v_pool", "block_tables", "slots", "page_size", "writes", "state", "group")
+
+    def __init__(self):
+        self.k_pool = self.v_pool = self.block_tables = self.slots = self.state = None
+        self.page_size = 0
+        self.writes = True
+        self.group = -1
+
+
+class CacheStorage:
+    def __init__(self, layout: CacheLayout, manager: CacheManager, device, dtype: torch.dtype):
+        self.layout = layout
+        self.page_size = manager.page_size
+        self.device = device
+        self.dtype = dtype
+        self.pools: List[torch.Tensor] = []
+        for g, need in enumerate(layout.paged_groups):
+            n_pages = manager.allocators[g].num_pages
+            shape = (len(layout.group_caches[g]), 2, n_pages, need.n_kv_heads, self.page_size, need.head_dim)
+            self.pools.append(torch.zeros(shape, dtype=dtype, device=device))
+        self.states: Dict[int, torch.Tensor] = {}
+        for cid, need in layout.state_caches.items():
+            self.states[cid] = torch.zeros((manager.max_requests, *need.shape),
+                                           dtype=getattr(torch, need.dtype), device=device)
+
+    def bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in list(self.pools) + list(self.states.values()))
+
+    def reset_states(self, slots: Sequence[int]) -> None:
+        """Zero the state slots of requests that start in this step."""
+        if not slots or not self.states:
+            return
+        idx = torch.tensor(list(slots), dtype=torch.int64, device=self.device)
+        for t in self.states.values():
+            t.index_fill_(0, idx, 0)
+
+    def view(self, cache_id: int, ctx, writes: bool) -> LayerCache:
+        lc = LayerCache()
+        lc.writes = writes
+        if cache_id in self.states:
+            lc.state = self.states[cache_id]
+            return lc
+        g, plane = self.layout.locate(cache_id)
+        pool = self.pools[g]
+        lc.k_pool, lc.v_pool = pool[plane, 0], pool[plane, 1]
+        lc.block_tables = ctx.block_tables[g]
+        lc.slots = ctx.slots[g]
+        lc.page_size = self.page_size
+        lc.group = g
+        return lc

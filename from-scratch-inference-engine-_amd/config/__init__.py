@@ -1,0 +1,6 @@
+"""Typed model configurations read from config.json."""
+
+from .base import ConfigError, ModelConfig, read_config_json
+from .qwen2 import Qwen2Config
+
+__all__ = ["ConfigError", "ModelConfig", "Qwen2Config", "read_config_json"]

@@ -1,0 +1,63 @@
+// C interface of the kernel library (loaded from Python through ctypes).
+//
+// Conventions: every function returns 0 on success; otherwise fsie_last_error() describes the
+// refusal (sizes a kernel does not take are refused here, never computed wrongly).  Pointers are
+// device pointers unless said otherwise.  `dtype` is the type of activations and matrices:
+// 0 = float32, 1 = bfloat16.  All work is queued on `stream`; nothing synchronises.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define FSIE_GEMM_SKINNY_MAX_M 8
+
+// one attention work item = 8 int32
+#define FSIE_ATTN_ITEM_INTS 8
+#define FSIE_ATTN_ITEM_SEQ 0      // row of the block table
+#define FSIE_ATTN_ITEM_QROW 1     // first query row (token index within the step)
+#define FSIE_ATTN_ITEM_NQ 2       // query tokens in the tile (0 = padding item, skipped)
+#define FSIE_ATTN_ITEM_POS 3      // absolute position of the first query token
+#define FSIE_ATTN_ITEM_KBEGIN 4   // first key
+#define FSIE_ATTN_ITEM_KEND 5     // one past the last key
+#define FSIE_ATTN_ITEM_PARTIAL 6  // -1: write the output; >= 0: first partial slot of the tile
+// one merge item = 4 int32: {output row, first partial slot, number of splits, slot stride}
+#define FSIE_ATTN_MERGE_INTS 4
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* fsie_last_error(void);
+int fsie_version(void);
+// Name of the architecture the device code was built for and of the device present.
+int fsie_device_info(char* arch_out, int arch_len, int* n_compute_units);
+
+int fsie_embedding(const void* table, int dtype, const int32_t* ids, float* out, int n_tokens, int hidden,
+                   int vocab, hipStream_t stream);
+int fsie_rmsnorm(float* residual, const void* delta, const float* weight, void* out, const int32_t* rows,
+                 int n_rows, int hidden, float eps, int dtype, int write_back, hipStream_t stream);
+int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream);
+int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream);
+int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream);
+
+int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int32_t* slots, const double* inv_freq,
+                       const float* bias, void* k_pool, void* v_pool, int n_tokens, int n_heads, int n_kv, int head_dim,
+                       int rotary_dim, int page_size, int64_t pool_slots, int dtype, hipStream_t stream);
+
+int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, int N, int K, int dtype,
+              int out_f32, int kind, hipStream_t stream);
+
+int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                          const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
+                          void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,
+                          int window, float scale, int dtype, hipStream_t stream);
+int fsie_attention_merge(const float* partials, const int32_t* merges, int n_merges, void* out, int n_heads,
+                         int head_dim, int dtype, hipStream_t stream);
+int fsie_attention_scalar_tile_tokens(int n_heads, int n_kv);
+
+int fsie_sample(const float* logits, int n_rows, int vocab, const float* temperature, const int32_t* top_k,
+                const float* top_p, const double* uniform, int32_t* out, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,279 @@
+// Causal grouped-query attention over the pages of the cache: float32 arithmetic throughout
+// (products, softmax, sums), for float32 or bfloat16 storage.  It is the attention of the 32-bit
+// path and takes any head size up to 256.
+//
+// The host cuts the step into work items (api.h: FSIE_ATTN_ITEM_*): a tile of up to 16/gh query
+// tokens of one request, a range of keys, and where the result goes: the output (normalised), or a
+// partial record (unnormalised sum, running maximum, denominator) that attention_merge combines
+// when a key range was split over several items.  grid = (items, kv_heads * head_chunks); a block
+// holds rows = tokens x heads of one kv head's group (gh heads per chunk), four rows per wave.
+//
+// Page layout: [page][kv_head][slot][head_dim]; block_tables[seq * max_pages + i] = page id of the
+// request's i-th page, or -1 where a window has passed.
+#include "common.h"
+#include "api.h"
+
+#include <math.h>
+
+namespace {
+
+constexpr int kRows = 16;      // query rows per block
+constexpr int kKeys = 32;      // keys per tile
+constexpr int kMaxChunks = 8;  // head_dim <= 32 * 8
+
+__device__ __forceinline__ float half_wave_max(float v) {
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, FSIE_WAVE));
+    return v;
+}
+__device__ __forceinline__ float half_wave_sum(float v) {
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) v += __shfl_xor(v, off, FSIE_WAVE);
+    return v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void attention_scalar_kernel(
+    const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
+    const int32_t* __restrict__ block_tables, int max_pages, const int32_t* __restrict__ items,
+    T* __restrict__ out, float* __restrict__ partials, int n_heads, int n_kv, int hd, int page_size,
+    int window, float scale, int gh, int head_chunks) {
+    extern __shared__ float lds[];
+    float* qs = lds;                          // [kRows][hd]
+    float* kv = qs + kRows * hd;              // [kKeys][hd + 1]
+    float* ps = kv + kKeys * (hd + 1);        // [kRows][kKeys]
+    const int kv_stride = hd + 1;
+
+    const int32_t* item = items + static_cast<int64_t>(blockIdx.x) * FSIE_ATTN_ITEM_INTS;
+    const int seq = item[FSIE_ATTN_ITEM_SEQ];
+    const int q_row0 = item[FSIE_ATTN_ITEM_QROW];
+    const int n_q = item[FSIE_ATTN_ITEM_NQ];
+    const int pos0 = item[FSIE_ATTN_ITEM_POS];
+    const int key_begin = item[FSIE_ATTN_ITEM_KBEGIN];
+    const int key_end = item[FSIE_ATTN_ITEM_KEND];
+    const int partial_base = item[FSIE_ATTN_ITEM_PARTIAL];
+    if (n_q <= 0) return;  // padding item
+
+    const int group = n_heads / n_kv;
+    const int kvh = blockIdx.y / head_chunks;
+    const int chunk = blockIdx.y - kvh * head_chunks;
+    const int gh_here = min(gh, group - chunk * gh);
+    const int h_base = kvh * group + chunk * gh;
+    const int n_rows = n_q * gh;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (FSIE_WAVE - 1);
+    const int wave = tid / FSIE_WAVE;
+    const int sub = lane >> 5;    // which of the two rows of a pass
+    const int lane32 = lane & 31;
+
+    // queries of this block's rows
+    for (int e = tid; e < kRows * hd; e += blockDim.x) {
+        const int r = e / hd, d = e - r * hd;
+        float v = 0.f;
+        if (r < n_rows && (r % gh) < gh_here) {
+            const int tq = r / gh, hq = h_base + (r % gh);
+            v = to_float(q[static_cast<int64_t>(q_row0 + tq) * q_stride + static_cast<int64_t>(hq) * hd + d]);
+        }
+        qs[e] = v;
+    }
+
+    float m_run[2], l_run[2], acc[2][kMaxChunks];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        m_run[p] = -INFINITY;
+        l_run[p] = 0.f;
+#pragma unroll
+        for (int i = 0; i < kMaxChunks; ++i) acc[p][i] = 0.f;
+    }
+    const int n_chunks = (hd + 31) / 32;
+    const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
+
+    for (int kt = key_begin; kt < key_end; kt += kKeys) {
+        __syncthreads();  // previous tile's values are no longer read (first pass: qs is written)
+        for (int e = tid; e < kKeys * hd; e += blockDim.x) {
+            const int j = e / hd, d = e - j * hd;
+            const int kj = kt + j;
+            float v = 0.f;
+            if (kj < key_end) {
+                const int page = table[kj / page_size];
+                if (page >= 0) {
+                    v = to_float(k_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + kj % page_size) * hd + d]);
+                }
+            }
+            kv[j * kv_stride + d] = v;
+        }
+        __syncthreads();
+        float corr[2];
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int r = wave * 4 + p * 2 + sub;
+            const bool row_ok = r < n_rows && (r % gh) < gh_here;
+            const int pos = pos0 + r / gh;
+            const int kj = kt + lane32;
+            bool visible = row_ok && kj < key_end && kj <= pos && (window <= 0 || kj > pos - window);
+            if (visible) visible = table[kj / page_size] >= 0;
+            float s = -INFINITY;
+            if (visible) {
+                const float* qr = qs + r * hd;
+                const float* kr = kv + lane32 * kv_stride;
+                float dot = 0.f;
+                for (int d = 0; d < hd; ++d) dot = fmaf(qr[d], kr[d], dot);
+                s = dot * scale;
+            }
+            const float m_new = fmaxf(m_run[p], half_wave_max(s));
+            const float pe = (s == -INFINITY) ? 0.f : expf(s - m_new);
+            corr[p] = (m_run[p] == -INFINITY) ? 1.f : expf(m_run[p] - m_new);
+            l_run[p] = l_run[p] * corr[p] + half_wave_sum(pe);
+            m_run[p] = m_new;
+            ps[r * kKeys + lane32] = pe;
+        }
+        __syncthreads();  // scores done: the tile buffer can take the values
+        for (int e = tid; e < kKeys * hd; e += blockDim.x) {
+            const int j = e / hd, d = e - j * hd;
+            const int kj = kt + j;
+            float v = 0.f;
+            if (kj < key_end) {
+                const int page = table[kj / page_size];
+                if (page >= 0) {
+                    v = to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + kj % page_size) * hd + d]);
+                }
+            }
+            kv[j * kv_stride + d] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int r = wave * 4 + p * 2 + sub;
+            const float* pr = ps + r * kKeys;
+#pragma unroll
+            for (int i = 0; i < kMaxChunks; ++i) {
+                if (i < n_chunks) {
+                    const int d = lane32 + 32 * i;
+                    float a = acc[p][i] * corr[p];
+                    if (d < hd) {
+                        for (int j = 0; j < kKeys; ++j) a = fmaf(pr[j], kv[j * kv_stride + d], a);
+                    }
+                    acc[p][i] = a;
+                }
+            }
+        }
+    }
+
+    // results
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int r = wave * 4 + p * 2 + sub;
+        if (!(r < n_rows && (r % gh) < gh_here)) continue;
+        const int tq = r / gh, hq = h_base + (r % gh);
+        if (partial_base < 0) {
+            const float inv = l_run[p] > 0.f ? 1.0f / l_run[p] : 0.f;
+            T* o = out + (static_cast<int64_t>(q_row0 + tq) * n_heads + hq) * hd;
+#pragma unroll
+            for (int i = 0; i < kMaxChunks; ++i) {
+                const int d = lane32 + 32 * i;
+                if (i < n_chunks && d < hd) o[d] = from_float<T>(acc[p][i] * inv);
+            }
+        } else {
+            float* rec = partials + (static_cast<int64_t>(partial_base + tq) * n_heads + hq) * (hd + 2);
+#pragma unroll
+            for (int i = 0; i < kMaxChunks; ++i) {
+                const int d = lane32 + 32 * i;
+                if (i < n_chunks && d < hd) rec[d] = acc[p][i];
+            }
+            if (lane32 == 0) {
+                rec[hd] = m_run[p];
+                rec[hd + 1] = l_run[p];
+            }
+        }
+    }
+}
+
+// Combine the partial records of one query token in the fixed order of its splits.
+// merge item: {out_row, first_slot, n_splits, slot_stride}
+template <typename T>
+__global__ void attention_merge_kernel(const float* __restrict__ partials, const int32_t* __restrict__ merges,
+                                       T* __restrict__ out, int n_heads, int hd) {
+    const int32_t* mi = merges + static_cast<int64_t>(blockIdx.x) * FSIE_ATTN_MERGE_INTS;
+    const int out_row = mi[0], first = mi[1], n_splits = mi[2], stride = mi[3];
+    if (n_splits <= 0) return;
+    const int hq = blockIdx.y;
+    const int64_t rec_size = hd + 2;
+    float m = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) {
+        const float* rec = partials + (static_cast<int64_t>(first + s * stride) * n_heads + hq) * rec_size;
+        m = fmaxf(m, rec[hd]);
+    }
+    float denom = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float* rec = partials + (static_cast<int64_t>(first + s * stride) * n_heads + hq) * rec_size;
+        if (rec[hd] != -INFINITY) denom += rec[hd + 1] * expf(rec[hd] - m);
+    }
+    const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float a = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float* rec = partials + (static_cast<int64_t>(first + s * stride) * n_heads + hq) * rec_size;
+            if (rec[hd] != -INFINITY) a += rec[d] * expf(rec[hd] - m);
+        }
+        out[(static_cast<int64_t>(out_row) * n_heads + hq) * hd + d] = from_float<T>(a * inv);
+    }
+}
+
+}  // namespace
+
+extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                                     const int32_t* block_tables, int max_pages, const int32_t* items,
+                                     int n_items, void* out, float* partials, int n_heads, int n_kv,
+                                     int head_dim, int page_size, int window, float scale, int dtype,
+                                     hipStream_t stream) {
+    FSIE_REQUIRE(n_items >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
+                 "attention: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
+    FSIE_REQUIRE(head_dim > 0 && head_dim <= 32 * kMaxChunks, "attention: head_dim %d must be in 1..%d",
+                 head_dim, 32 * kMaxChunks);
+    FSIE_REQUIRE(page_size > 0 && max_pages > 0, "attention: bad page geometry");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "attention: unknown dtype %d", dtype);
+    if (n_items == 0) return 0;
+    const int group = n_heads / n_kv;
+    const int gh = group < kRows ? group : kRows;
+    const int head_chunks = (group + gh - 1) / gh;
+    const dim3 grid(n_items, n_kv * head_chunks);
+    const size_t lds = sizeof(float) * (static_cast<size_t>(kRows) * head_dim + kKeys * (head_dim + 1) + kRows * kKeys);
+    if (dtype == FSIE_F32) {
+        attention_scalar_kernel<float><<<grid, 256, lds, stream>>>(
+            static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pool), static_cast<const float*>(v_pool),
+            block_tables, max_pages, items, static_cast<float*>(out), partials, n_heads, n_kv, head_dim, page_size,
+            window, scale, gh, head_chunks);
+    } else {
+        attention_scalar_kernel<bf16_t><<<grid, 256, lds, stream>>>(
+            static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool),
+            static_cast<const bf16_t*>(v_pool), block_tables, max_pages, items, static_cast<bf16_t*>(out), partials,
+            n_heads, n_kv, head_dim, page_size, window, scale, gh, head_chunks);
+    }
+    FSIE_CHECK_LAUNCH("attention_scalar");
+    return 0;
+}
+
+extern "C" int fsie_attention_merge(const float* partials, const int32_t* merges, int n_merges, void* out,
+                                    int n_heads, int head_dim, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(n_merges >= 0 && n_heads > 0 && head_dim > 0, "attention_merge: bad sizes");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "attention_merge: unknown dtype %d", dtype);
+    if (n_merges == 0) return 0;
+    const dim3 grid(n_merges, n_heads);
+    if (dtype == FSIE_F32) {
+        attention_merge_kernel<float><<<grid, 64, 0, stream>>>(partials, merges, static_cast<float*>(out), n_heads, head_dim);
+    } else {
+        attention_merge_kernel<bf16_t><<<grid, 64, 0, stream>>>(partials, merges, static_cast<bf16_t*>(out), n_heads, head_dim);
+    }
+    FSIE_CHECK_LAUNCH("attention_merge");
+    return 0;
+}
+
+// Query tokens per work item for a model with `n_heads` and `n_kv` heads, so that the host cuts
+// tiles the way the kernel expects.
+extern "C" int fsie_attention_scalar_tile_tokens(int n_heads, int n_kv) {
+    if (n_kv <= 0 || n_heads <= 0 || n_heads % n_kv) return 0;
+    const int group = n_heads / n_kv;
+    const int gh = group < kRows ? group : kRows;
+    return kRows / gh;
+}

@@ -1,0 +1,160 @@
+// Embedding gather, RMSNorm (alone, fused with the residual sum, or over chosen rows), SiLU*up
+// and the plain residual sum.  The residual stream is float32 in both precisions; T is the
+// type of activations and matrices (float or bfloat16).
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// out[t, :] = table[ids[t], :] as float32.  An id outside the table gives a row of zeros; the
+// host refuses such ids before the launch.
+template <typename T>
+__global__ void embedding_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
+                                 float* __restrict__ out, int hidden, int vocab) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* dst = out + static_cast<int64_t>(t) * hidden;
+    if (id < 0 || id >= vocab) {
+        for (int j = threadIdx.x; j < hidden; j += blockDim.x) dst[j] = 0.f;
+        return;
+    }
+    const T* src = table + static_cast<int64_t>(id) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) dst[j] = to_float(src[j]);
+}
+
+// One block per output row r; source row = rows ? rows[r] : r.
+//   v = residual[row] (+ delta[row]);  if write_back: residual[row] = v
+//   out[r] = (v * rsqrt(mean(v^2) + eps)) * weight
+// Sum of squares, scale and the residual sum are float32.
+template <typename T>
+__global__ void rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                               const float* __restrict__ weight, T* __restrict__ out,
+                               const int32_t* __restrict__ rows, int hidden, float eps,
+                               int write_back) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int64_t row = rows ? rows[r] : r;
+    float* res = residual + row * hidden;
+    const T* del = delta ? delta + row * hidden : nullptr;
+    float sum_sq = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        float v = res[j];
+        if (del) v += to_float(del[j]);
+        if (write_back) res[j] = v;
+        sum_sq += v * v;
+    }
+    const float total = block_sum(sum_sq, scratch);
+    const float scale = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    T* dst = out + static_cast<int64_t>(r) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        float v = res[j];
+        if (del && !write_back) v += to_float(del[j]);
+        dst[j] = from_float<T>((v * scale) * weight[j]);
+    }
+}
+
+// out[t, j] = silu(x[t, j]) * x[t, inter + j]; x is [T, 2*inter] (gate columns, then up).
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t total, int inter) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int64_t t = i / inter;
+    const int j = static_cast<int>(i - t * inter);
+    const float g = to_float(x[t * 2 * inter + j]);
+    const float u = to_float(x[t * 2 * inter + inter + j]);
+    out[i] = from_float<T>((g / (1.0f + expf(-g))) * u);
+}
+
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ residual, const T* __restrict__ delta, int64_t total) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < total) residual[i] += to_float(delta[i]);
+}
+
+template <typename T>
+__global__ void bias_add_kernel(T* __restrict__ y, const float* __restrict__ bias, int64_t total, int cols) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < total) y[i] = from_float<T>(to_float(y[i]) + bias[i % cols]);
+}
+
+}  // namespace
+
+extern "C" int fsie_embedding(const void* table, int dtype, const int32_t* ids, float* out,
+                              int n_tokens, int hidden, int vocab, hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes T=%d H=%d V=%d",
+                 n_tokens, hidden, vocab);
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "embedding: unknown dtype %d", dtype);
+    if (n_tokens == 0) return 0;
+    if (dtype == FSIE_F32) {
+        embedding_kernel<float><<<n_tokens, kThreads, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab);
+    } else {
+        embedding_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, hidden, vocab);
+    }
+    FSIE_CHECK_LAUNCH("embedding");
+    return 0;
+}
+
+extern "C" int fsie_rmsnorm(float* residual, const void* delta, const float* weight, void* out,
+                            const int32_t* rows, int n_rows, int hidden, float eps, int dtype,
+                            int write_back, hipStream_t stream) {
+    FSIE_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, hidden);
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "rmsnorm: unknown dtype %d", dtype);
+    FSIE_REQUIRE(!(write_back && rows), "rmsnorm: write_back cannot be combined with a row list");
+    FSIE_REQUIRE(!(write_back && !delta), "rmsnorm: write_back without a delta");
+    if (n_rows == 0) return 0;
+    if (dtype == FSIE_F32) {
+        rmsnorm_kernel<float><<<n_rows, kThreads, 0, stream>>>(residual, static_cast<const float*>(delta), weight,
+                                                               static_cast<float*>(out), rows, hidden, eps, write_back);
+    } else {
+        rmsnorm_kernel<bf16_t><<<n_rows, kThreads, 0, stream>>>(residual, static_cast<const bf16_t*>(delta), weight,
+                                                                static_cast<bf16_t*>(out), rows, hidden, eps, write_back);
+    }
+    FSIE_CHECK_LAUNCH("rmsnorm");
+    return 0;
+}
+
+extern "C" int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "swiglu: unknown dtype %d", dtype);
+    const int64_t total = static_cast<int64_t>(n_tokens) * inter;
+    if (total == 0) return 0;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(total, kThreads));
+    if (dtype == FSIE_F32) {
+        swiglu_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(out), total, inter);
+    } else {
+        swiglu_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(out), total, inter);
+    }
+    FSIE_CHECK_LAUNCH("swiglu");
+    return 0;
+}
+
+extern "C" int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(total >= 0, "residual_add: negative size");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "residual_add: unknown dtype %d", dtype);
+    if (total == 0) return 0;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(total, kThreads));
+    if (dtype == FSIE_F32) {
+        residual_add_kernel<float><<<grid, kThreads, 0, stream>>>(residual, static_cast<const float*>(delta), total);
+    } else {
+        residual_add_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(residual, static_cast<const bf16_t*>(delta), total);
+    }
+    FSIE_CHECK_LAUNCH("residual_add");
+    return 0;
+}
+
+extern "C" int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(rows >= 0 && cols > 0, "bias_add: bad sizes %d x %d", rows, cols);
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "bias_add: unknown dtype %d", dtype);
+    const int64_t total = static_cast<int64_t>(rows) * cols;
+    if (total == 0) return 0;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(total, kThreads));
+    if (dtype == FSIE_F32) {
+        bias_add_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<float*>(y), bias, total, cols);
+    } else {
+        bias_add_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<bf16_t*>(y), bias, total, cols);
+    }
+    FSIE_CHECK_LAUNCH("bias_add");
+    return 0;
+}

@@ -1,0 +1,110 @@
+// Rotary position encoding on q and k, fused with the q/k/v bias and with the write of k (rotated)
+// and v into the pages of the cache.  One block per token.  The v columns of the row itself are
+// left without the bias: only the cache is read afterwards.
+//
+// Page layout (keys and values alike): [page][kv_head][slot in page][head_dim].
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxHalf = 256;  // head_dim <= 512
+
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                     const int32_t* __restrict__ slots, const double* __restrict__ inv_freq,
+                                     const float* __restrict__ bias, T* __restrict__ k_pool, T* __restrict__ v_pool, int n_heads, int n_kv,
+                                     int head_dim, int rotary_half, int page_size, int write_kv,
+                                     int64_t pool_slots) {
+    __shared__ float cs[kMaxHalf];
+    __shared__ float sn[kMaxHalf];
+    const int t = blockIdx.x;
+    const int q_dim = n_heads * head_dim;
+    const int kv_dim = n_kv * head_dim;
+    T* row = qkv + static_cast<int64_t>(t) * (q_dim + 2 * kv_dim);
+
+    // angle = position * inv_freq in float64, as the plain formula has it; cos and sin are
+    // rounded to float32 once.
+    const double pos = static_cast<double>(positions[t]);
+    for (int i = threadIdx.x; i < rotary_half; i += blockDim.x) {
+        double s, c;
+        sincos(pos * inv_freq[i], &s, &c);
+        cs[i] = static_cast<float>(c);
+        sn[i] = static_cast<float>(s);
+    }
+    __syncthreads();
+
+    const int slot = (write_kv && slots) ? slots[t] : -1;
+    const int64_t page = slot >= 0 ? slot / page_size : 0;
+    const int off = slot >= 0 ? slot % page_size : 0;
+
+    // q and k heads: add the bias, then rotate the pairs (i, i + rotary_half) of the first
+    // 2*rotary_half dimensions in place; the remaining dimensions only take the bias.
+    const int n_rot_heads = n_heads + n_kv;  // k heads follow the q heads directly in a row
+    for (int idx = threadIdx.x; idx < n_rot_heads * rotary_half; idx += blockDim.x) {
+        const int h = idx / rotary_half;
+        const int i = idx - h * rotary_half;
+        T* head = row + h * head_dim;
+        float x1 = to_float(head[i]);
+        float x2 = to_float(head[i + rotary_half]);
+        if (bias) {
+            x1 += bias[h * head_dim + i];
+            x2 += bias[h * head_dim + i + rotary_half];
+        }
+        const float c = cs[i], s = sn[i];
+        head[i] = from_float<T>(x1 * c - x2 * s);
+        head[i + rotary_half] = from_float<T>(x2 * c + x1 * s);
+    }
+    const int rest = head_dim - 2 * rotary_half;
+    if (bias && rest > 0) {
+        for (int idx = threadIdx.x; idx < n_rot_heads * rest; idx += blockDim.x) {
+            const int h = idx / rest;
+            const int d = 2 * rotary_half + (idx - h * rest);
+            T* head = row + h * head_dim;
+            head[d] = from_float<T>(to_float(head[d]) + bias[h * head_dim + d]);
+        }
+    }
+    if (slot < 0 || slot >= pool_slots) return;  // uniform over the block
+    __syncthreads();  // the k written above is read back below by other threads
+    const T* k = row + q_dim;
+    const T* v = row + q_dim + kv_dim;
+    for (int idx = threadIdx.x; idx < kv_dim; idx += blockDim.x) {
+        const int kvh = idx / head_dim;
+        const int d = idx - kvh * head_dim;
+        const int64_t dst = ((page * n_kv + kvh) * page_size + off) * head_dim + d;
+        k_pool[dst] = k[idx];
+        v_pool[dst] = bias ? from_float<T>(to_float(v[idx]) + bias[q_dim + kv_dim + idx]) : v[idx];
+    }
+}
+
+}  // namespace
+
+extern "C" int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int32_t* slots,
+                                  const double* inv_freq, const float* bias, void* k_pool, void* v_pool, int n_tokens,
+                                  int n_heads, int n_kv, int head_dim, int rotary_dim, int page_size,
+                                  int64_t pool_slots, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv > 0, "rope_kv_write: bad sizes");
+    FSIE_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim / 2 <= kMaxHalf,
+                 "rope_kv_write: head_dim %d must be even and <= %d", head_dim, 2 * kMaxHalf);
+    FSIE_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
+                 "rope_kv_write: rotary_dim %d must be even and within head_dim %d", rotary_dim, head_dim);
+    FSIE_REQUIRE(rotary_dim == 0 || inv_freq, "rope_kv_write: no frequency table");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "rope_kv_write: unknown dtype %d", dtype);
+    const int write_kv = (k_pool && v_pool && slots) ? 1 : 0;
+    FSIE_REQUIRE(!write_kv || (page_size > 0 && pool_slots > 0), "rope_kv_write: bad page geometry");
+    if (n_tokens == 0) return 0;
+    if (dtype == FSIE_F32) {
+        rope_kv_write_kernel<float><<<n_tokens, kThreads, 0, stream>>>(
+            static_cast<float*>(qkv), positions, slots, inv_freq, bias, static_cast<float*>(k_pool),
+            static_cast<float*>(v_pool), n_heads, n_kv, head_dim, rotary_dim / 2, page_size, write_kv,
+            pool_slots);
+    } else {
+        rope_kv_write_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(
+            static_cast<bf16_t*>(qkv), positions, slots, inv_freq, bias, static_cast<bf16_t*>(k_pool),
+            static_cast<bf16_t*>(v_pool), n_heads, n_kv, head_dim, rotary_dim / 2, page_size, write_kv,
+            pool_slots);
+    }
+    FSIE_CHECK_LAUNCH("rope_kv_write");
+    return 0;
+}

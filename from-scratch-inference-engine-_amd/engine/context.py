@@ -1,0 +1,166 @@
+"""What one step looks like to the parts: the tokens of the batch and their index tables.
+
+The host collects every int32 table of the step (token ids, positions, block tables, cache slots,
+attention work items, ...) into one pinned buffer and sends it with one copy; the parts see
+device views of it."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from types import SimpleNamespace
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, RequestCache
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens and the places among them whose logits
+    are wanted."""
+
+    cache: RequestCache
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class HostBatch:
+    """Host view of the step, in the order of the entries."""
+
+    def __init__(self, entries: Sequence[StepEntry]):
+        self.n_seqs = len(entries)
+        self.q_lens = [len(e.tokens) for e in entries]
+        self.past_lens = [e.cache.length for e in entries]
+        self.q_starts = [0]
+        for n in self.q_lens:
+            self.q_starts.append(self.q_starts[-1] + n)
+        self.n_tokens = self.q_starts[-1]
+        self.seq_slots = [e.cache.slot for e in entries]
+        self.token_ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64,
+                                     count=self.n_tokens)
+        self.positions = np.concatenate(
+            [np.arange(p, p + n, dtype=np.int32) for p, n in zip(self.past_lens, self.q_lens)]
+        ) if entries else np.zeros(0, np.int32)
+        self.want_rows = np.asarray([self.q_starts[i] + w for i, e in enumerate(entries) for w in e.want],
+                                    dtype=np.int32)
+
+
+class _Packer:
+    """Collects int32 arrays; one pinned buffer, one copy."""
+
+    ALIGN = 4  # ints: every table starts on 16 bytes
+
+    def __init__(self):
+        self._arrays: List[np.ndarray] = []
+        self._offsets: List[int] = []
+        self._total = 0
+
+    def add(self, array: np.ndarray) -> int:
+        array = np.ascontiguousarray(array, dtype=np.int32)
+        self._arrays.append(array)
+        self._offsets.append(self._total)
+        self._total += -(-max(array.size, 1) // self.ALIGN) * self.ALIGN
+        return len(self._arrays) - 1
+
+    def upload(self, staging: "PinnedStaging", device) -> List[torch.Tensor]:
+        host = staging.acquire(self._total)
+        flat = host.numpy()
+        for a, off in zip(self._arrays, self._offsets):
+            flat[off:off + a.size] = a.reshape(-1)
+        dev = torch.empty((self._total,), dtype=torch.int32, device=device)
+        dev.copy_(host[:self._total], non_blocking=True)
+        staging.release()
+        return [dev[off:off + a.size].view(a.shape) for a, off in zip(self._arrays, self._offsets)]
+
+
+class PinnedStaging:
+    """A pinned host buffer reused from step to step; an event guards it until the copy that
+    read it has run."""
+
+    def __init__(self):
+        self._buf: Optional[torch.Tensor] = None
+        self._event: Optional[torch.cuda.Event] = None
+
+    def acquire(self, n_ints: int) -> torch.Tensor:
+        if self._event is not None:
+            self._event.synchronize()
+        if self._buf is None or self._buf.numel() < n_ints:
+            self._buf = torch.empty((max(n_ints, 1 << 14),), dtype=torch.int32, pin_memory=True)
+        return self._buf
+
+    def release(self) -> None:
+        if self._event is None:
+            self._event = torch.cuda.Event()
+        self._event.record()
+
+
+class StepContext:
+    """Passed to every part.  Device tensors are int32.
+
+    ``token_ids`` [T], ``positions`` [T], ``want_rows`` [wanted], ``seq_slots`` [n] (state slot of
+    each request), ``q_starts`` [n+1], ``past_lens`` [n]; per paged group ``block_tables[g]``
+    [n, pages] and ``slots[g]`` [T]; ``host`` holds the same as Python lists/arrays.
+    ``plan(planner)`` gives the tables a part asked for through its ``planner()``."""
+
+    def __init__(self, host: HostBatch, compute_dtype: torch.dtype, device):
+        self.host = host
+        self.compute_dtype = compute_dtype
+        self.device = device
+        self.n_tokens = host.n_tokens
+        self.n_seqs = host.n_seqs
+        self.token_ids = self.positions = self.want_rows = None
+        self.seq_slots = self.q_starts = self.past_lens = None
+        self.block_tables: List[torch.Tensor] = []
+        self.slots: List[torch.Tensor] = []
+        self._plans: Dict[Hashable, SimpleNamespace] = {}
+
+    def plan(self, planner) -> SimpleNamespace:
+        try:
+            return self._plans[planner.key]
+        except KeyError:
+            raise KeyError(f"no plan for {planner.key!r}: the part's planner() was not collected "
+                           f"when the model was built") from None
+
+
+def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners: Sequence, staging: PinnedStaging,
+                  compute_dtype: torch.dtype, device) -> StepContext:
+    """Tables of one step.  The entries' pages must have been reserved already."""
+    host = HostBatch(entries)
+    ctx = StepContext(host, compute_dtype, device)
+    pk = _Packer()
+    i_ids = pk.add(host.token_ids.astype(np.int32))
+    i_pos = pk.add(host.positions)
+    i_want = pk.add(host.want_rows)
+    i_slots = pk.add(np.asarray(host.seq_slots, dtype=np.int32))
+    i_qs = pk.add(np.asarray(host.q_starts, dtype=np.int32))
+    i_past = pk.add(np.asarray(host.past_lens, dtype=np.int32))
+    ps = manager.page_size
+    group_idx = []
+    for g in range(len(manager.groups)):
+        max_pages = max([len(e.cache.tables[g]) for e in entries] + [1])
+        table = np.full((len(entries), max_pages), -1, dtype=np.int32)
+        slot_map = np.full((host.n_tokens,), -1, dtype=np.int32)
+        for s, e in enumerate(entries):
+            pages = np.asarray(e.cache.tables[g], dtype=np.int32)
+            table[s, :pages.size] = pages
+            pos = host.positions[host.q_starts[s]:host.q_starts[s + 1]]
+            page_of = pages[pos // ps]
+            slot_map[host.q_starts[s]:host.q_starts[s + 1]] = np.where(page_of >= 0, page_of * ps + pos % ps, -1)
+        group_idx.append((pk.add(table), pk.add(slot_map)))
+    plan_idx = []
+    for planner in planners:
+        made = planner.plan(host)
+        arrays = {k: pk.add(v) for k, v in made.items() if isinstance(v, np.ndarray)}
+        scalars = {k: v for k, v in made.items() if not isinstance(v, np.ndarray)}
+        plan_idx.append((planner.key, arrays, scalars))
+    dev = pk.upload(staging, device)
+    ctx.token_ids, ctx.positions, ctx.want_rows = dev[i_ids], dev[i_pos], dev[i_want]
+    ctx.seq_slots, ctx.q_starts, ctx.past_lens = dev[i_slots], dev[i_qs], dev[i_past]
+    for it, isl in group_idx:
+        ctx.block_tables.append(dev[it])
+        ctx.slots.append(dev[isl])
+    for key, arrays, scalars in plan_idx:
+        ctx._plans[key] = SimpleNamespace(**{k: dev[i] for k, i in arrays.items()}, **scalars)
+    return ctx

@@ -1,0 +1,203 @@
+"""The model on the device and the step function.
+
+``Model`` owns the parts with their weights.  ``Runner`` joins a model with a cache (manager +
+storage) and offers ``step``: run the given tokens of the given requests as one batch, from the
+cache that earlier steps left, and return the logits at the wanted places.
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..cache.allocator import OutOfPages
+from ..cache.manager import CacheManager, PagedNeed, StateNeed
+from ..cache.storage import CacheLayout, CacheStorage
+from ..config.base import ModelConfig, read_config_json
+from ..models.registry import build_model_spec, parse_config
+from ..models.spec import ModelSpec
+from ..parts.base import HiddenState
+from ..weights.loader import fill_parts, load_weights
+from ..weights.random_init import random_tensor, expected_tensors
+from .context import PinnedStaging, StepContext, StepEntry, build_context
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
+
+
+def resolve_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"the engine runs in bfloat16 or float32, not {dtype}")
+        return dtype
+    try:
+        return _DTYPES[str(dtype)]
+    except KeyError:
+        raise ValueError(f"unknown dtype '{dtype}' (bfloat16 or float32)") from None
+
+
+def _require_gpu(device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError("the engine needs a GPU: there is no CPU path")
+    ops.load()  # fails loudly when the kernel library is missing
+    return device
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, dtype, device):
+        self.spec = spec
+        self.config = spec.config
+        self.dtype = resolve_dtype(dtype)
+        self.device = torch.device(device)
+        self.weight_bytes = 0
+        # caches: one per call of the schedule that keeps one
+        self.call_cache: List[int] = []
+        needs: Dict[int, object] = {}
+        for i, call in enumerate(spec.schedule):
+            if not 0 <= call.layer < len(spec.layers):
+                raise ValueError(f"schedule entry {i} names layer {call.layer}, which does not exist")
+            if call.cache_of is None:
+                self.call_cache.append(i)
+                need = spec.layers[call.layer].mixer.cache_need()
+                if need is not None:
+                    needs[i] = need
+            else:
+                if not 0 <= call.cache_of < i or spec.schedule[call.cache_of].cache_of is not None:
+                    raise ValueError(f"schedule entry {i}: cache_of must name an earlier call that keeps a cache")
+                self.call_cache.append(call.cache_of)
+        groups: List[PagedNeed] = []
+        group_caches: List[List[int]] = []
+        states: Dict[int, StateNeed] = {}
+        for cid, need in needs.items():
+            if isinstance(need, PagedNeed):
+                if need not in groups:
+                    groups.append(need)
+                    group_caches.append([])
+                group_caches[groups.index(need)].append(cid)
+            elif isinstance(need, StateNeed):
+                states[cid] = need
+            else:
+                raise TypeError(f"cache_need() of call {cid} returned {type(need).__name__}")
+        self.cache_layout = CacheLayout(groups, group_caches, states)
+        self.cached_calls = set(needs)
+        # planners of all mixers, one per distinct key
+        self.planners = []
+        seen = set()
+        for block in spec.layers:
+            planner = block.mixer.planner()
+            if planner is not None and planner.key not in seen:
+                seen.add(planner.key)
+                self.planners.append(planner)
+
+    # ---------------------------------------------------------------- construction
+    @classmethod
+    def from_pretrained(cls, model_dir, dtype="bfloat16", device="cuda:0") -> "Model":
+        device = _require_gpu(device)
+        config = parse_config(read_config_json(model_dir))
+        model = cls(build_model_spec(config), dtype, device)
+        path = Path(model_dir) / "model.safetensors"
+        model.weight_bytes = load_weights(path, model.spec.bindings, model.dtype, device,
+                                          model.spec.ignore_unexpected)
+        model._prepare()
+        return model
+
+    @classmethod
+    def from_random(cls, config: ModelConfig, seed: int = 0, dtype="bfloat16", device="cuda:0") -> "Model":
+        """Random weights generated on the device (nothing is written; ``write_random_model``
+        makes a folder instead)."""
+        device = _require_gpu(device)
+        model = cls(build_model_spec(config), dtype, device)
+        specs = expected_tensors(model.spec.bindings)
+        model.weight_bytes = fill_parts(
+            model.spec.bindings, lambda name: random_tensor(specs[name], seed, torch.float32, device=device),
+            model.dtype, device)
+        model._prepare()
+        return model
+
+    def _prepare(self) -> None:
+        for part in self.spec.all_parts():
+            part.prepare(self.device, self.dtype)
+
+    # ---------------------------------------------------------------- cache
+    def make_cache(self, page_size: int, num_pages: int, max_requests: int):
+        manager = CacheManager(self.cache_layout.paged_groups, page_size, num_pages, max_requests)
+        storage = CacheStorage(self.cache_layout, manager, self.device, self.dtype)
+        return manager, storage
+
+    def cache_bytes_per_token(self) -> int:
+        item = torch.empty((), dtype=self.dtype).element_size()
+        return sum(2 * need.n_kv_heads * need.head_dim * item * len(ids)
+                   for need, ids in zip(self.cache_layout.paged_groups, self.cache_layout.group_caches))
+
+    # ---------------------------------------------------------------- compute
+    def forward(self, ctx: StepContext, storage: CacheStorage) -> torch.Tensor:
+        """float32 logits [wanted, vocab] for the step described by ``ctx``."""
+        spec = self.spec
+        hidden = HiddenState(spec.embedding.forward(ctx.token_ids))
+        for i, call in enumerate(spec.schedule):
+            cid = self.call_cache[i]
+            cache = storage.view(cid, ctx, writes=call.cache_of is None) if cid in self.cached_calls else None
+            spec.layers[call.layer].forward(hidden, ctx, cache)
+        if ctx.want_rows.shape[0] == 0:
+            return torch.empty((0, spec.lm_head.vocab_size), dtype=torch.float32, device=self.device)
+        normed = spec.final_norm.rows(hidden, ctx.want_rows, self.dtype)
+        return spec.lm_head.forward(normed)
+
+
+class Runner:
+    """The step function over one model and one cache."""
+
+    def __init__(self, model: Model, page_size: int = 16, num_pages: int = 2048, max_requests: int = 256):
+        self.model = model
+        self.manager, self.storage = model.make_cache(page_size, num_pages, max_requests)
+        self._staging = PinnedStaging()
+        self.vocab_size = model.spec.embedding.vocab_size
+        self.max_position = int(getattr(model.config, "max_position_embeddings", 0) or 0)
+        self.steps = 0
+        self.tokens = 0
+
+    def check(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise ValueError("step: empty batch")
+        seen = set()
+        for e in entries:
+            n = len(e.tokens)
+            if n == 0:
+                raise ValueError(f"step: request {e.cache.request_id!r} brings no tokens")
+            if e.cache.closed:
+                raise ValueError(f"step: request {e.cache.request_id!r} is closed")
+            if id(e.cache) in seen:
+                raise ValueError(f"step: request {e.cache.request_id!r} appears twice in one step")
+            seen.add(id(e.cache))
+            lo, hi = min(e.tokens), max(e.tokens)
+            if lo < 0 or hi >= self.vocab_size:
+                raise IndexError(f"step: token id {lo if lo < 0 else hi} of request {e.cache.request_id!r} "
+                                 f"is outside the vocabulary [0, {self.vocab_size})")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise IndexError(f"step: wanted place {w} is outside the {n} tokens of request "
+                                     f"{e.cache.request_id!r}")
+            if self.max_position and e.cache.length + n > self.max_position:
+                raise ValueError(f"step: request {e.cache.request_id!r} would reach {e.cache.length + n} "
+                                 f"positions, more than max_position_embeddings {self.max_position}")
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run one batch.  Nothing is changed when the batch is refused (bad ids, no pages)."""
+        self.check(entries)
+        if not self.manager.can_reserve((e.cache, len(e.tokens)) for e in entries):
+            raise OutOfPages("step: the batch needs more pages than the pool has free")
+        for e in entries:
+            self.manager.reserve(e.cache, len(e.tokens))
+        self.storage.reset_states([e.cache.slot for e in entries if e.cache.length == 0])
+        ctx = build_context(entries, self.manager, self.model.planners, self._staging, self.model.dtype,
+                            self.model.device)
+        logits = self.model.forward(ctx, self.storage)
+        for e in entries:
+            self.manager.commit(e.cache, len(e.tokens))
+        self.steps += 1
+        self.tokens += ctx.n_tokens
+        return logits

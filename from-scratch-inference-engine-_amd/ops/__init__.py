@@ -1,0 +1,14 @@
+"""The hand-written kernels as functions over torch tensors.
+
+Each function checks on the host that the operands have the shapes, types and contiguity that the
+kernel and its grid assume, then queues the kernel on torch's current stream.  Nothing here
+computes with torch; a missing kernel library is an error, not a reason to fall back.
+"""
+
+from .functions import (bias_add, attention_merge, attention_scalar, attention_tile_tokens, dtype_code,
+                        embedding, gemm, residual_add, rmsnorm, rope_kv_write, sample, swiglu)
+from .library import KernelError, KernelLibraryMissing, load
+
+__all__ = ["KernelError", "KernelLibraryMissing", "attention_merge", "attention_scalar", "bias_add",
+           "attention_tile_tokens", "dtype_code", "embedding", "gemm", "load", "residual_add",
+           "rmsnorm", "rope_kv_write", "sample", "swiglu"]

@@ -1,0 +1,242 @@
+"""Host-side checks and launches of the kernels."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .library import KernelError, check, load
+
+F32, BF16 = 0, 1
+ATTN_ITEM_INTS = 8
+ATTN_MERGE_INTS = 4
+GEMM_SKINNY_MAX_M = 8
+GEMM_AUTO, GEMM_TILED, GEMM_SKINNY = 0, 1, 2
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16, not {dtype}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape=None, ndim=None) -> None:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name}: must be a tensor on the GPU")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, found {t.dtype}")
+    if ndim is not None and t.dim() != ndim:
+        raise KernelError(f"{name}: expected {ndim} dimensions, found shape {tuple(t.shape)}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name}: expected shape {tuple(shape)}, found {tuple(t.shape)}")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 rows of ``table`` [V, H] at ``ids`` (int32 [T]).  The caller has checked the ids."""
+    _need(table, "embedding table", ndim=2)
+    _need(ids, "embedding ids", dtype=torch.int32, ndim=1)
+    v, h = table.shape
+    t = ids.shape[0]
+    if out is None:
+        out = torch.empty((t, h), dtype=torch.float32, device=table.device)
+    _need(out, "embedding out", dtype=torch.float32, shape=(t, h))
+    check(load().fsie_embedding(table.data_ptr(), dtype_code(table.dtype), ids.data_ptr(), out.data_ptr(),
+                                t, h, v, _stream()))
+    return out
+
+
+def rmsnorm(residual: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+            write_back: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm of ``residual (+ delta)`` (float32 stream, delta in ``out_dtype``) times ``weight``
+    (float32).  ``write_back`` stores the sum into ``residual``; ``rows`` (int32) selects rows."""
+    _need(residual, "rmsnorm residual", dtype=torch.float32, ndim=2)
+    t, h = residual.shape
+    _need(weight, "rmsnorm weight", dtype=torch.float32, shape=(h,))
+    if delta is not None:
+        _need(delta, "rmsnorm delta", dtype=out_dtype, shape=(t, h))
+    n_rows = t
+    if rows is not None:
+        _need(rows, "rmsnorm rows", dtype=torch.int32, ndim=1)
+        n_rows = rows.shape[0]
+    if out is None:
+        out = torch.empty((n_rows, h), dtype=out_dtype, device=residual.device)
+    _need(out, "rmsnorm out", dtype=out_dtype, shape=(n_rows, h))
+    check(load().fsie_rmsnorm(residual.data_ptr(), _ptr(delta), weight.data_ptr(), out.data_ptr(), _ptr(rows),
+                              n_rows, h, float(eps), dtype_code(out_dtype), int(write_back), _stream()))
+    return out
+
+
+def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """silu(x[:, :I]) * x[:, I:] for x [T, 2I]."""
+    _need(x, "swiglu input", ndim=2)
+    t, two_i = x.shape
+    if two_i % 2:
+        raise KernelError(f"swiglu: the input width {two_i} must be even")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((t, inter), dtype=x.dtype, device=x.device)
+    _need(out, "swiglu out", dtype=x.dtype, shape=(t, inter))
+    check(load().fsie_swiglu(x.data_ptr(), out.data_ptr(), t, inter, dtype_code(x.dtype), _stream()))
+    return out
+
+
+def residual_add(residual: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    _need(residual, "residual", dtype=torch.float32)
+    _need(delta, "delta", shape=residual.shape)
+    check(load().fsie_residual_add(residual.data_ptr(), delta.data_ptr(), residual.numel(),
+                                   dtype_code(delta.dtype), _stream()))
+    return residual
+
+
+def bias_add(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """y[r, :] += bias (float32) in place."""
+    _need(y, "bias_add y", ndim=2)
+    _need(bias, "bias", dtype=torch.float32, shape=(y.shape[1],))
+    check(load().fsie_bias_add(y.data_ptr(), bias.data_ptr(), y.shape[0], y.shape[1], dtype_code(y.dtype), _stream()))
+    return y
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
+                  inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor] = None,
+                  k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None,
+                  page_size: int = 0, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rotate the q and k heads of ``qkv`` [T, (n_heads + 2 n_kv) head_dim] in place by the angles
+    ``positions * inv_freq`` (float64 table of rotary_dim/2 entries; ``None`` = no rotation) and
+    copy k and v to the cache slots ``slots`` (int32 [T], negative = not stored) of pools laid out
+    [pages, n_kv, page_size, head_dim]."""
+    _need(qkv, "qkv", ndim=2)
+    t = qkv.shape[0]
+    if qkv.shape[1] != (n_heads + 2 * n_kv) * head_dim:
+        raise KernelError(f"qkv: width {qkv.shape[1]} != (heads {n_heads} + 2 * kv heads {n_kv}) * {head_dim}")
+    _need(positions, "positions", dtype=torch.int32, shape=(t,))
+    rotary_dim = 0
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", dtype=torch.float64, ndim=1)
+        rotary_dim = 2 * inv_freq.shape[0]
+    if bias is not None:
+        _need(bias, "qkv bias", dtype=torch.float32, shape=(qkv.shape[1],))
+    pool_slots = 0
+    if k_pool is not None:
+        if v_pool is None or slots is None:
+            raise KernelError("rope_kv_write: k_pool needs v_pool and slots")
+        _need(slots, "slots", dtype=torch.int32, shape=(t,))
+        _need(k_pool, "k_pool", dtype=qkv.dtype, ndim=4)
+        _need(v_pool, "v_pool", dtype=qkv.dtype, shape=k_pool.shape)
+        if tuple(k_pool.shape[1:]) != (n_kv, page_size, head_dim):
+            raise KernelError(f"k_pool: shape {tuple(k_pool.shape)} is not [pages, {n_kv}, {page_size}, {head_dim}]")
+        pool_slots = k_pool.shape[0] * page_size
+    check(load().fsie_rope_kv_write(qkv.data_ptr(), positions.data_ptr(), _ptr(slots), _ptr(inv_freq),
+                                    _ptr(bias), _ptr(k_pool), _ptr(v_pool), t, n_heads, n_kv, head_dim, rotary_dim,
+                                    page_size, pool_slots, dtype_code(qkv.dtype), _stream()))
+    return qkv
+
+
+def gemm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+         out_dtype: Optional[torch.dtype] = None, kind: int = GEMM_AUTO,
+         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [M, K] . weight [N, K]^T + bias [N] (float32) with float32 accumulation."""
+    _need(x, "gemm x", ndim=2)
+    _need(weight, "gemm weight", dtype=x.dtype, ndim=2)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"gemm: weight inner size {weight.shape[1]} does not match x's {k}")
+    if bias is not None:
+        _need(bias, "gemm bias", dtype=torch.float32, shape=(n,))
+    out_dtype = out_dtype or x.dtype
+    if out_dtype not in (x.dtype, torch.float32):
+        raise KernelError(f"gemm: output {out_dtype} from {x.dtype} operands is not offered")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _need(out, "gemm out", dtype=out_dtype, shape=(m, n))
+    check(load().fsie_gemm(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
+                           dtype_code(x.dtype), int(out_dtype == torch.float32), kind, _stream()))
+    return out
+
+
+def attention_tile_tokens(n_heads: int, n_kv: int) -> int:
+    n = load().fsie_attention_scalar_tile_tokens(n_heads, n_kv)
+    if n <= 0:
+        raise KernelError(f"attention: heads {n_heads} must be a positive multiple of kv heads {n_kv}")
+    return n
+
+
+def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                     block_tables: torch.Tensor, items: torch.Tensor, n_items: int, out: torch.Tensor,
+                     partials: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
+                     window: Optional[int], scale: float, n_query_rows: int) -> torch.Tensor:
+    """Attention of the work items over the paged cache (float32 arithmetic).
+
+    ``q`` is a view into rows of stride ``q_stride`` elements whose first n_heads*head_dim columns
+    are the queries; ``out`` is [n_query_rows, n_heads*head_dim]."""
+    if not q.is_cuda:
+        raise KernelError("attention q: must be on the GPU")
+    _need(k_pool, "k_pool", dtype=q.dtype, ndim=4)
+    _need(v_pool, "v_pool", dtype=q.dtype, shape=k_pool.shape)
+    _need(block_tables, "block_tables", dtype=torch.int32, ndim=2)
+    _need(items, "attention items", dtype=torch.int32, ndim=2)
+    if items.shape[1] != ATTN_ITEM_INTS or items.shape[0] < n_items:
+        raise KernelError(f"attention items: shape {tuple(items.shape)} does not hold {n_items} items")
+    _need(out, "attention out", dtype=q.dtype, shape=(n_query_rows, n_heads * head_dim))
+    pages, kvh, page_size, hd = k_pool.shape
+    if kvh != n_kv or hd != head_dim:
+        raise KernelError(f"k_pool: shape {tuple(k_pool.shape)} does not match kv heads {n_kv}, head_dim {head_dim}")
+    if q_stride < n_heads * head_dim:
+        raise KernelError("attention: q_stride is smaller than the query width")
+    if partials is not None:
+        _need(partials, "attention partials", dtype=torch.float32, ndim=1)
+    check(load().fsie_attention_scalar(q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+                                       block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(),
+                                       n_items, out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim,
+                                       page_size, int(window or 0), float(scale), dtype_code(q.dtype), _stream()))
+    return out
+
+
+def attention_merge(partials: torch.Tensor, merges: torch.Tensor, n_merges: int, out: torch.Tensor,
+                    n_heads: int, head_dim: int) -> torch.Tensor:
+    _need(partials, "attention partials", dtype=torch.float32, ndim=1)
+    _need(merges, "attention merges", dtype=torch.int32, ndim=2)
+    if merges.shape[1] != ATTN_MERGE_INTS or merges.shape[0] < n_merges:
+        raise KernelError(f"attention merges: shape {tuple(merges.shape)} does not hold {n_merges} items")
+    _need(out, "attention out", ndim=2)
+    check(load().fsie_attention_merge(partials.data_ptr(), merges.data_ptr(), n_merges, out.data_ptr(),
+                                      n_heads, head_dim, dtype_code(out.dtype), _stream()))
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+           top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+           uniform: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token id per row of float32 ``logits`` [n, V]: argmax where temperature <= 0 (or no
+    temperatures are given), else temperature/top-k/top-p sampling against ``uniform`` (float64)."""
+    _need(logits, "logits", dtype=torch.float32, ndim=2)
+    n, v = logits.shape
+    if temperature is not None:
+        _need(temperature, "temperature", dtype=torch.float32, shape=(n,))
+        if uniform is None:
+            raise KernelError("sample: temperatures need uniform numbers")
+        _need(uniform, "uniform", dtype=torch.float64, shape=(n,))
+    if top_k is not None:
+        _need(top_k, "top_k", dtype=torch.int32, shape=(n,))
+    if top_p is not None:
+        _need(top_p, "top_p", dtype=torch.float32, shape=(n,))
+    if out is None:
+        out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _need(out, "sample out", dtype=torch.int32, shape=(n,))
+    check(load().fsie_sample(logits.data_ptr(), n, v, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+                             _ptr(uniform), out.data_ptr(), _stream()))
+    return out

@@ -1,0 +1,132 @@
+"""Grouped-query attention over the paged cache."""
+
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..cache.manager import PagedNeed
+from ..ops.functions import ATTN_ITEM_INTS, ATTN_MERGE_INTS
+from .base import Mixer, ParamDecl, PositionEncoding, register_part
+from .linear import Linear
+from .rope import KVStore
+
+
+class AttentionPlanner:
+    """Cuts a step into the work items of the attention kernel (host side, once per step for all
+    layers with the same geometry).
+
+    A request's portion of n tokens at past length p becomes tiles of ``tile_tokens`` query
+    tokens; a tile reads the keys from the start of its window to its last token.  A portion
+    that fits one tile and reads more than ``split_keys`` keys (decoding against a long
+    context) is split over the keys instead, ``split_keys`` per item, and merged afterwards in
+    the order of the splits.  Whether a portion is split depends on the portion alone, never
+    on what else is in the batch.
+    """
+
+    def __init__(self, window: Optional[int], tile_tokens: int, split_keys: int):
+        self.window = window
+        self.tile_tokens = tile_tokens
+        self.split_keys = split_keys
+        self.key = ("attention", window, tile_tokens, split_keys)
+
+    def plan(self, host) -> Dict[str, object]:
+        items, merges = [], []
+        n_partial = 0
+        for s in range(host.n_seqs):
+            n, p, row0 = host.q_lens[s], host.past_lens[s], host.q_starts[s]
+            first_key = max(0, p - self.window + 1) if self.window else 0
+            total = p + n
+            if n <= self.tile_tokens and total - first_key > self.split_keys:
+                n_splits = -(-(total - first_key) // self.split_keys)
+                base = n_partial
+                for i in range(n_splits):
+                    kb = first_key + i * self.split_keys
+                    items.append((s, row0, n, p, kb, min(total, kb + self.split_keys), base + i * n, 0))
+                for t in range(n):
+                    merges.append((row0 + t, base + t, n_splits, n))
+                n_partial += n_splits * n
+            else:
+                for t0 in range(0, n, self.tile_tokens):
+                    nq = min(self.tile_tokens, n - t0)
+                    pos0 = p + t0
+                    kb = max(0, pos0 - self.window + 1) if self.window else 0
+                    items.append((s, row0 + t0, nq, pos0, kb, pos0 + nq, -1, 0))
+        return {
+            "items": np.asarray(items, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS),
+            "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
+            "n_items": len(items), "n_merges": len(merges), "n_partial": n_partial,
+        }
+
+
+@register_part("mixer", "gqa_attention")
+class GQAttention(Mixer):
+    """q/k/v projections (one matrix, optional bias), position encoding, causal attention with
+    kv head = q head // (heads / kv heads) and scale 1/sqrt(head_dim), output projection without
+    bias (src/model/model.cpp:110-129, src/model/nn.cpp:151-226).  ``window`` = number of latest
+    positions a query reads (None: all)."""
+
+    SPLIT_KEYS = 256
+
+    def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
+                 position: PositionEncoding, window: Optional[int] = None):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"attention: heads {n_heads} must be a multiple of kv heads {n_kv_heads}")
+        if head_dim > 256:
+            raise ValueError(f"attention: head_dim {head_dim} is larger than the kernels take (256)")
+        self.hidden_size, self.n_heads, self.n_kv, self.head_dim = hidden_size, n_heads, n_kv_heads, head_dim
+        self.window = window
+        self.position = position
+        self.q_dim, self.kv_dim = n_heads * head_dim, n_kv_heads * head_dim
+        self.qkv = Linear(hidden_size, self.q_dim + 2 * self.kv_dim, bias=qkv_bias)
+        self.o = Linear(self.q_dim, hidden_size)
+        self.scale = 1.0 / math.sqrt(head_dim)
+        self._planner: Optional[AttentionPlanner] = None
+
+    # parameters -------------------------------------------------------------------------
+    def param_decls(self) -> Dict[str, ParamDecl]:
+        decls = {"qkv_weight": ParamDecl((self.q_dim + 2 * self.kv_dim, self.hidden_size)),
+                 "o_weight": ParamDecl((self.hidden_size, self.q_dim))}
+        if self.qkv.has_bias:
+            decls["qkv_bias"] = ParamDecl((self.q_dim + 2 * self.kv_dim,), "vector", "bias")
+        return decls
+
+    qkv_weight = property(lambda s: s.qkv.weight, lambda s, t: setattr(s.qkv, "weight", t))
+    qkv_bias = property(lambda s: s.qkv.bias, lambda s, t: setattr(s.qkv, "bias", t))
+    o_weight = property(lambda s: s.o.weight, lambda s, t: setattr(s.o, "weight", t))
+
+    def prepare(self, device, compute_dtype) -> None:
+        self.position.prepare(device, compute_dtype)
+
+    # cache and plan ---------------------------------------------------------------------
+    def cache_need(self) -> PagedNeed:
+        return PagedNeed(self.n_kv, self.head_dim, self.window)
+
+    def planner(self) -> AttentionPlanner:
+        if self._planner is None:
+            self._planner = AttentionPlanner(self.window, ops.attention_tile_tokens(self.n_heads, self.n_kv),
+                                             self.SPLIT_KEYS)
+        return self._planner
+
+    # compute ----------------------------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        qkv = self.qkv(x, skip_bias=True)
+        store = KVStore(cache.k_pool, cache.v_pool, cache.slots, cache.page_size) if cache.writes else None
+        self.position.apply(qkv, self.n_heads, self.n_kv, self.head_dim, ctx, store, bias=self.qkv.bias)
+        plan = ctx.plan(self.planner())
+        t = x.shape[0]
+        out = torch.empty((t, self.q_dim), dtype=x.dtype, device=x.device)
+        partials = None
+        if plan.n_partial:
+            partials = torch.empty((plan.n_partial * self.n_heads * (self.head_dim + 2),), dtype=torch.float32,
+                                   device=x.device)
+        ops.attention_scalar(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
+                             plan.n_items, out, partials, self.n_heads, self.n_kv, self.head_dim, self.window,
+                             self.scale, t)
+        if plan.n_merges:
+            ops.attention_merge(partials, plan.merges, plan.n_merges, out, self.n_heads, self.head_dim)
+        return self.o(out)

@@ -1,0 +1,136 @@
+"""Interfaces of the parts a layer is put together from, and the registries that name them.
+
+A part is constructed from explicit sizes and constants, declares its parameters and what it
+needs from the cache, and computes on the tokens of one step.  It never sees a model
+configuration and does not know which model it is in.
+
+Kinds and their interfaces (``ctx`` is the step's ``StepContext``):
+
+  Norm             ``normed = norm(hidden)``; ``norm.rows(hidden, rows)`` for chosen rows.
+                   ``hidden`` is a ``HiddenState``: the float32 residual stream plus a pending
+                   delta that the next norm folds in (fused residual sum + norm).
+  Mixer            ``y = mixer.forward(x, ctx, cache)``; ``cache_need()`` says what it keeps per
+                   request: a ``PagedNeed`` (entries per token), a ``StateNeed`` (fixed size) or
+                   nothing; ``planner()`` may name per-step index tables it wants built on the host.
+  FeedForward      ``y = ffn.forward(x, ctx)``.
+  PositionEncoding ``pos.apply(qkv, n_heads, n_kv, head_dim, ctx, store)`` rotates/marks q and k
+                   in place and hands k and v to the cache through ``store``.
+  Block            the arrangement: ``block.forward(hidden, ctx, cache)``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamDecl:
+    """A parameter of a part.  ``storage``: 'matrix' (compute dtype), 'vector' (float32) or
+    'int_table' (int32).  ``init`` names the random-weights distribution."""
+
+    shape: Tuple[int, ...]
+    storage: str = "matrix"
+    init: str = "weight"
+
+
+class HiddenState:
+    """The residual stream of a step: ``residual`` float32 [T, H] and a pending ``delta``
+    [T, H] in the compute dtype that has not been added yet."""
+
+    __slots__ = ("residual", "delta")
+
+    def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None):
+        self.residual = residual
+        self.delta = delta
+
+
+class Part:
+    kind: str = "part"
+
+    def param_decls(self) -> Dict[str, ParamDecl]:
+        return {}
+
+    def prepare(self, device, compute_dtype: torch.dtype) -> None:
+        """Called once after the parameters are set (tables, constants on the device)."""
+
+
+class Norm(Part):
+    kind = "norm"
+
+    def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
+        raise NotImplementedError
+
+    def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    kind = "mixer"
+
+    def cache_need(self):
+        return None
+
+    def planner(self):
+        return None
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    kind = "feed_forward"
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    kind = "position"
+
+    def apply(self, qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, ctx, store,
+              bias: Optional[torch.Tensor] = None) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    kind = "block"
+
+    def forward(self, hidden: HiddenState, ctx, cache) -> None:
+        raise NotImplementedError
+
+    def sub_parts(self) -> Dict[str, Part]:
+        return {}
+
+
+# ------------------------------------------------------------------------------ registries
+_REGISTRIES: Dict[str, Dict[str, Callable[..., Part]]] = {
+    "norm": {}, "mixer": {}, "feed_forward": {}, "position": {}, "block": {},
+}
+
+
+def register_part(kind: str, name: str):
+    """Class decorator: make a part constructible by name, e.g.
+    ``@register_part("mixer", "my_mixer")``.  A test or an extension can register parts of its
+    own without touching the engine's files."""
+    if kind not in _REGISTRIES:
+        raise KeyError(f"unknown part kind '{kind}' (known: {sorted(_REGISTRIES)})")
+
+    def deco(cls):
+        _REGISTRIES[kind][name] = cls
+        return cls
+
+    return deco
+
+
+def make_part(kind: str, name: str, **params) -> Part:
+    table = _REGISTRIES[kind]
+    if name not in table:
+        raise KeyError(f"no {kind} named '{name}' (known: {sorted(table)})")
+    return table[name](**params)
+
+
+def known_parts(kind: str):
+    return sorted(_REGISTRIES[kind])

@@ -1,0 +1,127 @@
+"""Loading by tensor name.
+
+An architecture describes what it expects as a list of ``ParamBinding``: "this parameter of
+this part is made of these checkpoint tensors (concatenated along dim 0), stored this way".
+The loader compares the expectation with the file, reports *all* missing and unexpected tensors
+and wrong shapes in one error, then fills the parts.
+
+Storage on the device:
+  * ``matrix``  - the run's compute dtype (bfloat16, or float32 in the 32-bit path);
+  * ``vector``  - float32 always (norm weights, biases: exact for either stored precision, so
+                  a tensor stored in 32-bit stays so);
+  * ``int_table`` - int32.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .safetensors_file import SafetensorsFile
+
+
+class WeightsError(RuntimeError):
+    """The checkpoint does not hold what the architecture expects."""
+
+    def __init__(self, message: str, missing=(), unexpected=(), wrong_shape=()):
+        super().__init__(message)
+        self.missing = list(missing)
+        self.unexpected = list(unexpected)
+        self.wrong_shape = list(wrong_shape)
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """One tensor of the checkpoint.  ``init`` names the distribution of the random-weights
+    mode: 'weight' N(0, 0.02), 'norm' 1 + N(0, 0.02), 'bias' N(0, 0.02), 'int' uniform ids."""
+
+    name: str
+    shape: Tuple[int, ...]
+    init: str = "weight"
+
+
+@dataclass
+class ParamBinding:
+    """Parameter ``attr`` of ``owner`` = concat(sources, dim 0), kept as ``storage``."""
+
+    owner: Any
+    attr: str
+    sources: Sequence[TensorSpec]
+    storage: str = "matrix"  # matrix | vector | int_table
+
+
+def expected_tensors(bindings: Sequence[ParamBinding]) -> Dict[str, TensorSpec]:
+    out: Dict[str, TensorSpec] = {}
+    for b in bindings:
+        for s in b.sources:
+            if s.name in out and out[s.name].shape != s.shape:
+                raise ValueError(f"tensor {s.name} is expected with two shapes")
+            out[s.name] = s
+    return out
+
+
+def check_against(bindings: Sequence[ParamBinding], found: Dict[str, Tuple[int, ...]],
+                  ignore_unexpected: Sequence[str] = ()) -> None:
+    """Raise one ``WeightsError`` that lists everything wrong."""
+    expect = expected_tensors(bindings)
+    missing = sorted(n for n in expect if n not in found)
+    unexpected = sorted(n for n in found if n not in expect and n not in ignore_unexpected)
+    wrong = sorted((n, expect[n].shape, tuple(found[n])) for n in expect
+                   if n in found and tuple(found[n]) != tuple(expect[n].shape))
+    if not (missing or unexpected or wrong):
+        return
+    lines = ["checkpoint does not match the model:"]
+    if missing:
+        lines.append(f"  missing tensors ({len(missing)}):")
+        lines += [f"    {n}  expected shape {list(expect[n].shape)}" for n in missing]
+    if unexpected:
+        lines.append(f"  unexpected tensors ({len(unexpected)}):")
+        lines += [f"    {n}  shape {list(found[n])}" for n in unexpected]
+    if wrong:
+        lines.append(f"  wrong shapes ({len(wrong)}):")
+        lines += [f"    {n}  expected {list(e)}, found {list(f)}" for n, e, f in wrong]
+    raise WeightsError("\n".join(lines), missing, unexpected, wrong)
+
+
+def _to_storage(t: torch.Tensor, storage: str, compute_dtype: torch.dtype) -> torch.dtype:
+    if storage == "matrix":
+        return compute_dtype
+    if storage == "vector":
+        return torch.float32
+    if storage == "int_table":
+        return torch.int32
+    raise ValueError(f"unknown storage '{storage}'")
+
+
+def fill_parts(bindings: Sequence[ParamBinding], get_tensor, compute_dtype: torch.dtype,
+               device) -> int:
+    """Set every bound parameter; returns the bytes placed on the device.  Bindings with the
+    same sources and storage share one device tensor (tied embeddings)."""
+    shared: Dict[Tuple, torch.Tensor] = {}
+    total = 0
+    for b in bindings:
+        key = (tuple(s.name for s in b.sources), b.storage)
+        if key not in shared:
+            target = _to_storage(None, b.storage, compute_dtype)
+            pieces = []
+            for s in b.sources:
+                t = get_tensor(s.name)
+                if b.storage == "int_table" and t.dtype.is_floating_point:
+                    raise WeightsError(f"tensor {s.name} must hold integers, found {t.dtype}")
+                pieces.append(t.to(device=device, dtype=target, non_blocking=False))
+            value = pieces[0] if len(pieces) == 1 else torch.cat(pieces, dim=0)
+            value = value.contiguous()
+            shared[key] = value
+            total += value.numel() * value.element_size()
+        setattr(b.owner, b.attr, shared[key])
+    return total
+
+
+def load_weights(path, bindings: Sequence[ParamBinding], compute_dtype: torch.dtype, device,
+                 ignore_unexpected: Sequence[str] = ()) -> int:
+    """Check ``path`` (a .safetensors file) against ``bindings`` and fill the parts."""
+    f = SafetensorsFile(path)
+    check_against(bindings, {n: f.shape(n) for n in f.names()}, ignore_unexpected)
+    return fill_parts(bindings, f.get, compute_dtype, device)
