@@ -1,0 +1,85 @@
+"""Text-in / text-out entry point, in the manner of the reference's ``engine.llm``
+(python/engine/llm.py:33-77)."""
+
+from __future__ import annotations
+
+import json
+from dataclasses import dataclass
+from pathlib import Path
+from typing import List, Optional, Sequence
+
+from ..sampling.params import SamplingParams
+from .engine import Engine
+from .model import Model
+
+
+def _read_eos_id(model_dir: Path) -> int:
+    """generation_config.json, then config.json: ``eos_token_id``; a list gives its first
+    element; -1 if unspecified (python/engine/llm.py:18-30)."""
+    for name in ("generation_config.json", "config.json"):
+        path = model_dir / name
+        if not path.exists():
+            continue
+        eos = json.loads(path.read_text(encoding="utf-8")).get("eos_token_id")
+        if isinstance(eos, list):
+            eos = eos[0] if eos else None
+        if eos is not None:
+            return int(eos)
+    return -1
+
+
+@dataclass
+class GenerationConfig:
+    max_tokens: int = 64
+    temperature: float = 0.0  # <= 0 is greedy
+    top_k: int = 0
+    top_p: float = 1.0
+
+
+class LLM:
+    """Load a model folder and generate through the engine.
+
+    Options of the reference keep their names and meanings: ``block_size`` (tokens per cache
+    page), ``num_blocks`` (pages in the pool), ``seed`` (sampling), ``max_batch`` (most requests
+    running at once), ``eos_id`` (default: read from the folder).  ``dtype`` ('bfloat16' or
+    'float32'), ``max_tokens_per_step`` and ``prefill_chunk`` are this engine's.
+    ``enable_prefix_cache`` is accepted and has no effect (no prefix cache here); ``quantize``
+    is refused (no quantized weights here)."""
+
+    def __init__(self, model_dir, *, block_size: int = 16, num_blocks: int = 2048, seed: int = 0,
+                 max_batch: int = 256, eos_id: Optional[int] = None, enable_prefix_cache: bool = True,
+                 quantize: bool = False, dtype: str = "bfloat16", device: str = "cuda:0",
+                 max_tokens_per_step: int = 2048, prefill_chunk: Optional[int] = None):
+        if quantize:
+            raise NotImplementedError("LLM: quantized weights are not part of this engine")
+        model_dir = Path(model_dir)
+        self.model = Model.from_pretrained(model_dir, dtype=dtype, device=device)
+        self.engine = Engine(self.model, block_size, num_blocks, seed, max_batch, enable_prefix_cache,
+                             max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk)
+        self.eos_id = _read_eos_id(model_dir) if eos_id is None else eos_id
+        self._model_dir = model_dir
+        self._tokenizer = None
+
+    @property
+    def tokenizer(self):
+        if self._tokenizer is None:
+            from .tokenizer import EngineTokenizer
+
+            self._tokenizer = EngineTokenizer.from_model_dir(self._model_dir)
+        return self._tokenizer
+
+    def _params(self, config: GenerationConfig) -> SamplingParams:
+        return SamplingParams(config.temperature, config.top_k, config.top_p)
+
+    def generate_ids(self, prompt_ids: Sequence[int], config: Optional[GenerationConfig] = None) -> List[int]:
+        config = config or GenerationConfig()
+        return self.engine.generate(list(prompt_ids), self._params(config), config.max_tokens, self.eos_id)
+
+    def generate_ids_batch(self, prompts: Sequence[Sequence[int]],
+                           config: Optional[GenerationConfig] = None) -> List[List[int]]:
+        config = config or GenerationConfig()
+        return self.engine.generate_batch(prompts, self._params(config), config.max_tokens, self.eos_id)
+
+    def generate(self, prompt: str, config: Optional[GenerationConfig] = None) -> str:
+        ids = self.tokenizer.encode(prompt)
+        return self.tokenizer.decode(self.generate_ids(ids, config))

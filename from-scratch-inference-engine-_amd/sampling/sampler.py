@@ -1,0 +1,58 @@
+"""Chooses next tokens on the device.
+
+The reference samples on the host with one generator shared by all requests
+(src/sampler/sampler.cpp:25-88), so its draws depend on what else is in the batch.  Here every
+draw has its own uniform number, a pure function of (engine seed, request id, index of the
+token in the request's output), and the kernel turns it into a token: what a request samples
+does not depend on the batch it shares.
+"""
+
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from .. import ops
+from .params import SamplingParams
+
+_MASK = (1 << 64) - 1
+
+
+def _splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    z = x
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    return z ^ (z >> 31)
+
+
+def uniform_for(seed: int, request_id: int, index: int) -> float:
+    """A number in [0, 1) for the ``index``-th sampled token of ``request_id``."""
+    z = _splitmix64(seed & _MASK)
+    z = _splitmix64(z ^ (request_id & _MASK))
+    z = _splitmix64(z ^ (index & _MASK))
+    return (z >> 11) / float(1 << 53)
+
+
+class Sampler:
+    def __init__(self, seed: int = 0):
+        self.seed = int(seed)
+
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], request_ids: Sequence[int],
+               indices: Sequence[int]) -> List[int]:
+        """One token per row of ``logits`` [n, vocab] (float32, on the device)."""
+        n = logits.shape[0]
+        if not (len(params) == len(request_ids) == len(indices) == n):
+            raise ValueError("sample: one set of parameters, request id and index per row")
+        if n == 0:
+            return []
+        if all(p.greedy for p in params):
+            return ops.sample(logits).tolist()
+        dev = logits.device
+        temperature = torch.tensor([max(float(p.temperature), 0.0) for p in params], dtype=torch.float32, device=dev)
+        top_k = torch.tensor([int(p.top_k) for p in params], dtype=torch.int32, device=dev)
+        top_p = torch.tensor([float(p.top_p) for p in params], dtype=torch.float32, device=dev)
+        uniform = torch.tensor([uniform_for(self.seed, r, i) for r, i in zip(request_ids, indices)],
+                               dtype=torch.float64, device=dev)
+        return ops.sample(logits, temperature, top_k, top_p, uniform).tolist()

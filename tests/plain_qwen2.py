@@ -215,7 +215,7 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, u
     p_i = exp(l_i/T - max/T) normalised, keeps the smallest prefix whose cumulative mass
     reaches top_p, and draws against u * nucleus_sum.  Here the uniform number ``u`` is an
     argument, the kept set is the same, and the draw walks the kept tokens in vocabulary order
-    (the engine's documented order); ties at the top-k cut keep the lower token ids.
+    (the engine's documented order); tokens tied with the last kept one are kept too.
     """
     if temperature <= 0.0:
         return argmax(logits)
@@ -223,6 +223,8 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, u
     vocab = vals.numel()
     order = sorted(range(vocab), key=lambda i: (-float(vals[i]), i))
     keep = vocab if not (0 < top_k < vocab) else top_k
+    while keep < vocab and float(vals[order[keep]]) == float(vals[order[keep - 1]]):
+        keep += 1  # the engine keeps every token tied with the k-th
     order = order[:keep]
     mx = float(vals[order[0]]) / temperature
     probs = [math.exp(float(vals[i]) / temperature - mx) for i in order]

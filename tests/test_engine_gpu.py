@@ -1,0 +1,173 @@
+"""Generation through the entry points on the GPU: greedy against the plain implementation,
+long decoding, the first tokens of a sequence, the scheduler with a small pool, sampling."""
+
+import json
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_qwen2 as plain
+
+pytestmark = pytest.mark.gpu
+
+
+def plain_greedy(model_dir, prompt, n, eos=-1):
+    cfg, w = plain.read_config(model_dir), plain.read_weights(model_dir)
+    ids, out = list(prompt), []
+    for _ in range(n):
+        tok = plain.argmax(plain.forward(cfg, w, ids)[-1])
+        out.append(tok)
+        ids.append(tok)
+        if tok == eos:
+            break
+    return out
+
+
+@pytest.fixture(scope="module")
+def llms(model_dirs):
+    from from_scratch_inference_engine_amd import LLM
+
+    return {(name, dtype): LLM(model_dirs[name], dtype=dtype, block_size=bs, num_blocks=64, max_batch=8)
+            for name, bs in (("A", 4), ("B", 8)) for dtype in ("float32", "bfloat16")}
+
+
+@pytest.mark.parametrize("name, lengths", [("A", [5, 11, 17]), ("B", [1, 7, 33])])
+def test_greedy_generation_matches_plain_float32(llms, model_dirs, name, lengths):
+    from from_scratch_inference_engine_amd import GenerationConfig
+
+    llm = llms[(name, "float32")]
+    vocab = helpers.TINY[name][0]["vocab_size"]
+    prompts = [helpers.token_ids(vocab, n, 50 + n) for n in lengths]
+    want = [plain_greedy(model_dirs[name], p, 16) for p in prompts]
+    cfg = GenerationConfig(max_tokens=16, temperature=0.0)
+    saved, llm.eos_id = llm.eos_id, -1
+    try:
+        assert [llm.generate_ids(p, cfg) for p in prompts] == want           # one at a time
+        assert llm.generate_ids_batch(prompts, cfg) == want                   # batched by the scheduler
+    finally:
+        llm.eos_id = saved
+    assert llm.engine.free_blocks() == 64
+
+
+def test_eos_from_the_folder_stops_generation(llms, model_dirs):
+    from from_scratch_inference_engine_amd import GenerationConfig
+
+    llm = llms[("B", "float32")]
+    assert llm.eos_id == 7  # config.json of B
+    prompt = helpers.token_ids(509, 9, 3)
+    free = plain_greedy(model_dirs["B"], prompt, 12)
+    llm.eos_id = free[4]
+    try:
+        got = llm.generate_ids(prompt, GenerationConfig(max_tokens=12))
+    finally:
+        llm.eos_id = 7
+    stop = free.index(free[4])
+    assert got == free[:stop + 1]  # the end-of-sequence token is kept
+
+
+def test_bfloat16_generation_follows_plain_where_the_choice_is_clear(llms, model_dirs):
+    """bfloat16 rounding may flip a near-tie; wherever the plain top-2 gap is wide the token is
+    the plain one (teacher-forced on the plain continuation)."""
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+
+    llm = llms[("B", "bfloat16")]
+    prompt = helpers.token_ids(509, 40, 4)
+    cont = plain_greedy(model_dirs["B"], prompt, 24)
+    ids = prompt + cont
+    ref = plain.forward_dir(model_dirs["B"], ids)
+    runner = llm.engine.runner
+    rc = runner.manager.open("teacher")
+    logits = runner.step([StepEntry(rc, ids, list(range(len(ids))))]).cpu()
+    runner.manager.close(rc)
+    top2 = ref.topk(2, dim=-1).values
+    clear = (top2[:, 0] - top2[:, 1]) > 2 * helpers.BF16_REL * ref.abs().max()
+    assert clear.sum() >= 1
+    assert torch.equal(logits.argmax(-1)[clear], ref.argmax(-1)[clear])
+    helpers.assert_close_to_plain(logits.numpy(), ref.numpy(), "bfloat16", "teacher forced")
+
+
+def test_long_decoding_and_first_tokens(llms, model_dirs):
+    """250 positions of B, all but the first token decoded one by one: checks the first tokens of
+    a sequence (positions 0, 1, 2 at every page offset) and a long run over many pages."""
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+
+    ids = helpers.token_ids(509, 250, 5)
+    ref = plain.forward_dir(model_dirs["B"], ids).numpy()
+    for dtype in ("float32", "bfloat16"):
+        runner = llms[("B", dtype)].engine.runner
+        rc = runner.manager.open("long")
+        rows = [runner.step([StepEntry(rc, ids[t:t + 1], [0])]) for t in range(len(ids))]
+        runner.manager.close(rc)
+        got = torch.cat(rows).cpu().numpy()
+        helpers.assert_close_to_plain(got[:3], ref[:3], dtype, f"first tokens {dtype}")
+        helpers.assert_close_to_plain(got, ref, dtype, f"long decoding {dtype}")
+
+
+def test_small_pool_preempts_and_still_matches(model_dirs):
+    """tests/cpp/test_engine.cpp:103-128 on the GPU: pages run out, the youngest request is
+    preempted and recomputed; outputs equal the plain greedy continuation."""
+    from from_scratch_inference_engine_amd import Engine, SamplingParams, SeqStatus, load_model
+
+    model = load_model(model_dirs["A"], dtype="float32")
+    engine = Engine(model, block_size=4, num_blocks=6, max_batch=4, max_tokens_per_step=8)
+    prompts = [helpers.token_ids(256, n, 70 + n) for n in (4, 4, 7, 3)]
+    ids = [engine.add_request(p, SamplingParams(temperature=0.0), max_tokens=9) for p in prompts]
+    steps = 0
+    while engine.has_work():
+        engine.step()
+        steps += 1
+        assert steps < 400
+    assert engine.preemptions() > 0
+    assert all(engine.status(i) == SeqStatus.Finished for i in ids)
+    for i, p in zip(ids, prompts):
+        assert engine.output(i) == plain_greedy(model_dirs["A"], p, 9)
+    assert engine.free_blocks() == 6
+    with pytest.raises(ValueError, match="never run"):
+        engine.add_request(list(range(20)), max_tokens=8)
+    with pytest.raises(IndexError, match="vocabulary"):
+        engine.add_request([1, 256], max_tokens=2)
+
+
+def test_temperature_sampling_is_reproducible_and_independent_of_the_batch(llms):
+    """Two engines with the same seed: all requests at once in one, one at a time in the other.
+    Draws belong to (seed, request, token index), so the outputs are the same."""
+    from from_scratch_inference_engine_amd import Engine, SamplingParams
+
+    model = llms[("B", "float32")].model
+    prompts = [helpers.token_ids(509, n, 80 + n) for n in (1, 7, 33, 64, 90)]
+    params = SamplingParams(temperature=0.7)
+
+    def engine(seed):
+        return Engine(model, block_size=8, num_blocks=64, seed=seed, max_batch=8, max_tokens_per_step=48,
+                      prefill_chunk=16)
+
+    together = engine(5).generate_batch(prompts, params, max_tokens=12)
+    one = engine(5)
+    alone = [one.generate(p, params, max_tokens=12) for p in prompts]
+    assert together == alone
+    assert engine(6).generate_batch(prompts, params, max_tokens=12) != together
+    greedy = engine(5).generate_batch(prompts, SamplingParams(temperature=0.0), max_tokens=12)
+    assert greedy != together
+    # the same mixed, chunked run, greedy: the plain continuation of every prompt
+    assert greedy == [plain_greedy(llms[("B", "float32")]._model_dir, p, 12) for p in prompts]
+
+
+def test_command_line_generate(model_dirs):
+    prompt = helpers.token_ids(256, 6, 9)
+    cmd = [sys.executable, "-m", "from_scratch_inference_engine_amd", "generate", "--model-dir", str(model_dirs["A"]),
+           "--dtype", "float32", "--prompt-ids", " ".join(map(str, prompt)), "--max-tokens", "8", "--block-size", "4",
+           "--num-blocks", "32", "--json"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300, cwd=str(helpers.ROOT))
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    out = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert out["outputs"] == [plain_greedy(model_dirs["A"], prompt, 8)]
+
+
+def test_graft_entry_smoke():
+    import __graft_entry__ as entry
+
+    entry.smoke()

@@ -1,0 +1,164 @@
+"""The safetensors container, loading by tensor name with one clear error, random weights."""
+
+import json
+import struct
+
+import pytest
+import torch
+
+import helpers
+from from_scratch_inference_engine_amd.models import build_model_spec, parse_config
+from from_scratch_inference_engine_amd.weights import (SafetensorsError, SafetensorsFile, WeightsError,
+                                                       load_weights, write_random_model, write_safetensors)
+from from_scratch_inference_engine_amd.weights.loader import check_against, fill_parts
+
+
+def _raw_file(path, header: dict, data: bytes, header_len=None):
+    text = json.dumps(header).encode()
+    path.write_bytes(struct.pack("<Q", len(text) if header_len is None else header_len) + text + data)
+    return path
+
+
+def test_reads_the_reference_fixture(tmp_path):
+    # tests/cpp/test_safetensors.cpp:26-39: F32 [2,2] and BF16 [2] (0x3F80 -> 1, 0x4000 -> 2)
+    data = struct.pack("<4f", 1.0, 2.0, 3.0, 4.0) + struct.pack("<2H", 0x3F80, 0x4000)
+    f = SafetensorsFile(_raw_file(tmp_path / "m.safetensors", {
+        "__metadata__": {"format": "pt"},
+        "a": {"dtype": "F32", "shape": [2, 2], "data_offsets": [0, 16]},
+        "b": {"dtype": "BF16", "shape": [2], "data_offsets": [16, 20]}}, data))
+    assert f.get("a").tolist() == [[1.0, 2.0], [3.0, 4.0]] and f.dtype("a") == torch.float32
+    assert f.get("b").float().tolist() == [1.0, 2.0] and f.dtype("b") == torch.bfloat16
+    assert "a" in f and "c" not in f
+    with pytest.raises(SafetensorsError, match="missing tensor 'c'"):
+        f.get("c")
+
+
+@pytest.mark.parametrize("header, data, header_len, message", [
+    (None, b"\x01\x02", None, "smaller than"),
+    ({"a": {"dtype": "F32", "shape": [1], "data_offsets": [0, 4]}}, b"\0" * 4, 10 ** 9, "exceeds"),
+    ({"a": {"dtype": "F32", "shape": [2], "data_offsets": [0, 4]}}, b"\0" * 4, None, "byte count"),
+    ({"a": {"dtype": "F32", "shape": [1], "data_offsets": [0, 8]}}, b"\0" * 4, None, "out of range"),
+    ({"a": {"dtype": "Q4", "shape": [1], "data_offsets": [0, 4]}}, b"\0" * 4, None, "unsupported dtype"),
+    ({"a": {"dtype": "F32", "shape": [-1], "data_offsets": [0, 4]}}, b"\0" * 4, None, "negative"),
+    ({"a": {"dtype": "F32", "shape": [1], "data_offsets": [0, 4]},
+      "b": {"dtype": "F32", "shape": [1], "data_offsets": [2, 6]}}, b"\0" * 8, None, "overlapping"),
+    ({"a": {"dtype": "F32", "shape": [1]}}, b"\0" * 4, None, "malformed"),
+])
+def test_malformed_files_are_refused(tmp_path, header, data, header_len, message):
+    p = tmp_path / "bad.safetensors"
+    if header is None:
+        p.write_bytes(data)
+    else:
+        _raw_file(p, header, data, header_len)
+    with pytest.raises(SafetensorsError, match=message):
+        SafetensorsFile(p)
+
+
+def test_duplicate_names_and_bad_json(tmp_path):
+    text = b'{"a":{"dtype":"F32","shape":[1],"data_offsets":[0,4]},"a":{"dtype":"F32","shape":[1],"data_offsets":[4,8]}}'
+    p = tmp_path / "dup.safetensors"
+    p.write_bytes(struct.pack("<Q", len(text)) + text + b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="duplicate"):
+        SafetensorsFile(p)
+    p.write_bytes(struct.pack("<Q", 5) + b"{nope" + b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="invalid header JSON"):
+        SafetensorsFile(p)
+
+
+def test_round_trip_with_the_safetensors_package(tmp_path):
+    from safetensors.torch import load_file, save_file
+
+    g = torch.Generator().manual_seed(0)
+    tensors = {"w": torch.randn(3, 5, generator=g).bfloat16(), "v": torch.randn(7, generator=g),
+               "i": torch.arange(6, dtype=torch.int32).reshape(2, 3)}
+    write_safetensors(tmp_path / "ours.safetensors", tensors)
+    theirs = load_file(str(tmp_path / "ours.safetensors"))
+    save_file(tensors, str(tmp_path / "theirs.safetensors"))
+    ours = SafetensorsFile(tmp_path / "theirs.safetensors")
+    for k, t in tensors.items():
+        assert torch.equal(theirs[k], t) and torch.equal(ours.get(k), t) and ours.dtype(k) == t.dtype
+
+
+def _spec(cfg):
+    return build_model_spec(parse_config(cfg))
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    cfg = helpers.TINY_B
+    tensors = helpers.random_tensors(cfg, 0)
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["lm_head.weight"]
+    tensors["model.layers.0.self_attn.q_norm.weight"] = torch.zeros(32, dtype=torch.bfloat16)
+    tensors["model.layers.2.self_attn.k_proj.bias"] = torch.zeros(64, dtype=torch.bfloat16)
+    tensors["model.embed_tokens.weight"] = torch.zeros(509, 191, dtype=torch.bfloat16)
+    d = helpers.make_model_dir(tmp_path / "m", cfg, 0, tensors=tensors)
+    with pytest.raises(WeightsError) as err:
+        load_weights(d / "model.safetensors", _spec(cfg).bindings, torch.bfloat16, "cpu")
+    e = err.value
+    assert e.missing == ["lm_head.weight", "model.layers.1.mlp.up_proj.weight"]
+    assert e.unexpected == ["model.layers.0.self_attn.q_norm.weight"]
+    assert [w[0] for w in e.wrong_shape] == ["model.embed_tokens.weight", "model.layers.2.self_attn.k_proj.bias"]
+    text = str(e)
+    for piece in ("missing tensors (2)", "unexpected tensors (1)", "wrong shapes (2)", "expected [509, 192], found [509, 191]",
+                  "model.layers.1.mlp.up_proj.weight  expected shape [320, 192]"):
+        assert piece in text
+
+
+def test_storage_kinds_and_fusion(tmp_path):
+    """Matrices take the compute dtype, vectors stay float32 whatever the file stores, q/k/v
+    and gate/up are concatenated in that order, a tied head shares the embedding's memory."""
+    cfg = helpers.TINY_A
+    tensors = helpers.random_tensors(cfg, 3, torch.float32)
+    d = helpers.make_model_dir(tmp_path / "m", cfg, 3, tensors=tensors)
+    for dtype in (torch.bfloat16, torch.float32):
+        spec = _spec(cfg)
+        load_weights(d / "model.safetensors", spec.bindings, dtype, "cpu")
+        mixer, ffn = spec.layers[1].mixer, spec.layers[1].ffn
+        p = "model.layers.1."
+        want = torch.cat([tensors[p + f"self_attn.{n}_proj.weight"] for n in "qkv"]).to(dtype)
+        assert mixer.qkv_weight.dtype == dtype and torch.equal(mixer.qkv_weight, want)
+        assert mixer.qkv_bias.dtype == torch.float32
+        assert torch.equal(mixer.qkv_bias, torch.cat([tensors[p + f"self_attn.{n}_proj.bias"] for n in "qkv"]))
+        assert torch.equal(ffn.gate_up_weight, torch.cat([tensors[p + "mlp.gate_proj.weight"], tensors[p + "mlp.up_proj.weight"]]).to(dtype))
+        assert spec.layers[0].mixer_norm.weight.dtype == torch.float32
+        assert torch.equal(spec.final_norm.weight, tensors["model.norm.weight"])
+        assert spec.lm_head.weight.data_ptr() == spec.embedding.weight.data_ptr()
+
+
+def test_tied_checkpoint_may_carry_a_head_and_int_tables():
+    cfg = helpers.TINY_A
+    spec = _spec(cfg)
+    found = {n: s for n, s in helpers.expected_tensor_shapes(cfg).items()}
+    found["lm_head.weight"] = (256, 64)
+    check_against(spec.bindings, found, spec.ignore_unexpected)  # no error
+    with pytest.raises(WeightsError, match="unexpected"):
+        check_against(spec.bindings, found)
+    # integer tables are kept as int32, and a float tensor in their place is refused
+    from from_scratch_inference_engine_amd.weights import ParamBinding, TensorSpec
+
+    class Holder:
+        table = None
+    b = [ParamBinding(Holder, "table", [TensorSpec("t", (4,), "int")], "int_table")]
+    fill_parts(b, lambda n: torch.arange(4, dtype=torch.int64), torch.bfloat16, "cpu")
+    assert Holder.table.dtype == torch.int32 and Holder.table.tolist() == [0, 1, 2, 3]
+    with pytest.raises(WeightsError, match="integers"):
+        fill_parts(b, lambda n: torch.zeros(4), torch.bfloat16, "cpu")
+
+
+def test_random_model_folder(tmp_path):
+    cfg = parse_config(helpers.TINY_B)
+    a = write_random_model(cfg, 11, tmp_path / "a")
+    b = write_random_model(cfg, 11, tmp_path / "b")
+    c = write_random_model(cfg, 12, tmp_path / "c", torch.float32)
+    fa, fb, fc = (SafetensorsFile(x / "model.safetensors") for x in (a, b, c))
+    assert sorted(fa.names()) == sorted(helpers.expected_tensor_shapes(helpers.TINY_B))
+    for n in fa.names():
+        assert fa.shape(n) == helpers.expected_tensor_shapes(helpers.TINY_B)[n]
+        assert torch.equal(fa.get(n), fb.get(n)) and fa.dtype(n) == torch.bfloat16 and fc.dtype(n) == torch.float32
+    assert not torch.equal(fa.get("lm_head.weight").float(), fc.get("lm_head.weight"))
+    w = fc.get("model.layers.0.mlp.down_proj.weight")
+    assert abs(w.std().item() - 0.02) < 0.002 and abs(w.mean().item()) < 0.002
+    assert abs(fc.get("model.norm.weight").mean().item() - 1.0) < 0.01
+    assert parse_config(json.loads((a / "config.json").read_text())) == cfg
+    # the written folder loads without complaint
+    load_weights(a / "model.safetensors", _spec(helpers.TINY_B).bindings, torch.bfloat16, "cpu")
