@@ -10,6 +10,7 @@
 #include <stdint.h>
 
 #define FSIE_GEMM_SKINNY_MAX_M 8
+#define FSIE_GEMM_MFMA_SKINNY_MAX_M 64
 
 // one attention work item = 8 int32
 #define FSIE_ATTN_ITEM_INTS 8
@@ -46,6 +47,9 @@ int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int32_t* slots
 
 int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, int N, int K, int dtype,
               int out_f32, int kind, hipStream_t stream);
+
+int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
+                          int out_f32, int waves, hipStream_t stream);
 
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,

@@ -12,6 +12,7 @@ F32, BF16 = 0, 1
 ATTN_ITEM_INTS = 8
 ATTN_MERGE_INTS = 4
 GEMM_SKINNY_MAX_M = 8
+GEMM_MFMA_SKINNY_MAX_M = 64
 GEMM_AUTO, GEMM_TILED, GEMM_SKINNY = 0, 1, 2
 
 
@@ -165,6 +166,29 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = N
     _need(out, "gemm out", dtype=out_dtype, shape=(m, n))
     check(load().fsie_gemm(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
                            dtype_code(x.dtype), int(out_dtype == torch.float32), kind, _stream()))
+    return out
+
+
+def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                     out_dtype: Optional[torch.dtype] = None, waves: int = 0,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same product on the matrix cores for bfloat16 and at most 64 rows (K a multiple of 8)."""
+    _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
+    _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"gemm: weight inner size {weight.shape[1]} does not match x's {k}")
+    if bias is not None:
+        _need(bias, "gemm bias", dtype=torch.float32, shape=(n,))
+    out_dtype = out_dtype or x.dtype
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise KernelError(f"gemm: output {out_dtype} is not offered")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _need(out, "gemm out", dtype=out_dtype, shape=(m, n))
+    check(load().fsie_gemm_mfma_skinny(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
+                                       int(out_dtype == torch.float32), waves, _stream()))
     return out
 
 

@@ -7,16 +7,16 @@ from typing import Optional
 import torch
 
 from .. import ops
-from ..ops.functions import GEMM_SKINNY_MAX_M
+from ..ops.functions import GEMM_MFMA_SKINNY_MAX_M, GEMM_SKINNY_MAX_M
 
 
 class Linear:
     """Holds ``weight`` [N, K] in the compute dtype and an optional float32 ``bias`` [N].
 
     float32: the engine's own kernels only (true 32-bit products and sums).
-    bfloat16: the engine's skinny kernel for up to 8 rows; above that the library product
-    (hipBLASLt through torch, where the reference's engine calls cuBLAS) with float32
-    accumulation, the bias added by a kernel of the engine."""
+    bfloat16: up to 64 rows (decoding) the engine's matrix-core kernel that streams the weight
+    once; above that the library product (hipBLASLt through torch, where the reference's engine
+    calls cuBLAS) with float32 accumulation, the bias added by a kernel of the engine."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False):
         self.in_features = in_features
@@ -29,10 +29,13 @@ class Linear:
                  skip_bias: bool = False) -> torch.Tensor:
         bias = None if skip_bias else self.bias
         w = self.weight
-        if x.dtype == torch.float32 or x.shape[0] <= GEMM_SKINNY_MAX_M:
+        m = x.shape[0]
+        if x.dtype == torch.float32:
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
-        if out_dtype is not None and out_dtype != x.dtype:
-            # float32 result from bfloat16 operands (logits): the engine's tiled kernel
+        if m <= GEMM_MFMA_SKINNY_MAX_M and self.in_features % 8 == 0:
+            return ops.gemm_mfma_skinny(x, w, bias, out_dtype=out_dtype)
+        if m <= GEMM_SKINNY_MAX_M or (out_dtype is not None and out_dtype != x.dtype):
+            # odd inner sizes, and float32 results from bfloat16 operands (logits of many rows)
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
         y = torch.mm(x, w.t())
         if bias is not None:

@@ -1,0 +1,333 @@
+"""Each kernel alone against its plain reference, at other sizes than the tiny models'."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen2 as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def rnd(shape, seed, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def tol(dtype, ref, f32=1e-5, bf16=2.0 ** -7):
+    return f32 * max(1.0, ref.abs().max().item()) if dtype == torch.float32 else bf16 * ref.abs().max().item()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from from_scratch_inference_engine_amd import ops as o
+
+    o.load(build_if_missing=False)
+    return o
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(ops, dtype):
+    table = rnd((1000, 896), 0, dtype)
+    ids = torch.tensor([999, 0, 17, 17, 500], dtype=torch.int32)
+    out = ops.embedding(table.cuda(), ids.cuda()).cpu()
+    assert out.dtype == torch.float32 and torch.equal(out, plain.embedding(table.float(), ids.tolist()))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden, eps", [(896, 1e-6), (100, 1e-5), (4099, 0.5)])
+def test_rmsnorm_alone_fused_and_rows(ops, dtype, hidden, eps):
+    x, d, w = rnd((7, hidden), 1), rnd((7, hidden), 2, dtype), rnd((hidden,), 3) + 1.0
+    ref = plain.rms_norm(x, w, eps)
+    out = ops.rmsnorm(x.cuda(), w.cuda(), eps, dtype).float().cpu()
+    assert (out - ref).abs().max() <= tol(dtype, ref)
+    # fused with the residual sum: the stream is updated in float32, the norm sees the sum
+    res = x.clone().cuda()
+    out = ops.rmsnorm(res, w.cuda(), eps, dtype, delta=d.cuda(), write_back=True).float().cpu()
+    summed = x + d.float()
+    assert torch.equal(res.cpu(), summed)
+    ref = plain.rms_norm(summed, w, eps)
+    assert (out - ref).abs().max() <= tol(dtype, ref)
+    # chosen rows, pending delta not written back
+    rows = torch.tensor([6, 0, 3, 3], dtype=torch.int32)
+    res = x.clone().cuda()
+    out = ops.rmsnorm(res, w.cuda(), eps, dtype, delta=d.cuda(), rows=rows.cuda()).float().cpu()
+    assert torch.equal(res.cpu(), x) and (out - ref[rows.long()]).abs().max() <= tol(dtype, ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_and_adds(ops, dtype):
+    x = rnd((5, 2 * 4864), 4, dtype, 3.0)
+    ref = plain.silu_mul(x.float()[:, :4864], x.float()[:, 4864:])
+    out = ops.swiglu(x.cuda()).float().cpu()
+    assert (out - ref).abs().max() <= tol(dtype, ref)
+    res, d = rnd((3, 333), 5), rnd((3, 333), 6, dtype)
+    assert torch.equal(ops.residual_add(res.clone().cuda(), d.cuda()).cpu(), res + d.float())
+    y, b = rnd((4, 77), 7, dtype), rnd((77,), 8)
+    assert (ops.bias_add(y.clone().cuda(), b.cuda()).float().cpu() - (y.float() + b)).abs().max() <= tol(dtype, y.float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads, kv, hd, theta", [(14, 2, 64, 1e6), (3, 3, 48, 1e4), (5, 1, 256, 5e5)])
+def test_rope_and_cache_write(ops, dtype, heads, kv, hd, theta):
+    t, page, pages = 9, 4, 11
+    width = (heads + 2 * kv) * hd
+    qkv, bias = rnd((t, width), 9, dtype), rnd((width,), 10)
+    pos = torch.tensor([3, 4, 5, 0, 1, 4000, 17, 18, 19], dtype=torch.int32)
+    slots = torch.tensor([12, 13, 14, 40, 41, -1, 5, 6, 7], dtype=torch.int32)
+    inv = torch.tensor([theta ** (-2.0 * i / hd) for i in range(hd // 2)], dtype=torch.float64)
+    k_pool = torch.zeros((pages, kv, page, hd), dtype=dtype)
+    v_pool = torch.zeros_like(k_pool)
+    dq, dk, dv = qkv.clone().cuda(), k_pool.cuda(), v_pool.cuda()
+    ops.rope_kv_write(dq, pos.cuda(), heads, kv, hd, inv.cuda(), slots=slots.cuda(), k_pool=dk, v_pool=dv,
+                      page_size=page, bias=bias.cuda())
+    full = qkv.float() + bias
+    q_ref = plain.rope(full[:, :heads * hd], heads, hd, theta, pos.tolist())
+    k_ref = plain.rope(full[:, heads * hd:(heads + kv) * hd], kv, hd, theta, pos.tolist())
+    v_ref = full[:, (heads + kv) * hd:]
+    got = dq.float().cpu()
+    assert (got[:, :heads * hd] - q_ref).abs().max() <= tol(dtype, q_ref, f32=2e-6)
+    assert (got[:, heads * hd:(heads + kv) * hd] - k_ref).abs().max() <= tol(dtype, k_ref, f32=2e-6)
+    kp, vp = dk.float().cpu(), dv.float().cpu()
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for i, s in enumerate(slots.tolist()):
+        if s < 0:
+            continue
+        written[s] = True
+        assert (kp[s // page, :, s % page, :].reshape(-1) - k_ref[i]).abs().max() <= tol(dtype, k_ref, f32=2e-6)
+        assert (vp[s // page, :, s % page, :].reshape(-1) - v_ref[i]).abs().max() <= tol(dtype, v_ref, f32=2e-6)
+    untouched = ~written.reshape(pages, 1, page, 1).expand_as(kp)
+    assert kp[untouched].abs().max() == 0 and vp[untouched].abs().max() == 0
+    # no rotation, no cache: only the bias on q and k
+    dq = qkv.clone().cuda()
+    ops.rope_kv_write(dq, pos.cuda(), heads, kv, hd, None, bias=bias.cuda())
+    assert (dq.float().cpu()[:, :(heads + kv) * hd] - full[:, :(heads + kv) * hd]).abs().max() <= tol(dtype, full)
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 4864, 896), (5, 151, 100), (8, 1000, 4864), (37, 300, 129), (130, 896, 1000)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm(ops, dtype, m, n, k):
+    x, w, b = rnd((m, k), 11, dtype), rnd((n, k), 12, dtype, 0.05), rnd((n,), 13)
+    ref = plain.linear(x.float(), w.float(), b)
+    for kind in (1, 2) if m <= 8 else (1,):
+        out = ops.gemm(x.cuda(), w.cuda(), b.cuda(), kind=kind).float().cpu()
+        assert (out - ref).abs().max() <= tol(dtype, ref, f32=2e-6), f"kind {kind}"
+    out32 = ops.gemm(x.cuda(), w.cuda(), None, out_dtype=torch.float32).cpu()
+    assert out32.dtype == torch.float32 and (out32 - plain.linear(x.float(), w.float())).abs().max() <= 2e-5 * ref.abs().max() + 1e-6
+
+
+@pytest.mark.parametrize("m, n, k, waves", [(1, 4864, 896, 0), (8, 1000, 4864, 0), (16, 48, 64, 1), (17, 151, 104, 2),
+                                             (33, 896, 1000, 4), (64, 3584, 2048, 16), (50, 16, 8, 8), (7, 4608, 3584, 0)])
+def test_gemm_mfma_skinny(ops, m, n, k, waves):
+    x, w, b = rnd((m, k), 14, torch.bfloat16), rnd((n, k), 15, torch.bfloat16, 0.05), rnd((n,), 16)
+    ref = plain.linear(x.float(), w.float(), b)
+    out = ops.gemm_mfma_skinny(x.cuda(), w.cuda(), b.cuda(), out_dtype=torch.float32, waves=waves).cpu()
+    assert (out - ref).abs().max() <= 2e-5 * ref.abs().max()  # float32 sums of exact bfloat16 products
+    out = ops.gemm_mfma_skinny(x.cuda(), w.cuda(), None, waves=waves).float().cpu()
+    ref = plain.linear(x.float(), w.float())
+    assert (out - ref).abs().max() <= tol(torch.bfloat16, ref)
+
+
+def test_refusals(ops):
+    from from_scratch_inference_engine_amd.ops import KernelError
+
+    x, w = torch.zeros(65, 64, dtype=torch.bfloat16).cuda(), torch.zeros(32, 64, dtype=torch.bfloat16).cuda()
+    with pytest.raises(KernelError, match="at most 64 rows"):
+        ops.gemm_mfma_skinny(x, w)
+    with pytest.raises(KernelError, match="multiple of 8"):
+        ops.gemm_mfma_skinny(x[:4, :60].contiguous(), w[:, :60].contiguous())
+    with pytest.raises(KernelError, match="inner size"):
+        ops.gemm(x, w[:, :32].contiguous())
+    with pytest.raises(KernelError, match="contiguous"):
+        ops.gemm(x[:, ::2], w[:, ::2])
+    with pytest.raises(KernelError, match="GPU"):
+        ops.swiglu(torch.zeros(2, 4))
+    with pytest.raises(KernelError, match="float32 or bfloat16"):
+        ops.swiglu(torch.zeros(2, 4, dtype=torch.float16).cuda())
+    with pytest.raises(KernelError, match="head_dim"):
+        q = torch.zeros(1, 3 * 300).cuda()
+        ops.attention_scalar(q, 900, torch.zeros(1, 1, 4, 300).cuda(), torch.zeros(1, 1, 4, 300).cuda(),
+                             torch.zeros(1, 1, dtype=torch.int32).cuda(), torch.zeros(1, 8, dtype=torch.int32).cuda(), 1,
+                             torch.zeros(1, 300).cuda(), None, 1, 1, 300, None, 1.0, 1)
+
+
+# ------------------------------------------------------------------------------ attention
+def paged_case(seqs, heads, kv, hd, page, dtype, seed, window=None, shuffle=True, edit=None):
+    """seqs: list of (past, n_new).  Returns device inputs for the kernel and per-seq q/k/v.
+    ``edit(qs, ks, vs)`` may change the random tensors in place before the pages are filled."""
+    from from_scratch_inference_engine_amd.parts.attention import AttentionPlanner
+    from from_scratch_inference_engine_amd import ops
+
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-(p + n) // page) for p, n in seqs) + 3
+    order = (torch.randperm(total_pages, generator=torch.Generator().manual_seed(seed + 1)).tolist()
+             if shuffle else list(range(total_pages)))
+    k_pool = torch.full((total_pages, kv, page, hd), 7.0)  # stale content in unused slots
+    v_pool = torch.full((total_pages, kv, page, hd), -9.0)
+    max_pages = max(-(-(p + n) // page) for p, n in seqs)
+    tables = torch.full((len(seqs), max_pages), -1, dtype=torch.int32)
+    qs, ks, vs = [], [], []
+    for p, n in seqs:
+        qs.append(torch.randn(n, heads * hd, generator=g).to(dtype).float())
+        ks.append(torch.randn(p + n, kv * hd, generator=g).to(dtype).float())
+        vs.append(torch.randn(p + n, kv * hd, generator=g).to(dtype).float())
+    if edit is not None:
+        edit(qs, ks, vs)
+    for s, (p, n) in enumerate(seqs):
+        total = p + n
+        for i in range(-(-total // page)):
+            tables[s, i] = order.pop()
+        for j in range(total):
+            pg, off = tables[s, j // page].item(), j % page
+            k_pool[pg, :, off, :] = ks[s][j].reshape(kv, hd)
+            v_pool[pg, :, off, :] = vs[s][j].reshape(kv, hd)
+
+    class Host:
+        n_seqs = len(seqs)
+        q_lens = [n for _, n in seqs]
+        past_lens = [p for p, _ in seqs]
+        q_starts = [0]
+    for _, n in seqs:
+        Host.q_starts.append(Host.q_starts[-1] + n)
+    plan = AttentionPlanner(window, ops.attention_tile_tokens(heads, kv), 256).plan(Host)
+    return dict(q=torch.cat(qs).to(dtype), k_pool=k_pool.to(dtype), v_pool=v_pool.to(dtype), tables=tables, plan=plan,
+                qs=qs, ks=ks, vs=vs)
+
+
+def run_attention(ops, case, heads, kv, hd, window=None):
+    q = case["q"].cuda()
+    t = q.shape[0]
+    plan = case["plan"]
+    out = torch.zeros((t, heads * hd), dtype=q.dtype).cuda()
+    partials = torch.empty(max(plan["n_partial"], 1) * heads * (hd + 2), dtype=torch.float32).cuda()
+    items = torch.from_numpy(plan["items"]).cuda()
+    ops.attention_scalar(q, heads * hd, case["k_pool"].cuda(), case["v_pool"].cuda(), case["tables"].cuda(), items,
+                         plan["n_items"], out, partials, heads, kv, hd, window, 1.0 / math.sqrt(hd), t)
+    if plan["n_merges"]:
+        ops.attention_merge(partials, torch.from_numpy(plan["merges"]).cuda(), plan["n_merges"], out, heads, hd)
+    return out.float().cpu()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads, kv, hd, page, window", [
+    (14, 2, 64, 16, None),   # the reference's kernel test sizes (tests/cpp/test_cuda_kernels.cpp:126-164)
+    (4, 4, 48, 4, None),     # plain multi-head, head size no power of two
+    (20, 1, 32, 8, None),    # more heads per kv head than rows of a block
+    (6, 2, 128, 16, 37),     # a window
+    (3, 1, 256, 64, None),
+])
+def test_attention_over_pages(ops, dtype, heads, kv, hd, page, window):
+    # (past, new): the reference's (7, 5) and (19, 1), a long decode that is split, whole prompts,
+    # portions starting mid-page, a two-token portion
+    seqs = [(7, 5), (19, 1), (600, 1), (0, 33), (300, 2), (123, 70), (0, 1)]
+    case = paged_case(seqs, heads, kv, hd, page, dtype, seed=hd + heads, window=window)
+    out = run_attention(ops, case, heads, kv, hd, window)
+    row = 0
+    for (p, n), q, k, v in zip(seqs, case["qs"], case["ks"], case["vs"]):
+        ref = plain.attention(q, k, v, heads, kv, hd, query_offset=p, window=window)
+        err = (out[row:row + n] - ref).abs().max().item()
+        assert err <= (2e-6 if dtype == torch.float32 else 2.0 ** -7 * ref.abs().max().item()), f"seq past {p} new {n}: {err}"
+        row += n
+
+
+def test_attention_finds_one_far_key_and_respects_edges(ops):
+    """Inputs that random data would hide a fault behind: for every query one key far back (or
+    at the far edge of its window) carries nearly the whole softmax, so the output must be that
+    key's value; and louder keys sit where the query must not look: right after its own
+    position and right before its window."""
+    heads, kv, hd, page = 4, 2, 32, 8
+    group = heads // kv
+    for window in (None, 100):
+        seqs = [(700, 1), (350, 3)]
+        chosen = {}
+
+        def edit(qs, ks, vs):
+            for s, (p, n) in enumerate(seqs):
+                for i in range(n):
+                    pos = p + i
+                    far = pos - window + 1 if window else 3 + 8 * i   # the window's first key / hundreds back
+                    chosen[(s, i)] = far
+                    q = qs[s][i].reshape(heads, hd)
+                    for kvh in range(kv):
+                        # the heads of one group share the key: point all of them at it
+                        q[kvh * group:(kvh + 1) * group] = q[kvh * group] * 1.0
+                        u = q[kvh * group] / q[kvh * group].norm()
+                        ks[s][far].reshape(kv, hd)[kvh] = 40.0 * u
+                        q[kvh * group:(kvh + 1) * group] = 8.0 * u
+                        loud = 400.0 * u
+                        if pos + 1 < p + n:
+                            ks[s][pos + 1].reshape(kv, hd)[kvh] = loud       # the future
+                        if window and pos - window >= 0 and pos - window not in chosen.values():
+                            ks[s][pos - window].reshape(kv, hd)[kvh] = loud  # just outside the window
+
+        case = paged_case(seqs, heads, kv, hd, page, torch.float32, seed=3, window=window, edit=edit)
+        out = run_attention(ops, case, heads, kv, hd, window)
+        row = 0
+        for s, ((p, n), q, k, v) in enumerate(zip(seqs, case["qs"], case["ks"], case["vs"])):
+            ref = plain.attention(q, k, v, heads, kv, hd, query_offset=p, window=window)
+            assert (out[row:row + n] - ref).abs().max() <= 5e-6
+            for i in range(n):  # and the plain result is what the construction says: the far key's value
+                want = v[chosen[(s, i)]].reshape(kv, 1, hd).expand(kv, group, hd).reshape(-1)
+                if i == 0:
+                    assert (ref[i] - want).abs().max() < 1e-3
+            row += n
+
+
+def test_attention_does_not_depend_on_page_ids(ops):
+    heads, kv, hd, page = 8, 2, 64, 16
+    seqs = [(100, 1), (0, 40)]
+    a = run_attention(ops, paged_case(seqs, heads, kv, hd, page, torch.float32, 5, shuffle=True), heads, kv, hd)
+    b = run_attention(ops, paged_case(seqs, heads, kv, hd, page, torch.float32, 5, shuffle=False), heads, kv, hd)
+    assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------------------ sampling
+def test_argmax_ties_and_large_vocab(ops):
+    # tests/cpp/test_cuda_kernels.cpp:201-235: V = 151936 rows equal a host scan; ties -> smallest index
+    logits = rnd((5, 151936), 20)
+    logits[1, 77] = logits[1, 140000] = 50.0
+    logits[2, 151935] = 60.0
+    logits[3, 0] = 60.0
+    out = ops.sample(logits.cuda()).cpu().tolist()
+    assert out == [plain.argmax(r) for r in logits] and out[1] == 77 and out[2] == 151935 and out[3] == 0
+    small = torch.tensor([[0.0, 1.0, 5.0, 1.0, 0.0, 5.0]])
+    assert ops.sample(small.cuda()).item() == 2
+
+
+@pytest.mark.parametrize("vocab", [509, 151936])
+def test_sampling_matches_plain_given_u(ops, vocab):
+    g = torch.Generator().manual_seed(21)
+    rows = []
+    for temp, k, p in [(0.7, 0, 1.0), (1.0, 0, 1.0), (0.3, 5, 1.0), (1.5, 50, 0.9), (1.0, 0, 0.5), (2.0, 1, 1.0),
+                       (0.0, 0, 1.0), (0.9, 3, 0.2)]:
+        for u in (0.0, 0.013, 0.37, 0.5, 0.81, 0.999):
+            rows.append((temp, k, p, u))
+    logits = torch.randn(len(rows), vocab, generator=g) * 2.0
+    logits[3, 10] = logits[3, 11] = logits[3].max() + 1.0  # a tie at the top
+    dev = lambda v, dt: torch.tensor(v, dtype=dt).cuda()
+    out = ops.sample(logits.cuda(), dev([r[0] for r in rows], torch.float32), dev([r[1] for r in rows], torch.int32),
+                     dev([r[2] for r in rows], torch.float32), dev([r[3] for r in rows], torch.float64)).cpu().tolist()
+    bad = []
+    for i, (temp, k, p, u) in enumerate(rows):
+        want = plain.sample(logits[i], temp, k, p, u)
+        if out[i] != want:
+            # tolerate a draw that sits on a boundary of the cumulative sum within float rounding
+            alt = {plain.sample(logits[i], temp, k, p, min(max(u + d, 0.0), 0.999999)) for d in (-1e-6, 1e-6)}
+            if out[i] not in alt:
+                bad.append((i, rows[i], out[i], want))
+    assert not bad, bad
+
+
+def test_sampling_distribution(ops):
+    # tests/cpp/test_sampler.cpp:44-56: logits {0, 2, 0} pick index 1 with probability 0.787
+    n = 4000
+    logits = torch.tensor([[0.0, 2.0, 0.0]]).repeat(n, 1).cuda()
+    u = ((torch.arange(n, dtype=torch.float64) + 0.5) / n).cuda()
+    ones = torch.ones(n, dtype=torch.float32).cuda()
+    out = ops.sample(logits, ones, torch.zeros(n, dtype=torch.int32).cuda(), ones, u).cpu()
+    assert abs((out == 1).float().mean().item() - 0.7869) < 0.002
+    assert (out[:400] == 0).all() and (out[-400:] == 2).all()  # vocabulary order of the draw
