@@ -31,7 +31,8 @@ class CacheLayout:
 class LayerCache:
     """What a mixer sees of the cache in one step.
 
-    Paged: ``k_pool``/``v_pool`` [pages, kv_heads, page_size, head_dim] of this layer,
+    Paged: ``k_pool`` [pages, kv_heads, page_size, head_dim] and ``v_pool`` [pages, kv_heads,
+    head_dim, page_size] of this layer,
     ``block_tables`` int32 [requests in the step, pages] (-1 = no page), ``slots`` int32 [tokens]
     (where each token's entry goes), ``page_size``, and ``writes`` (False when this call only
     reads a cache that another call fills).
@@ -52,18 +53,24 @@ class CacheStorage:
         self.page_size = manager.page_size
         self.device = device
         self.dtype = dtype
-        self.pools: List[torch.Tensor] = []
+        # per group: keys [caches, pages, kv_heads, page_size, head_dim] and values, transposed
+        # within a page, [caches, pages, kv_heads, head_dim, page_size]
+        self.k_pools: List[torch.Tensor] = []
+        self.v_pools: List[torch.Tensor] = []
         for g, need in enumerate(layout.paged_groups):
             n_pages = manager.allocators[g].num_pages
-            shape = (len(layout.group_caches[g]), 2, n_pages, need.n_kv_heads, self.page_size, need.head_dim)
-            self.pools.append(torch.zeros(shape, dtype=dtype, device=device))
+            n_caches = len(layout.group_caches[g])
+            self.k_pools.append(torch.zeros((n_caches, n_pages, need.n_kv_heads, self.page_size, need.head_dim),
+                                            dtype=dtype, device=device))
+            self.v_pools.append(torch.zeros((n_caches, n_pages, need.n_kv_heads, need.head_dim, self.page_size),
+                                            dtype=dtype, device=device))
         self.states: Dict[int, torch.Tensor] = {}
         for cid, need in layout.state_caches.items():
             self.states[cid] = torch.zeros((manager.max_requests, *need.shape),
                                            dtype=getattr(torch, need.dtype), device=device)
 
     def bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in list(self.pools) + list(self.states.values()))
+        return sum(t.numel() * t.element_size() for t in self.k_pools + self.v_pools + list(self.states.values()))
 
     def reset_states(self, slots: Sequence[int]) -> None:
         """Zero the state slots of requests that start in this step."""
@@ -80,8 +87,7 @@ class CacheStorage:
             lc.state = self.states[cache_id]
             return lc
         g, plane = self.layout.locate(cache_id)
-        pool = self.pools[g]
-        lc.k_pool, lc.v_pool = pool[plane, 0], pool[plane, 1]
+        lc.k_pool, lc.v_pool = self.k_pools[g][plane], self.v_pools[g][plane]
         lc.block_tables = ctx.block_tables[g]
         lc.slots = ctx.slots[g]
         lc.page_size = self.page_size

@@ -1,0 +1,40 @@
+// Entry point of the matrix-core attention (bfloat16): picks the instantiation for the head size.
+#include "attention_mfma_impl.h"
+
+namespace fsie_attn {
+LaunchFn table_a(int hdt, int large);
+LaunchFn table_b(int hdt, int large);
+LaunchFn table_c(int hdt, int large);
+LaunchFn table_d(int hdt, int large);
+}  // namespace fsie_attn
+
+// Query tiles of 16 rows that one wave of the `large` variant holds for this head size.
+extern "C" int fsie_attention_mfma_tiles(int head_dim, int large) {
+    if (head_dim <= 0 || head_dim % 16 || head_dim > 256) return 0;
+    if (!large) return 1;
+    return head_dim <= 128 ? 4 : 2;
+}
+
+// bfloat16 only; head_dim a multiple of 16 up to 256; page_size a multiple of 4.
+// large = 0: items of at most 16 rows (tokens x heads of a group); large = 1: up to 16 * tiles rows.
+extern "C" int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                                   const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
+                                   void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,
+                                   int window, float scale, int large, hipStream_t stream) {
+    FSIE_REQUIRE(n_items >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0,
+                 "attention_mfma: heads %d must be a positive multiple of kv heads %d", n_heads, n_kv);
+    FSIE_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= 256,
+                 "attention_mfma: head_dim %d must be a multiple of 16 up to 256", head_dim);
+    FSIE_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_mfma: page_size %d must be a multiple of 4", page_size);
+    FSIE_REQUIRE(max_pages > 0, "attention_mfma: empty block table");
+    FSIE_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0,
+                 "attention_mfma: query rows must be 16-byte aligned");
+    if (n_items == 0) return 0;
+    const int hdt = head_dim / 16;
+    fsie_attn::LaunchFn fn = hdt <= 4 ? fsie_attn::table_a(hdt, large)
+                           : hdt <= 8 ? fsie_attn::table_b(hdt, large)
+                           : hdt <= 12 ? fsie_attn::table_c(hdt, large) : fsie_attn::table_d(hdt, large);
+    FSIE_REQUIRE(fn != nullptr, "attention_mfma: no kernel for head_dim %d", head_dim);
+    return fn(q, q_stride, k_pool, v_pool, block_tables, max_pages, items, n_items, out, partials, n_heads, n_kv,
+              page_size, window, scale, stream);
+}

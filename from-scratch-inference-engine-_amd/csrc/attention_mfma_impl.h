@@ -1,0 +1,268 @@
+// Causal grouped-query attention over the pages of the cache on the matrix cores (bfloat16).
+//
+// One wave per work item and kv head (chunk).  Everything is computed transposed so that no
+// operand ever has to change lanes or pass through LDS:
+//
+//   S^T[key, row] = K[key, :] . Q[row, :]      A = K rows from the cache (16 B per lane),
+//                                              B = Q rows, kept in registers for the whole item
+//   softmax over the keys of a column: 4 keys per lane, the rest by two xor shuffles (16, 32)
+//   O^T[d, row]  += V^T[d, key] . P^T[key, row] A = V^T from the cache, which stores values
+//                                              transposed ([head_dim][slot]: 4 consecutive keys of
+//                                              one dimension are one 8-byte load),
+//                                              B = P^T, which is exactly the layout in which the
+//                                              first product left S^T
+//
+// The running maximum and sum of a query row and its accumulators live in the same lanes
+// (column = lane % 16), so the online-softmax rescale is lane-local.  Scores use
+// v_mfma_f32_16x16x32_bf16 over the head dimension (16x16x16 steps when head_dim is an odd
+// multiple of 16); the second product uses 16x16x16 over 16 keys.
+//
+// HDT = head_dim / 16, NT = column tiles of 16 query rows per wave (rows = tokens x heads of the
+// kv head's group).  Keys are walked in blocks of 32.  Requires page_size % 4 == 0.
+#pragma once
+
+#include "common.h"
+#include "api.h"
+
+#include <math.h>
+
+namespace fsie_attn {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+union F16B {
+    uint4 raw;
+    bf16x8 v;
+};
+union F8B {
+    uint2 raw;
+    shortx4 v;
+};
+
+__device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ uint2 ld8(const bf16_t* p) { return *reinterpret_cast<const uint2*>(p); }
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+template <int HDT, int NT>
+__global__ __launch_bounds__(64) void attention_mfma_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
+    const int32_t* __restrict__ items, bf16_t* __restrict__ out, float* __restrict__ partials, int n_heads,
+    int n_kv, int page_size, int window, float scale, int gh, int head_chunks) {
+    constexpr int HD = HDT * 16;
+    // scores: 32-wide steps over the head dimension when head_dim is a multiple of 32, else
+    // 16-wide steps throughout (the two shapes are never chained on one accumulator)
+    constexpr bool X32 = (HDT % 2) == 0;
+    constexpr int S32 = X32 ? HDT / 2 : 0;
+    constexpr int S16 = X32 ? 0 : HDT;
+    constexpr int S32A = S32 > 0 ? S32 : 1;
+    constexpr int S16A = S16 > 0 ? S16 : 1;
+
+    const int32_t* item = items + static_cast<int64_t>(blockIdx.x) * FSIE_ATTN_ITEM_INTS;
+    const int seq = item[FSIE_ATTN_ITEM_SEQ];
+    const int q_row0 = item[FSIE_ATTN_ITEM_QROW];
+    const int n_q = item[FSIE_ATTN_ITEM_NQ];
+    const int pos0 = item[FSIE_ATTN_ITEM_POS];
+    const int key_begin = item[FSIE_ATTN_ITEM_KBEGIN];
+    const int key_end = item[FSIE_ATTN_ITEM_KEND];
+    const int partial_base = item[FSIE_ATTN_ITEM_PARTIAL];
+    if (n_q <= 0) return;  // padding item
+
+    const int group = n_heads / n_kv;
+    const int kvh = blockIdx.y / head_chunks;
+    const int chunk = blockIdx.y - kvh * head_chunks;
+    const int gh_here = min(gh, group - chunk * gh);
+    const int h_base = kvh * group + chunk * gh;
+    const int n_rows = n_q * gh;
+
+    const int lane = threadIdx.x;
+    const int c = lane & 15;  // column of S^T and O^T (query row of a tile); row of the A tiles
+    const int G = lane >> 4;  // lane group: which 4 (or 8) of the reduction indices this lane holds
+    const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
+    const float scale2 = scale * kLog2e;  // scores in units of log2 e: exp() becomes exp2()
+
+    // ---- the item's queries: B operands, kept for the whole item
+    bool rvalid[NT];
+    int rpos[NT], rtok[NT], rhead[NT];
+    F16B qf[NT][S32A];
+    F8B qt[NT][S16A];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const int rg = nt * 16 + c;
+        const int tq = rg / gh, hh = rg - tq * gh;
+        rvalid[nt] = rg < n_rows && hh < gh_here;
+        rtok[nt] = tq;
+        rhead[nt] = h_base + hh;
+        rpos[nt] = pos0 + tq;
+        const bf16_t* qp = q + static_cast<int64_t>(q_row0 + (rvalid[nt] ? tq : 0)) * q_stride +
+                           static_cast<int64_t>(rvalid[nt] ? rhead[nt] : h_base) * HD;
+#pragma unroll
+        for (int s = 0; s < S32; ++s) qf[nt][s].raw = rvalid[nt] ? ld16(qp + s * 32 + 8 * G) : uint4{0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < S16; ++s) qt[nt][s].raw = rvalid[nt] ? ld8(qp + s * 16 + 4 * G) : uint2{0, 0};
+    }
+
+    float m_run[NT], l_run[NT];
+    floatx4 acc[NT][HDT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        m_run[nt] = -INFINITY;
+        l_run[nt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < HDT; ++dt) acc[nt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int64_t head_stride = static_cast<int64_t>(page_size) * HD;  // one kv head of one page
+    for (int kb = key_begin & ~31; kb < key_end; kb += 32) {
+        // ---- keys (A operand of the scores) and values (A operand of the second product)
+        F16B kf[2][S32A];
+        F8B kt[2][S16A];
+        F8B vf[2][HDT];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int key = kb + t * 16 + c;
+            const int idx = key / page_size;
+            const int page = (key < key_end && idx < max_pages) ? table[idx] : -1;
+            const bool ok = page >= 0;
+            const bf16_t* kp = k_pool + (static_cast<int64_t>(ok ? page : 0) * n_kv + kvh) * head_stride +
+                               static_cast<int64_t>(key - idx * page_size) * HD;
+#pragma unroll
+            for (int s = 0; s < S32; ++s) kf[t][s].raw = ok ? ld16(kp + s * 32 + 8 * G) : uint4{0, 0, 0, 0};
+#pragma unroll
+            for (int s = 0; s < S16; ++s) kt[t][s].raw = ok ? ld8(kp + s * 16 + 4 * G) : uint2{0, 0};
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int key0 = kb + t * 16 + 4 * G;  // 4 consecutive keys, never across a page (page_size % 4 == 0)
+            const int idx = key0 / page_size;
+            const int page = (key0 < key_end && idx < max_pages) ? table[idx] : -1;
+            const bool ok = page >= 0;
+            const bf16_t* vp = v_pool + (static_cast<int64_t>(ok ? page : 0) * n_kv + kvh) * head_stride +
+                               (key0 - idx * page_size);
+#pragma unroll
+            for (int dt = 0; dt < HDT; ++dt) {
+                vf[t][dt].raw = ok ? ld8(vp + static_cast<int64_t>(dt * 16 + c) * page_size) : uint2{0, 0};
+            }
+        }
+
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            // ---- S^T for 32 keys x 16 rows
+            floatx4 st[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < S32; ++s)
+                    st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][s].v, qf[nt][s].v, st[t], 0, 0, 0);
+#pragma unroll
+                for (int s = 0; s < S16; ++s)
+                    st[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kt[t][s].v, qt[nt][s].v, st[t], 0, 0, 0);
+            }
+            // ---- mask, running maximum
+            float sv[8];
+            float m_loc = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = kb + t * 16 + 4 * G + r;
+                    const bool vis = rvalid[nt] && key >= key_begin && key < key_end && key <= rpos[nt] &&
+                                     (window <= 0 || key > rpos[nt] - window);
+                    sv[t * 4 + r] = vis ? st[t][r] * scale2 : -INFINITY;
+                    m_loc = fmaxf(m_loc, sv[t * 4 + r]);
+                }
+            m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16, FSIE_WAVE));
+            m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32, FSIE_WAVE));
+            const float m_new = fmaxf(m_run[nt], m_loc);
+            const float corr = (m_run[nt] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[nt] - m_new);
+            float p[8];
+            float p_sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                p[i] = (sv[i] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sv[i] - m_new);
+                p_sum += p[i];
+            }
+            l_run[nt] = l_run[nt] * corr + p_sum;  // this lane's keys only; lane groups are summed at the end
+            m_run[nt] = m_new;
+            F8B pb[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                pb[t].raw.x = static_cast<uint32_t>(float_to_bf16_bits(p[t * 4 + 0])) |
+                              (static_cast<uint32_t>(float_to_bf16_bits(p[t * 4 + 1])) << 16);
+                pb[t].raw.y = static_cast<uint32_t>(float_to_bf16_bits(p[t * 4 + 2])) |
+                              (static_cast<uint32_t>(float_to_bf16_bits(p[t * 4 + 3])) << 16);
+            }
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int dt = 0; dt < HDT; ++dt) {
+                floatx4 a = acc[nt][dt];
+                a[0] *= corr;
+                a[1] *= corr;
+                a[2] *= corr;
+                a[3] *= corr;
+                a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[0][dt].v, pb[0].v, a, 0, 0, 0);
+                a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[1][dt].v, pb[1].v, a, 0, 0, 0);
+                acc[nt][dt] = a;
+            }
+        }
+    }
+
+    // ---- results: lane holds O^T[d = 16 dt + 4 G + r][row c]
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        float l_tot = l_run[nt];
+        l_tot += __shfl_xor(l_tot, 16, FSIE_WAVE);
+        l_tot += __shfl_xor(l_tot, 32, FSIE_WAVE);
+        if (!rvalid[nt]) continue;
+        if (partial_base < 0) {
+            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+            bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[nt]) * n_heads + rhead[nt]) * HD + 4 * G;
+#pragma unroll
+            for (int dt = 0; dt < HDT; ++dt) {
+                uint2 w;
+                w.x = static_cast<uint32_t>(float_to_bf16_bits(acc[nt][dt][0] * inv)) |
+                      (static_cast<uint32_t>(float_to_bf16_bits(acc[nt][dt][1] * inv)) << 16);
+                w.y = static_cast<uint32_t>(float_to_bf16_bits(acc[nt][dt][2] * inv)) |
+                      (static_cast<uint32_t>(float_to_bf16_bits(acc[nt][dt][3] * inv)) << 16);
+                *reinterpret_cast<uint2*>(o + dt * 16) = w;
+            }
+        } else {
+            float* rec = partials + (static_cast<int64_t>(partial_base + rtok[nt]) * n_heads + rhead[nt]) * (HD + 2);
+#pragma unroll
+            for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) rec[dt * 16 + 4 * G + r] = acc[nt][dt][r];
+            if (G == 0) {
+                rec[HD] = m_run[nt] * kLn2;  // back to natural units for the merge
+                rec[HD + 1] = l_tot;
+            }
+        }
+    }
+}
+
+template <int HDT, int NT>
+int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+           int max_pages, const int32_t* items, int n_items, void* out, float* partials, int n_heads, int n_kv,
+           int page_size, int window, float scale, hipStream_t stream) {
+    const int group = n_heads / n_kv;
+    const int rows = 16 * NT;
+    const int gh = group < rows ? group : rows;
+    const int head_chunks = (group + gh - 1) / gh;
+    const dim3 grid(n_items, n_kv * head_chunks);
+    attention_mfma_kernel<HDT, NT><<<grid, 64, 0, stream>>>(
+        static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
+        block_tables, max_pages, items, static_cast<bf16_t*>(out), partials, n_heads, n_kv, page_size, window, scale,
+        gh, head_chunks);
+    FSIE_CHECK_LAUNCH("attention_mfma");
+    return 0;
+}
+
+typedef int (*LaunchFn)(const void*, int64_t, const void*, const void*, const int32_t*, int, const int32_t*, int, void*,
+                        float*, int, int, int, int, float, hipStream_t);
+
+}  // namespace fsie_attn

@@ -8,7 +8,7 @@
 // when a key range was split over several items.  grid = (items, kv_heads * head_chunks); a block
 // holds rows = tokens x heads of one kv head's group (gh heads per chunk), four rows per wave.
 //
-// Page layout: [page][kv_head][slot][head_dim]; block_tables[seq * max_pages + i] = page id of the
+// Page layout: keys [page][kv_head][slot][head_dim], values [page][kv_head][head_dim][slot]; block_tables[seq * max_pages + i] = page id of the
 // request's i-th page, or -1 where a window has passed.
 #include "common.h"
 #include "api.h"
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
             if (kj < key_end) {
                 const int page = table[kj / page_size];
                 if (page >= 0) {
-                    v = to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + kj % page_size) * hd + d]);
+                    v = to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + kj % page_size]);
                 }
             }
             kv[j * kv_stride + d] = v;

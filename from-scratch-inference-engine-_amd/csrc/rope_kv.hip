@@ -2,7 +2,9 @@
 // and v into the pages of the cache.  One block per token.  The v columns of the row itself are
 // left without the bias: only the cache is read afterwards.
 //
-// Page layout (keys and values alike): [page][kv_head][slot in page][head_dim].
+// Page layout: keys [page][kv_head][slot in page][head_dim]; values transposed,
+// [page][kv_head][head_dim][slot in page], so that the matrix-core attention kernel reads
+// consecutive keys of one dimension with one load.
 #include "common.h"
 #include "api.h"
 
@@ -72,9 +74,10 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
     for (int idx = threadIdx.x; idx < kv_dim; idx += blockDim.x) {
         const int kvh = idx / head_dim;
         const int d = idx - kvh * head_dim;
-        const int64_t dst = ((page * n_kv + kvh) * page_size + off) * head_dim + d;
-        k_pool[dst] = k[idx];
-        v_pool[dst] = bias ? from_float<T>(to_float(v[idx]) + bias[q_dim + kv_dim + idx]) : v[idx];
+        const int64_t head = (page * n_kv + kvh) * page_size * head_dim;
+        k_pool[head + static_cast<int64_t>(off) * head_dim + d] = k[idx];
+        v_pool[head + static_cast<int64_t>(d) * page_size + off] =
+            bias ? from_float<T>(to_float(v[idx]) + bias[q_dim + kv_dim + idx]) : v[idx];
     }
 }
 

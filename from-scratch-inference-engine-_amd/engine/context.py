@@ -29,7 +29,9 @@ class StepEntry:
 class HostBatch:
     """Host view of the step, in the order of the entries."""
 
-    def __init__(self, entries: Sequence[StepEntry]):
+    def __init__(self, entries: Sequence[StepEntry], page_size: int = 0, compute_dtype=None):
+        self.page_size = page_size
+        self.compute_dtype = compute_dtype
         self.n_seqs = len(entries)
         self.q_lens = [len(e.tokens) for e in entries]
         self.past_lens = [e.cache.length for e in entries]
@@ -127,7 +129,7 @@ class StepContext:
 def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners: Sequence, staging: PinnedStaging,
                   compute_dtype: torch.dtype, device) -> StepContext:
     """Tables of one step.  The entries' pages must have been reserved already."""
-    host = HostBatch(entries)
+    host = HostBatch(entries, manager.page_size, compute_dtype)
     ctx = StepContext(host, compute_dtype, device)
     pk = _Packer()
     i_ids = pk.add(host.token_ids.astype(np.int32))

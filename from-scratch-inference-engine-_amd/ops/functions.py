@@ -117,8 +117,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
                   page_size: int = 0, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rotate the q and k heads of ``qkv`` [T, (n_heads + 2 n_kv) head_dim] in place by the angles
     ``positions * inv_freq`` (float64 table of rotary_dim/2 entries; ``None`` = no rotation) and
-    copy k and v to the cache slots ``slots`` (int32 [T], negative = not stored) of pools laid out
-    [pages, n_kv, page_size, head_dim]."""
+    copy k and v to the cache slots ``slots`` (int32 [T], negative = not stored) of the pools: keys
+    [pages, n_kv, page_size, head_dim], values [pages, n_kv, head_dim, page_size]."""
     _need(qkv, "qkv", ndim=2)
     t = qkv.shape[0]
     if qkv.shape[1] != (n_heads + 2 * n_kv) * head_dim:
@@ -136,7 +136,7 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
             raise KernelError("rope_kv_write: k_pool needs v_pool and slots")
         _need(slots, "slots", dtype=torch.int32, shape=(t,))
         _need(k_pool, "k_pool", dtype=qkv.dtype, ndim=4)
-        _need(v_pool, "v_pool", dtype=qkv.dtype, shape=k_pool.shape)
+        _need(v_pool, "v_pool", dtype=qkv.dtype, shape=(k_pool.shape[0], n_kv, head_dim, page_size))
         if tuple(k_pool.shape[1:]) != (n_kv, page_size, head_dim):
             raise KernelError(f"k_pool: shape {tuple(k_pool.shape)} is not [pages, {n_kv}, {page_size}, {head_dim}]")
         pool_slots = k_pool.shape[0] * page_size
@@ -210,7 +210,7 @@ def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_poo
     if not q.is_cuda:
         raise KernelError("attention q: must be on the GPU")
     _need(k_pool, "k_pool", dtype=q.dtype, ndim=4)
-    _need(v_pool, "v_pool", dtype=q.dtype, shape=k_pool.shape)
+    _need(v_pool, "v_pool", dtype=q.dtype, shape=(k_pool.shape[0], k_pool.shape[1], k_pool.shape[3], k_pool.shape[2]))
     _need(block_tables, "block_tables", dtype=torch.int32, ndim=2)
     _need(items, "attention items", dtype=torch.int32, ndim=2)
     if items.shape[1] != ATTN_ITEM_INTS or items.shape[0] < n_items:
@@ -227,6 +227,41 @@ def attention_scalar(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_poo
                                        block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(),
                                        n_items, out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim,
                                        page_size, int(window or 0), float(scale), dtype_code(q.dtype), _stream()))
+    return out
+
+
+def attention_mfma_rows(head_dim: int, large: bool) -> int:
+    """Query rows (tokens x heads of a kv head's group) that one work item of the matrix-core
+    attention holds; 0 if the head size is not offered."""
+    return 16 * load().fsie_attention_mfma_tiles(head_dim, int(large))
+
+
+def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                   block_tables: torch.Tensor, items: torch.Tensor, n_items: int, out: torch.Tensor,
+                   partials: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
+                   window: Optional[int], scale: float, n_query_rows: int, large: bool) -> torch.Tensor:
+    """Attention of the work items over the paged cache on the matrix cores (bfloat16; head_dim a
+    multiple of 16; page size a multiple of 4).  ``items`` may be a view into a longer table."""
+    if not q.is_cuda or q.dtype != torch.bfloat16:
+        raise KernelError("attention_mfma q: must be bfloat16 on the GPU")
+    _need(k_pool, "k_pool", dtype=q.dtype, ndim=4)
+    _need(v_pool, "v_pool", dtype=q.dtype, shape=(k_pool.shape[0], k_pool.shape[1], k_pool.shape[3], k_pool.shape[2]))
+    _need(block_tables, "block_tables", dtype=torch.int32, ndim=2)
+    _need(items, "attention items", dtype=torch.int32, ndim=2)
+    if items.shape[1] != ATTN_ITEM_INTS or items.shape[0] < n_items:
+        raise KernelError(f"attention items: shape {tuple(items.shape)} does not hold {n_items} items")
+    _need(out, "attention out", dtype=q.dtype, shape=(n_query_rows, n_heads * head_dim))
+    pages, kvh, page_size, hd = k_pool.shape
+    if kvh != n_kv or hd != head_dim:
+        raise KernelError(f"k_pool: shape {tuple(k_pool.shape)} does not match kv heads {n_kv}, head_dim {head_dim}")
+    if q_stride < n_heads * head_dim:
+        raise KernelError("attention: q_stride is smaller than the query width")
+    if partials is not None:
+        _need(partials, "attention partials", dtype=torch.float32, ndim=1)
+    check(load().fsie_attention_mfma(q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+                                     block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(), n_items,
+                                     out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim, page_size,
+                                     int(window or 0), float(scale), int(large), _stream()))
     return out
 
 

@@ -17,49 +17,75 @@ from .rope import KVStore
 
 
 class AttentionPlanner:
-    """Cuts a step into the work items of the attention kernel (host side, once per step for all
+    """Cuts a step into the work items of the attention kernels (host side, once per step for all
     layers with the same geometry).
 
-    A request's portion of n tokens at past length p becomes tiles of ``tile_tokens`` query
-    tokens; a tile reads the keys from the start of its window to its last token.  A portion
-    that fits one tile and reads more than ``split_keys`` keys (decoding against a long
-    context) is split over the keys instead, ``split_keys`` per item, and merged afterwards in
-    the order of the splits.  Whether a portion is split depends on the portion alone, never
-    on what else is in the batch.
-    """
+    A request's portion of n tokens at past length p becomes tiles of query tokens; a tile reads
+    the keys from the start of its window to its last token.  A portion of at most
+    ``small_tokens`` tokens is one *small* item; if it reads more than ``split_keys`` keys
+    (decoding against a long context) it is split over the keys instead, ``split_keys`` per
+    item, and merged afterwards in the order of the splits.  Longer portions are cut into *large*
+    tiles of ``large_tokens``.  Whether and how a portion is cut depends on the portion alone,
+    never on what else is in the batch.  The item table lists the small items first.
 
-    def __init__(self, window: Optional[int], tile_tokens: int, split_keys: int):
-        self.window = window
-        self.tile_tokens = tile_tokens
-        self.split_keys = split_keys
-        self.key = ("attention", window, tile_tokens, split_keys)
+    Two geometries exist: the matrix-core kernel (bfloat16, head size a multiple of 16, page size
+    a multiple of 4) and the float32-arithmetic kernel for everything else; which one a step
+    uses follows from the step's dtype and page size."""
+
+    def __init__(self, n_heads: int, n_kv: int, head_dim: int, window: Optional[int]):
+        self.n_heads, self.n_kv, self.head_dim, self.window = n_heads, n_kv, head_dim, window
+        self.key = ("attention", n_heads, n_kv, head_dim, window)
+        self._geometry = {}
+
+    def geometry(self, mfma: bool):
+        """(small_tokens, large_tokens, split_keys) of a kernel family."""
+        if mfma not in self._geometry:
+            group = self.n_heads // self.n_kv
+            if mfma:
+                small = max(1, ops.attention_mfma_rows(self.head_dim, False) // min(group, 16))
+                rows = ops.attention_mfma_rows(self.head_dim, True)
+                large = max(1, rows // min(group, rows))
+                self._geometry[mfma] = (small, large, 128)
+            else:
+                t = ops.attention_tile_tokens(self.n_heads, self.n_kv)
+                self._geometry[mfma] = (t, t, 256)
+        return self._geometry[mfma]
+
+    def uses_mfma(self, compute_dtype, page_size: int) -> bool:
+        return (compute_dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.head_dim <= 256
+                and page_size % 4 == 0)
 
     def plan(self, host) -> Dict[str, object]:
-        items, merges = [], []
+        mfma = self.uses_mfma(host.compute_dtype, host.page_size)
+        small_tokens, large_tokens, split_keys = self.geometry(mfma)
+        small, large, merges = [], [], []
         n_partial = 0
         for s in range(host.n_seqs):
             n, p, row0 = host.q_lens[s], host.past_lens[s], host.q_starts[s]
             first_key = max(0, p - self.window + 1) if self.window else 0
             total = p + n
-            if n <= self.tile_tokens and total - first_key > self.split_keys:
-                n_splits = -(-(total - first_key) // self.split_keys)
+            if n <= small_tokens and total - first_key > split_keys:
+                n_splits = -(-(total - first_key) // split_keys)
                 base = n_partial
                 for i in range(n_splits):
-                    kb = first_key + i * self.split_keys
-                    items.append((s, row0, n, p, kb, min(total, kb + self.split_keys), base + i * n, 0))
+                    kb = first_key + i * split_keys
+                    small.append((s, row0, n, p, kb, min(total, kb + split_keys), base + i * n, 0))
                 for t in range(n):
                     merges.append((row0 + t, base + t, n_splits, n))
                 n_partial += n_splits * n
+            elif n <= small_tokens:
+                small.append((s, row0, n, p, first_key, total, -1, 0))
             else:
-                for t0 in range(0, n, self.tile_tokens):
-                    nq = min(self.tile_tokens, n - t0)
+                for t0 in range(0, n, large_tokens):
+                    nq = min(large_tokens, n - t0)
                     pos0 = p + t0
                     kb = max(0, pos0 - self.window + 1) if self.window else 0
-                    items.append((s, row0 + t0, nq, pos0, kb, pos0 + nq, -1, 0))
+                    (small if nq <= small_tokens else large).append((s, row0 + t0, nq, pos0, kb, pos0 + nq, -1, 0))
         return {
-            "items": np.asarray(items, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS),
+            "items": np.asarray(small + large, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS),
             "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
-            "n_items": len(items), "n_merges": len(merges), "n_partial": n_partial,
+            "n_small": len(small), "n_large": len(large), "n_merges": len(merges), "n_partial": n_partial,
+            "mfma": mfma,
         }
 
 
@@ -69,8 +95,6 @@ class GQAttention(Mixer):
     kv head = q head // (heads / kv heads) and scale 1/sqrt(head_dim), output projection without
     bias (src/model/model.cpp:110-129, src/model/nn.cpp:151-226).  ``window`` = number of latest
     positions a query reads (None: all)."""
-
-    SPLIT_KEYS = 256
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
                  position: PositionEncoding, window: Optional[int] = None):
@@ -108,8 +132,7 @@ class GQAttention(Mixer):
 
     def planner(self) -> AttentionPlanner:
         if self._planner is None:
-            self._planner = AttentionPlanner(self.window, ops.attention_tile_tokens(self.n_heads, self.n_kv),
-                                             self.SPLIT_KEYS)
+            self._planner = AttentionPlanner(self.n_heads, self.n_kv, self.head_dim, self.window)
         return self._planner
 
     # compute ----------------------------------------------------------------------------
@@ -124,9 +147,17 @@ class GQAttention(Mixer):
         if plan.n_partial:
             partials = torch.empty((plan.n_partial * self.n_heads * (self.head_dim + 2),), dtype=torch.float32,
                                    device=x.device)
-        ops.attention_scalar(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
-                             plan.n_items, out, partials, self.n_heads, self.n_kv, self.head_dim, self.window,
-                             self.scale, t)
+        args = (partials, self.n_heads, self.n_kv, self.head_dim, self.window, self.scale, t)
+        if plan.mfma:
+            if plan.n_small:
+                ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
+                                   plan.n_small, out, *args, large=False)
+            if plan.n_large:
+                ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
+                                   plan.items[plan.n_small:], plan.n_large, out, *args, large=True)
+        else:
+            ops.attention_scalar(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
+                                 plan.n_small + plan.n_large, out, *args)
         if plan.n_merges:
             ops.attention_merge(partials, plan.merges, plan.n_merges, out, self.n_heads, self.head_dim)
         return self.o(out)

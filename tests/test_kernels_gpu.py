@@ -81,7 +81,7 @@ def test_rope_and_cache_write(ops, dtype, heads, kv, hd, theta):
     slots = torch.tensor([12, 13, 14, 40, 41, -1, 5, 6, 7], dtype=torch.int32)
     inv = torch.tensor([theta ** (-2.0 * i / hd) for i in range(hd // 2)], dtype=torch.float64)
     k_pool = torch.zeros((pages, kv, page, hd), dtype=dtype)
-    v_pool = torch.zeros_like(k_pool)
+    v_pool = torch.zeros((pages, kv, hd, page), dtype=dtype)
     dq, dk, dv = qkv.clone().cuda(), k_pool.cuda(), v_pool.cuda()
     ops.rope_kv_write(dq, pos.cuda(), heads, kv, hd, inv.cuda(), slots=slots.cuda(), k_pool=dk, v_pool=dv,
                       page_size=page, bias=bias.cuda())
@@ -99,9 +99,9 @@ def test_rope_and_cache_write(ops, dtype, heads, kv, hd, theta):
             continue
         written[s] = True
         assert (kp[s // page, :, s % page, :].reshape(-1) - k_ref[i]).abs().max() <= tol(dtype, k_ref, f32=2e-6)
-        assert (vp[s // page, :, s % page, :].reshape(-1) - v_ref[i]).abs().max() <= tol(dtype, v_ref, f32=2e-6)
+        assert (vp[s // page, :, :, s % page].reshape(-1) - v_ref[i]).abs().max() <= tol(dtype, v_ref, f32=2e-6)
     untouched = ~written.reshape(pages, 1, page, 1).expand_as(kp)
-    assert kp[untouched].abs().max() == 0 and vp[untouched].abs().max() == 0
+    assert kp[untouched].abs().max() == 0 and vp.transpose(2, 3)[untouched].abs().max() == 0
     # no rotation, no cache: only the bias on q and k
     dq = qkv.clone().cuda()
     ops.rope_kv_write(dq, pos.cuda(), heads, kv, hd, None, bias=bias.cuda())
@@ -150,13 +150,13 @@ def test_refusals(ops):
         ops.swiglu(torch.zeros(2, 4, dtype=torch.float16).cuda())
     with pytest.raises(KernelError, match="head_dim"):
         q = torch.zeros(1, 3 * 300).cuda()
-        ops.attention_scalar(q, 900, torch.zeros(1, 1, 4, 300).cuda(), torch.zeros(1, 1, 4, 300).cuda(),
+        ops.attention_scalar(q, 900, torch.zeros(1, 1, 4, 300).cuda(), torch.zeros(1, 1, 300, 4).cuda(),
                              torch.zeros(1, 1, dtype=torch.int32).cuda(), torch.zeros(1, 8, dtype=torch.int32).cuda(), 1,
                              torch.zeros(1, 300).cuda(), None, 1, 1, 300, None, 1.0, 1)
 
 
 # ------------------------------------------------------------------------------ attention
-def paged_case(seqs, heads, kv, hd, page, dtype, seed, window=None, shuffle=True, edit=None):
+def paged_case(seqs, heads, kv, hd, page, dtype, seed, window=None, shuffle=True, edit=None, scalar=False):
     """seqs: list of (past, n_new).  Returns device inputs for the kernel and per-seq q/k/v.
     ``edit(qs, ks, vs)`` may change the random tensors in place before the pages are filled."""
     from from_scratch_inference_engine_amd.parts.attention import AttentionPlanner
@@ -167,7 +167,7 @@ def paged_case(seqs, heads, kv, hd, page, dtype, seed, window=None, shuffle=True
     order = (torch.randperm(total_pages, generator=torch.Generator().manual_seed(seed + 1)).tolist()
              if shuffle else list(range(total_pages)))
     k_pool = torch.full((total_pages, kv, page, hd), 7.0)  # stale content in unused slots
-    v_pool = torch.full((total_pages, kv, page, hd), -9.0)
+    v_pool = torch.full((total_pages, kv, hd, page), -9.0)
     max_pages = max(-(-(p + n) // page) for p, n in seqs)
     tables = torch.full((len(seqs), max_pages), -1, dtype=torch.int32)
     qs, ks, vs = [], [], []
@@ -184,16 +184,18 @@ def paged_case(seqs, heads, kv, hd, page, dtype, seed, window=None, shuffle=True
         for j in range(total):
             pg, off = tables[s, j // page].item(), j % page
             k_pool[pg, :, off, :] = ks[s][j].reshape(kv, hd)
-            v_pool[pg, :, off, :] = vs[s][j].reshape(kv, hd)
+            v_pool[pg, :, :, off] = vs[s][j].reshape(kv, hd)
 
     class Host:
         n_seqs = len(seqs)
         q_lens = [n for _, n in seqs]
         past_lens = [p for p, _ in seqs]
         q_starts = [0]
+        page_size = page
+        compute_dtype = torch.float32 if scalar else dtype  # scalar: the float32-arithmetic kernel on this storage
     for _, n in seqs:
         Host.q_starts.append(Host.q_starts[-1] + n)
-    plan = AttentionPlanner(window, ops.attention_tile_tokens(heads, kv), 256).plan(Host)
+    plan = AttentionPlanner(heads, kv, hd, window).plan(Host)
     return dict(q=torch.cat(qs).to(dtype), k_pool=k_pool.to(dtype), v_pool=v_pool.to(dtype), tables=tables, plan=plan,
                 qs=qs, ks=ks, vs=vs)
 
@@ -205,26 +207,36 @@ def run_attention(ops, case, heads, kv, hd, window=None):
     out = torch.zeros((t, heads * hd), dtype=q.dtype).cuda()
     partials = torch.empty(max(plan["n_partial"], 1) * heads * (hd + 2), dtype=torch.float32).cuda()
     items = torch.from_numpy(plan["items"]).cuda()
-    ops.attention_scalar(q, heads * hd, case["k_pool"].cuda(), case["v_pool"].cuda(), case["tables"].cuda(), items,
-                         plan["n_items"], out, partials, heads, kv, hd, window, 1.0 / math.sqrt(hd), t)
+    common = (out, partials, heads, kv, hd, window, 1.0 / math.sqrt(hd), t)
+    pools = (case["k_pool"].cuda(), case["v_pool"].cuda(), case["tables"].cuda())
+    if plan["mfma"]:
+        if plan["n_small"]:
+            ops.attention_mfma(q, heads * hd, *pools, items, plan["n_small"], *common, large=False)
+        if plan["n_large"]:
+            ops.attention_mfma(q, heads * hd, *pools, items[plan["n_small"]:], plan["n_large"], *common, large=True)
+    else:
+        ops.attention_scalar(q, heads * hd, *pools, items, plan["n_small"] + plan["n_large"], *common)
     if plan["n_merges"]:
         ops.attention_merge(partials, torch.from_numpy(plan["merges"]).cuda(), plan["n_merges"], out, heads, hd)
     return out.float().cpu()
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dtype, scalar", [(torch.float32, True), (torch.bfloat16, True), (torch.bfloat16, False)])
 @pytest.mark.parametrize("heads, kv, hd, page, window", [
     (14, 2, 64, 16, None),   # the reference's kernel test sizes (tests/cpp/test_cuda_kernels.cpp:126-164)
     (4, 4, 48, 4, None),     # plain multi-head, head size no power of two
     (20, 1, 32, 8, None),    # more heads per kv head than rows of a block
     (6, 2, 128, 16, 37),     # a window
     (3, 1, 256, 64, None),
+    (28, 4, 128, 16, None),  # a large model's geometry: 7 heads per kv head
+    (2, 1, 80, 12, 300),     # head size an odd multiple of 16, page size no power of two
 ])
-def test_attention_over_pages(ops, dtype, heads, kv, hd, page, window):
+def test_attention_over_pages(ops, dtype, scalar, heads, kv, hd, page, window):
     # (past, new): the reference's (7, 5) and (19, 1), a long decode that is split, whole prompts,
     # portions starting mid-page, a two-token portion
-    seqs = [(7, 5), (19, 1), (600, 1), (0, 33), (300, 2), (123, 70), (0, 1)]
-    case = paged_case(seqs, heads, kv, hd, page, dtype, seed=hd + heads, window=window)
+    seqs = [(7, 5), (19, 1), (600, 1), (0, 33), (300, 2), (123, 70), (0, 1), (40, 200)]
+    case = paged_case(seqs, heads, kv, hd, page, dtype, seed=hd + heads, window=window, scalar=scalar)
+    assert case["plan"]["mfma"] == (not scalar)
     out = run_attention(ops, case, heads, kv, hd, window)
     row = 0
     for (p, n), q, k, v in zip(seqs, case["qs"], case["ks"], case["vs"]):
@@ -234,7 +246,8 @@ def test_attention_over_pages(ops, dtype, heads, kv, hd, page, window):
         row += n
 
 
-def test_attention_finds_one_far_key_and_respects_edges(ops):
+@pytest.mark.parametrize("dtype, scalar", [(torch.float32, True), (torch.bfloat16, False)])
+def test_attention_finds_one_far_key_and_respects_edges(ops, dtype, scalar):
     """Inputs that random data would hide a fault behind: for every query one key far back (or
     at the far edge of its window) carries nearly the whole softmax, so the output must be that
     key's value; and louder keys sit where the query must not look: right after its own
@@ -256,20 +269,20 @@ def test_attention_finds_one_far_key_and_respects_edges(ops):
                         # the heads of one group share the key: point all of them at it
                         q[kvh * group:(kvh + 1) * group] = q[kvh * group] * 1.0
                         u = q[kvh * group] / q[kvh * group].norm()
-                        ks[s][far].reshape(kv, hd)[kvh] = 40.0 * u
-                        q[kvh * group:(kvh + 1) * group] = 8.0 * u
-                        loud = 400.0 * u
+                        ks[s][far].reshape(kv, hd)[kvh] = (40.0 * u).to(dtype).float()
+                        q[kvh * group:(kvh + 1) * group] = (8.0 * u).to(dtype).float()
+                        loud = (400.0 * u).to(dtype).float()
                         if pos + 1 < p + n:
                             ks[s][pos + 1].reshape(kv, hd)[kvh] = loud       # the future
                         if window and pos - window >= 0 and pos - window not in chosen.values():
                             ks[s][pos - window].reshape(kv, hd)[kvh] = loud  # just outside the window
 
-        case = paged_case(seqs, heads, kv, hd, page, torch.float32, seed=3, window=window, edit=edit)
+        case = paged_case(seqs, heads, kv, hd, page, dtype, seed=3, window=window, edit=edit, scalar=scalar)
         out = run_attention(ops, case, heads, kv, hd, window)
         row = 0
         for s, ((p, n), q, k, v) in enumerate(zip(seqs, case["qs"], case["ks"], case["vs"])):
             ref = plain.attention(q, k, v, heads, kv, hd, query_offset=p, window=window)
-            assert (out[row:row + n] - ref).abs().max() <= 5e-6
+            assert (out[row:row + n] - ref).abs().max() <= (5e-6 if dtype == torch.float32 else 2.0 ** -7 * ref.abs().max())
             for i in range(n):  # and the plain result is what the construction says: the far key's value
                 want = v[chosen[(s, i)]].reshape(kv, 1, hd).expand(kv, group, hd).reshape(-1)
                 if i == 0:
@@ -280,9 +293,10 @@ def test_attention_finds_one_far_key_and_respects_edges(ops):
 def test_attention_does_not_depend_on_page_ids(ops):
     heads, kv, hd, page = 8, 2, 64, 16
     seqs = [(100, 1), (0, 40)]
-    a = run_attention(ops, paged_case(seqs, heads, kv, hd, page, torch.float32, 5, shuffle=True), heads, kv, hd)
-    b = run_attention(ops, paged_case(seqs, heads, kv, hd, page, torch.float32, 5, shuffle=False), heads, kv, hd)
-    assert torch.equal(a, b)
+    for dtype in DTYPES:
+        a = run_attention(ops, paged_case(seqs, heads, kv, hd, page, dtype, 5, shuffle=True), heads, kv, hd)
+        b = run_attention(ops, paged_case(seqs, heads, kv, hd, page, dtype, 5, shuffle=False), heads, kv, hd)
+        assert torch.equal(a, b)
 
 
 # ------------------------------------------------------------------------------ sampling
