@@ -11,6 +11,7 @@
 
 #define FSIE_GEMM_SKINNY_MAX_M 8
 #define FSIE_GEMM_MFMA_SKINNY_MAX_M 64
+#define FSIE_GEMM_MFMA_SKINNY_BEST_M 16  // above this the library product is faster on MI355X
 
 // one attention work item = 8 int32
 #define FSIE_ATTN_ITEM_INTS 8
@@ -49,7 +50,7 @@ int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, i
               int out_f32, int kind, hipStream_t stream);
 
 int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
-                          int out_f32, int waves, hipStream_t stream);
+                          int out_f32, int waves, int blocks, hipStream_t stream);
 
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,

@@ -55,6 +55,95 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const T* __restrict
     }
 }
 
+// The same for hidden % 4 == 0 and hidden <= 1024 * ITERS: the row stays in registers between
+// the two passes and moves with 16-byte (float32) and 8- or 16-byte (T) accesses.
+template <typename T>
+struct Pack4;
+template <>
+struct Pack4<float> {
+    static __device__ __forceinline__ float4 load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+    static __device__ __forceinline__ void store(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+};
+template <>
+struct Pack4<bf16_t> {
+    static __device__ __forceinline__ float4 load(const bf16_t* p) {
+        const uint2 w = *reinterpret_cast<const uint2*>(p);
+        return float4{__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                      __uint_as_float(w.y & 0xffff0000u)};
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, float4 v) {
+        uint2 w;
+        w.x = static_cast<uint32_t>(float_to_bf16_bits(v.x)) | (static_cast<uint32_t>(float_to_bf16_bits(v.y)) << 16);
+        w.y = static_cast<uint32_t>(float_to_bf16_bits(v.z)) | (static_cast<uint32_t>(float_to_bf16_bits(v.w)) << 16);
+        *reinterpret_cast<uint2*>(p) = w;
+    }
+};
+
+template <typename T, int ITERS>
+__global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                                               const float* __restrict__ weight, T* __restrict__ out,
+                                                               const int32_t* __restrict__ rows, int hidden, float eps,
+                                                               int write_back) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int64_t row = rows ? rows[r] : r;
+    float* res = residual + row * hidden;
+    const T* del = delta ? delta + row * hidden : nullptr;
+    float4 v[ITERS];
+    float sum_sq = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (it * kThreads + threadIdx.x) * 4;
+        v[it] = float4{0.f, 0.f, 0.f, 0.f};
+        if (j < hidden) {
+            v[it] = Pack4<float>::load(res + j);
+            if (del) {
+                const float4 d = Pack4<T>::load(del + j);
+                v[it].x += d.x;
+                v[it].y += d.y;
+                v[it].z += d.z;
+                v[it].w += d.w;
+            }
+            if (write_back) Pack4<float>::store(res + j, v[it]);
+            sum_sq += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
+        }
+    }
+    const float total = block_sum(sum_sq, scratch);
+    const float scale = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    T* dst = out + static_cast<int64_t>(r) * hidden;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = (it * kThreads + threadIdx.x) * 4;
+        if (j < hidden) {
+            const float4 w = Pack4<float>::load(weight + j);
+            Pack4<T>::store(dst + j, float4{(v[it].x * scale) * w.x, (v[it].y * scale) * w.y, (v[it].z * scale) * w.z,
+                                            (v[it].w * scale) * w.w});
+        }
+    }
+}
+
+template <typename T>
+void launch_rmsnorm(float* residual, const void* delta, const float* weight, void* out, const int32_t* rows, int n_rows,
+                    int hidden, float eps, int write_back, hipStream_t stream) {
+    const T* d = static_cast<const T*>(delta);
+    T* o = static_cast<T*>(out);
+    const bool aligned = hidden % 4 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(weight) % 16 == 0 && reinterpret_cast<uintptr_t>(delta) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    const int per_iter = kThreads * 4;
+    if (aligned && hidden <= per_iter) {
+        rmsnorm_vec_kernel<T, 1><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
+    } else if (aligned && hidden <= 2 * per_iter) {
+        rmsnorm_vec_kernel<T, 2><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
+    } else if (aligned && hidden <= 4 * per_iter) {
+        rmsnorm_vec_kernel<T, 4><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
+    } else if (aligned && hidden <= 8 * per_iter) {
+        rmsnorm_vec_kernel<T, 8><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
+    } else {
+        rmsnorm_kernel<T><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
+    }
+}
+
 // out[t, j] = silu(x[t, j]) * x[t, inter + j]; x is [T, 2*inter] (gate columns, then up).
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t total, int inter) {
@@ -105,11 +194,9 @@ extern "C" int fsie_rmsnorm(float* residual, const void* delta, const float* wei
     FSIE_REQUIRE(!(write_back && !delta), "rmsnorm: write_back without a delta");
     if (n_rows == 0) return 0;
     if (dtype == FSIE_F32) {
-        rmsnorm_kernel<float><<<n_rows, kThreads, 0, stream>>>(residual, static_cast<const float*>(delta), weight,
-                                                               static_cast<float*>(out), rows, hidden, eps, write_back);
+        launch_rmsnorm<float>(residual, delta, weight, out, rows, n_rows, hidden, eps, write_back, stream);
     } else {
-        rmsnorm_kernel<bf16_t><<<n_rows, kThreads, 0, stream>>>(residual, static_cast<const bf16_t*>(delta), weight,
-                                                                static_cast<bf16_t*>(out), rows, hidden, eps, write_back);
+        launch_rmsnorm<bf16_t>(residual, delta, weight, out, rows, n_rows, hidden, eps, write_back, stream);
     }
     FSIE_CHECK_LAUNCH("rmsnorm");
     return 0;

@@ -26,14 +26,17 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
     const int kv_dim = n_kv * head_dim;
     T* row = qkv + static_cast<int64_t>(t) * (q_dim + 2 * kv_dim);
 
-    // angle = position * inv_freq in float64, as the plain formula has it; cos and sin are
-    // rounded to float32 once.
+    // angle = position * inv_freq in float64, as the plain formula has it, reduced in float64 to
+    // [-pi, pi]; there float32 sine and cosine are within a few 1e-7 of the float64 ones.
     const double pos = static_cast<double>(positions[t]);
     for (int i = threadIdx.x; i < rotary_half; i += blockDim.x) {
-        double s, c;
-        sincos(pos * inv_freq[i], &s, &c);
-        cs[i] = static_cast<float>(c);
-        sn[i] = static_cast<float>(s);
+        const double ang = pos * inv_freq[i];
+        const double turns = rint(ang * 0.15915494309189535);  // 1 / (2 pi)
+        const double red = fma(-turns, 6.283185307179586, ang) - turns * 2.4492935982947064e-16;  // 2 pi = hi + lo
+        float s, c;
+        sincosf(static_cast<float>(red), &s, &c);
+        cs[i] = c;
+        sn[i] = s;
     }
     __syncthreads();
 

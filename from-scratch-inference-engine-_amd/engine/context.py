@@ -32,6 +32,7 @@ class HostBatch:
     def __init__(self, entries: Sequence[StepEntry], page_size: int = 0, compute_dtype=None):
         self.page_size = page_size
         self.compute_dtype = compute_dtype
+        self.pad = None  # set for a step that replays a captured graph: tables padded to fixed sizes
         self.n_seqs = len(entries)
         self.q_lens = [len(e.tokens) for e in entries]
         self.past_lens = [e.cache.length for e in entries]
@@ -66,15 +67,24 @@ class _Packer:
         self._total += -(-max(array.size, 1) // self.ALIGN) * self.ALIGN
         return len(self._arrays) - 1
 
-    def upload(self, staging: "PinnedStaging", device) -> List[torch.Tensor]:
+    @property
+    def total(self) -> int:
+        return self._total
+
+    def upload(self, staging: "PinnedStaging", device, into: Optional[torch.Tensor] = None) -> List[torch.Tensor]:
+        """Copy everything to the device in one go; ``into`` = an existing buffer of the same
+        layout (a captured graph reads it), else a new one."""
         host = staging.acquire(self._total)
         flat = host.numpy()
         for a, off in zip(self._arrays, self._offsets):
             flat[off:off + a.size] = a.reshape(-1)
-        dev = torch.empty((self._total,), dtype=torch.int32, device=device)
-        dev.copy_(host[:self._total], non_blocking=True)
+        if into is None:
+            into = torch.empty((self._total,), dtype=torch.int32, device=device)
+        elif into.numel() != self._total:
+            raise RuntimeError("step tables do not have the layout of the captured graph")
+        into.copy_(host[:self._total], non_blocking=True)
         staging.release()
-        return [dev[off:off + a.size].view(a.shape) for a, off in zip(self._arrays, self._offsets)]
+        return [into[off:off + a.size].view(a.shape) for a, off in zip(self._arrays, self._offsets)]
 
 
 class PinnedStaging:
@@ -127,9 +137,16 @@ class StepContext:
 
 
 def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners: Sequence, staging: PinnedStaging,
-                  compute_dtype: torch.dtype, device) -> StepContext:
-    """Tables of one step.  The entries' pages must have been reserved already."""
+                  compute_dtype: torch.dtype, device, pad: Optional[dict] = None,
+                  into: Optional[torch.Tensor] = None):
+    """Tables of one step.  The entries' pages must have been reserved already.
+
+    ``pad`` fixes the sizes of everything whose size depends on the requests' lengths (for a
+    step that a captured graph replays): ``pad["pages"]`` = width of the block tables,
+    ``pad[planner.key]`` = what that planner's ``graph_bucket`` returned.  Returns the context
+    and the device buffer that holds all tables."""
     host = HostBatch(entries, manager.page_size, compute_dtype)
+    host.pad = pad
     ctx = StepContext(host, compute_dtype, device)
     pk = _Packer()
     i_ids = pk.add(host.token_ids.astype(np.int32))
@@ -142,6 +159,10 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
     group_idx = []
     for g in range(len(manager.groups)):
         max_pages = max([len(e.cache.tables[g]) for e in entries] + [1])
+        if pad is not None:
+            if max_pages > pad["pages"]:
+                raise RuntimeError("block tables are wider than the captured graph's")
+            max_pages = pad["pages"]
         table = np.full((len(entries), max_pages), -1, dtype=np.int32)
         slot_map = np.full((host.n_tokens,), -1, dtype=np.int32)
         for s, e in enumerate(entries):
@@ -157,7 +178,7 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
         arrays = {k: pk.add(v) for k, v in made.items() if isinstance(v, np.ndarray)}
         scalars = {k: v for k, v in made.items() if not isinstance(v, np.ndarray)}
         plan_idx.append((planner.key, arrays, scalars))
-    dev = pk.upload(staging, device)
+    dev = pk.upload(staging, device, into)
     ctx.token_ids, ctx.positions, ctx.want_rows = dev[i_ids], dev[i_pos], dev[i_want]
     ctx.seq_slots, ctx.q_starts, ctx.past_lens = dev[i_slots], dev[i_qs], dev[i_past]
     for it, isl in group_idx:
@@ -165,4 +186,5 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
         ctx.slots.append(dev[isl])
     for key, arrays, scalars in plan_idx:
         ctx._plans[key] = SimpleNamespace(**{k: dev[i] for k, i in arrays.items()}, **scalars)
-    return ctx
+    base = dev[0]._base if dev and dev[0]._base is not None else (dev[0] if dev else None)
+    return ctx, base

@@ -47,7 +47,7 @@ class Engine:
             return
         entries = [StepEntry(it.seq.cache, it.tokens, [len(it.tokens) - 1] if it.wants_logits else [])
                    for it in items]
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, keep=False)
         wanting = [it for it in items if it.wants_logits]
         tokens = self.sampler.sample(logits, [it.seq.request.params for it in wanting],
                                      [it.seq.id for it in wanting], [len(it.seq.output) for it in wanting])

@@ -1,0 +1,78 @@
+"""Decode steps as replayed HIP graphs.
+
+A decode step launches some ten kernels per layer, each a few microseconds long; queued one by
+one from Python they cost more host time than GPU time.  A step whose every request brings one
+token and wants its logits has a shape that depends only on the number of requests and, through
+the width of the block tables and the number of attention work items, on rounded-up context
+lengths.  For each such shape the whole forward is captured once into a graph that reads all
+its index tables from one fixed device buffer; a later step of the same shape copies its tables
+there and replays the graph.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Optional, Sequence, Tuple
+
+import torch
+
+from .context import HostBatch, StepEntry, build_context
+
+PAGE_BUCKET = 32  # block-table widths are rounded up to this many pages
+
+
+class DecodeGraphs:
+    def __init__(self, runner, max_graphs: int = 64):
+        self.runner = runner
+        self.max_graphs = max_graphs
+        self._graphs: Dict[Tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor]] = {}
+        model = runner.model
+        self.enabled = all(getattr(block.mixer, "graph_safe", False) for block in model.spec.layers) and all(
+            hasattr(p, "graph_bucket") for p in model.planners)
+        self.replays = 0
+        self.captures = 0
+
+    def shape_of(self, entries: Sequence[StepEntry]) -> Optional[dict]:
+        """The padded sizes of this step, or None if it is not a plain decode step."""
+        if not self.enabled or not all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            return None
+        runner = self.runner
+        host = HostBatch(entries, runner.manager.page_size, runner.model.dtype)
+        pages = max(len(t) for e in entries for t in e.cache.tables) if runner.manager.groups else 1
+        pad = {"pages": -(-pages // PAGE_BUCKET) * PAGE_BUCKET}
+        for planner in runner.model.planners:
+            bucket = planner.graph_bucket(host)
+            if bucket is None:
+                return None
+            pad[planner.key] = bucket
+        return pad
+
+    def step(self, entries: Sequence[StepEntry], pad: dict) -> torch.Tensor:
+        """Run the (already reserved) decode step through its graph; returns the logits, which
+        stay valid until the next step of the same shape."""
+        runner = self.runner
+        key = (len(entries),) + tuple(sorted((str(k), v) for k, v in pad.items()))
+        hit = self._graphs.get(key)
+        if hit is None:
+            if len(self._graphs) >= self.max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+            # eager run on the tables of this step first: allocates nothing the graph keeps, warms
+            # the library's kernel selection
+            ctx, tables = build_context(entries, runner.manager, runner.model.planners, runner._staging,
+                                        runner.model.dtype, runner.model.device, pad=pad)
+            runner.model.forward(ctx, runner.storage)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = runner.model.forward(ctx, runner.storage)
+            self._graphs[key] = (graph, tables, logits)
+            self.captures += 1
+            # the eager run above already wrote this step's keys and values; replaying writes the
+            # same values again
+            graph.replay()
+            return logits
+        graph, tables, logits = hit
+        build_context(entries, runner.manager, runner.model.planners, runner._staging, runner.model.dtype,
+                      runner.model.device, pad=pad, into=tables)
+        graph.replay()
+        self.replays += 1
+        return logits

@@ -151,7 +151,8 @@ class Model:
 class Runner:
     """The step function over one model and one cache."""
 
-    def __init__(self, model: Model, page_size: int = 16, num_pages: int = 2048, max_requests: int = 256):
+    def __init__(self, model: Model, page_size: int = 16, num_pages: int = 2048, max_requests: int = 256,
+                 use_graphs: bool = True):
         self.model = model
         self.manager, self.storage = model.make_cache(page_size, num_pages, max_requests)
         self._staging = PinnedStaging()
@@ -159,6 +160,9 @@ class Runner:
         self.max_position = int(getattr(model.config, "max_position_embeddings", 0) or 0)
         self.steps = 0
         self.tokens = 0
+        from .graphs import DecodeGraphs
+
+        self.graphs = DecodeGraphs(self) if use_graphs else None
 
     def check(self, entries: Sequence[StepEntry]) -> None:
         if not entries:
@@ -185,19 +189,27 @@ class Runner:
                 raise ValueError(f"step: request {e.cache.request_id!r} would reach {e.cache.length + n} "
                                  f"positions, more than max_position_embeddings {self.max_position}")
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Run one batch.  Nothing is changed when the batch is refused (bad ids, no pages)."""
+    def step(self, entries: Sequence[StepEntry], keep: bool = True) -> torch.Tensor:
+        """Run one batch.  Nothing is changed when the batch is refused (bad ids, no pages).
+        ``keep=False`` allows the returned logits to live in a buffer that the next step
+        overwrites (a caller that consumes them at once saves a copy)."""
         self.check(entries)
         if not self.manager.can_reserve((e.cache, len(e.tokens)) for e in entries):
             raise OutOfPages("step: the batch needs more pages than the pool has free")
         for e in entries:
             self.manager.reserve(e.cache, len(e.tokens))
         self.storage.reset_states([e.cache.slot for e in entries if e.cache.length == 0])
-        ctx = build_context(entries, self.manager, self.model.planners, self._staging, self.model.dtype,
-                            self.model.device)
-        logits = self.model.forward(ctx, self.storage)
+        pad = self.graphs.shape_of(entries) if self.graphs is not None else None
+        if pad is not None:
+            logits = self.graphs.step(entries, pad)
+            if keep:
+                logits = logits.clone()
+        else:
+            ctx, _ = build_context(entries, self.manager, self.model.planners, self._staging, self.model.dtype,
+                                   self.model.device)
+            logits = self.model.forward(ctx, self.storage)
         for e in entries:
             self.manager.commit(e.cache, len(e.tokens))
         self.steps += 1
-        self.tokens += ctx.n_tokens
+        self.tokens += sum(len(e.tokens) for e in entries)
         return logits

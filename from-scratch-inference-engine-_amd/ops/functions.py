@@ -13,6 +13,7 @@ ATTN_ITEM_INTS = 8
 ATTN_MERGE_INTS = 4
 GEMM_SKINNY_MAX_M = 8
 GEMM_MFMA_SKINNY_MAX_M = 64
+GEMM_MFMA_SKINNY_BEST_M = 16
 GEMM_AUTO, GEMM_TILED, GEMM_SKINNY = 0, 1, 2
 
 
@@ -170,7 +171,7 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = N
 
 
 def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-                     out_dtype: Optional[torch.dtype] = None, waves: int = 0,
+                     out_dtype: Optional[torch.dtype] = None, waves: int = 0, blocks: int = 0,
                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same product on the matrix cores for bfloat16 and at most 64 rows (K a multiple of 8)."""
     _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
@@ -188,7 +189,7 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     _need(out, "gemm out", dtype=out_dtype, shape=(m, n))
     check(load().fsie_gemm_mfma_skinny(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
-                                       int(out_dtype == torch.float32), waves, _stream()))
+                                       int(out_dtype == torch.float32), waves, blocks, _stream()))
     return out
 
 

@@ -55,6 +55,20 @@ class AttentionPlanner:
         return (compute_dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.head_dim <= 256
                 and page_size % 4 == 0)
 
+    def graph_bucket(self, host) -> Optional[int]:
+        """Number of (small) work items, rounded up, that a captured graph of this step's shape
+        must launch; None if the step has portions that do not fit small items."""
+        mfma = self.uses_mfma(host.compute_dtype, host.page_size)
+        small_tokens, _, split_keys = self.geometry(mfma)
+        n = 0
+        for s in range(host.n_seqs):
+            if host.q_lens[s] > small_tokens:
+                return None
+            first_key = max(0, host.past_lens[s] - self.window + 1) if self.window else 0
+            n += max(1, -(-(host.past_lens[s] + host.q_lens[s] - first_key) // split_keys))
+        step = 4 * host.n_seqs
+        return -(-n // step) * step
+
     def plan(self, host) -> Dict[str, object]:
         mfma = self.uses_mfma(host.compute_dtype, host.page_size)
         small_tokens, large_tokens, split_keys = self.geometry(mfma)
@@ -81,6 +95,15 @@ class AttentionPlanner:
                     pos0 = p + t0
                     kb = max(0, pos0 - self.window + 1) if self.window else 0
                     (small if nq <= small_tokens else large).append((s, row0 + t0, nq, pos0, kb, pos0 + nq, -1, 0))
+        if getattr(host, "pad", None) is not None:
+            # a captured graph launches fixed grids: pad with items and merges that do nothing
+            n_items = host.pad[self.key]
+            if large or len(small) > n_items:
+                raise RuntimeError("attention plan does not fit the captured graph")
+            small += [(0, 0, 0, 0, 0, 0, -1, 0)] * (n_items - len(small))
+            merged = {m[0] for m in merges}
+            merges += [(row, 0, 0, 0) for row in range(host.n_tokens) if row not in merged]
+            n_partial = n_items * small_tokens
         return {
             "items": np.asarray(small + large, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS),
             "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
@@ -95,6 +118,8 @@ class GQAttention(Mixer):
     kv head = q head // (heads / kv heads) and scale 1/sqrt(head_dim), output projection without
     bias (src/model/model.cpp:110-129, src/model/nn.cpp:151-226).  ``window`` = number of latest
     positions a query reads (None: all)."""
+
+    graph_safe = True  # forward reads the step only through device tables: a captured graph may replay it
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
                  position: PositionEncoding, window: Optional[int] = None):

@@ -69,6 +69,9 @@ class Norm(Part):
 
 class Mixer(Part):
     kind = "mixer"
+    # True if forward() takes everything that changes from step to step from device tensors of
+    # the context (never from ctx.host), so that a captured graph of a step can be replayed
+    graph_safe = False
 
     def cache_need(self):
         return None

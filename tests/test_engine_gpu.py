@@ -171,3 +171,35 @@ def test_graft_entry_smoke():
     import __graft_entry__ as entry
 
     entry.smoke()
+
+
+def test_graph_replays_equal_eager_steps(model_dirs):
+    """Decode steps run as replayed graphs.  Two runners over the same model, one with graphs and
+    one without, decode the same 20 requests (more rows than the engine's own small-matrix kernel
+    takes, so the library product is inside the graph too) for several steps, with other eager
+    work and synchronisations between the replays; every step's logits must agree, and contexts
+    that grow across a bucket edge must capture again and still agree."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    model = load_model(model_dirs["B"], dtype="bfloat16")
+    runners = [Runner(model, page_size=4, num_pages=640, max_requests=32, use_graphs=g) for g in (True, False)]
+    prompts = [helpers.token_ids(509, 3 + 5 * i, 300 + i) for i in range(20)]
+    caches = [[r.manager.open(i) for i in range(20)] for r in runners]
+    for r, cs in zip(runners, caches):
+        r.step([StepEntry(c, p, []) for c, p in zip(cs, prompts)])
+    feed = [helpers.token_ids(509, 40, 400 + i) for i in range(20)]
+    for t in range(40):
+        outs = []
+        for r, cs in zip(runners, caches):
+            outs.append(r.step([StepEntry(c, [feed[i][t]], [0]) for i, c in enumerate(cs)]).float().cpu())
+            torch.cuda.synchronize()
+            _ = (torch.randn(64, 64, device="cuda") @ torch.randn(64, 64, device="cuda")).sum().item()  # eager work between replays
+        assert torch.equal(outs[0], outs[1]), f"decode step {t}"
+    g = runners[0].graphs
+    assert g.captures >= 2 and g.replays >= 30
+    # a step that is not a plain decode step does not go through a graph
+    before = g.captures + g.replays
+    runners[0].step([StepEntry(caches[0][0], [1, 2], [1])])
+    assert g.captures + g.replays == before
