@@ -63,8 +63,9 @@ int fsie_attention_scalar_tile_tokens(int n_heads, int n_kv);
 int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                         const int32_t* block_tables, int max_pages, const int32_t* items, int n_items, void* out,
                         float* partials, int n_heads, int n_kv, int head_dim, int page_size, int window, float scale,
-                        int large, hipStream_t stream);
+                        int large, int waves, hipStream_t stream);
 int fsie_attention_mfma_tiles(int head_dim, int large);
+int fsie_attention_mfma_max_waves(int head_dim);
 
 int fsie_sample(const float* logits, int n_rows, int vocab, const float* temperature, const int32_t* top_k,
                 const float* top_p, const double* uniform, int32_t* out, hipStream_t stream);

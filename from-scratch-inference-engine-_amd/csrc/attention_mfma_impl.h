@@ -19,6 +19,12 @@
 //
 // HDT = head_dim / 16, NT = column tiles of 16 query rows per wave (rows = tokens x heads of the
 // kv head's group).  Keys are walked in blocks of 32.  Requires page_size % 4 == 0.
+//
+// A workgroup may have several waves (NT = 1 only, up to MAXW): they split the item's key range
+// into contiguous runs of blocks, and their partial results are combined inside the workgroup:
+// maxima and sums through LDS, then the rescaled accumulators are added into one LDS tile in the
+// fixed order of the waves.  Decoding against a long context therefore needs neither partial
+// records in memory nor a second kernel, and the result does not depend on timing.
 #pragma once
 
 #include "common.h"
@@ -47,8 +53,13 @@ __device__ __forceinline__ uint2 ld8(const bf16_t* p) { return *reinterpret_cast
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
-template <int HDT, int NT>
-__global__ __launch_bounds__(64) void attention_mfma_kernel(
+template <int HDT>
+constexpr int max_waves() {
+    return HDT <= 4 ? 16 : (HDT <= 8 ? 8 : 4);  // registers per wave grow with the head size
+}
+
+template <int HDT, int NT, int MAXW>
+__global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, bf16_t* __restrict__ out, float* __restrict__ partials, int n_heads,
@@ -79,7 +90,9 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     const int h_base = kvh * group + chunk * gh;
     const int n_rows = n_q * gh;
 
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n_waves = blockDim.x >> 6;
     const int c = lane & 15;  // column of S^T and O^T (query row of a tile); row of the A tiles
     const int G = lane >> 4;  // lane group: which 4 (or 8) of the reduction indices this lane holds
     const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
@@ -117,7 +130,16 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     }
 
     const int64_t head_stride = static_cast<int64_t>(page_size) * HD;  // one kv head of one page
-    for (int kb = key_begin & ~31; kb < key_end; kb += 32) {
+    // this wave's run of key blocks
+    const int kb_first = key_begin & ~31;
+    const int n_blocks = (key_end - kb_first + 31) >> 5;
+    // an item uses one wave per 4 blocks (128 keys) of its own, however many the launch has:
+    // how its keys are split depends on the item alone
+    const int n_active = min(n_waves, max(1, (n_blocks + 3) >> 2));
+    const int per_wave = (n_blocks + n_active - 1) / n_active;
+    const int kb_begin = kb_first + wave * per_wave * 32;
+    const int kb_end = min(key_end, kb_begin + per_wave * 32);
+    for (int kb = kb_begin; kb < kb_end; kb += 32) {
         // ---- keys (A operand of the scores) and values (A operand of the second product)
         F16B kf[2][S32A];
         F8B kt[2][S16A];
@@ -212,6 +234,54 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
         }
     }
 
+    // ---- several waves: combine inside the workgroup (NT == 1)
+    if (MAXW > 1 && NT == 1 && n_waves > 1) {
+        __shared__ float s_m[MAXW][16], s_l[MAXW][16];
+        __shared__ float s_o[MAXW > 1 ? HD * 16 : 1];
+        float l_w = l_run[0];
+        l_w += __shfl_xor(l_w, 16, FSIE_WAVE);
+        l_w += __shfl_xor(l_w, 32, FSIE_WAVE);
+        if (G == 0) {
+            s_m[wave][c] = m_run[0];
+            s_l[wave][c] = l_w;
+        }
+        __syncthreads();
+        float m_all = -INFINITY;
+        for (int w = 0; w < n_waves; ++w) m_all = fmaxf(m_all, s_m[w][c]);
+        float denom = 0.f;
+        for (int w = 0; w < n_waves; ++w) {
+            const float mw = s_m[w][c];
+            if (mw != -INFINITY) denom += s_l[w][c] * __builtin_amdgcn_exp2f(mw - m_all);
+        }
+        const float mine = (m_run[0] == -INFINITY || !(denom > 0.f)) ? 0.f
+                           : __builtin_amdgcn_exp2f(m_run[0] - m_all) / denom;
+        // add the rescaled accumulators into one tile, wave after wave
+        for (int w = 0; w < n_waves; ++w) {
+            if (wave == w) {
+#pragma unroll
+                for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float* slot = &s_o[(dt * 16 + 4 * G + r) * 16 + c];
+                        const float v = acc[0][dt][r] * mine;
+                        *slot = (w == 0) ? v : *slot + v;
+                    }
+            }
+            __syncthreads();
+        }
+        if (wave != 0 || !rvalid[0]) return;
+        bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[0]) * n_heads + rhead[0]) * HD + 4 * G;
+#pragma unroll
+        for (int dt = 0; dt < HDT; ++dt) {
+            const float* t = &s_o[(dt * 16 + 4 * G) * 16 + c];
+            uint2 wd;
+            wd.x = static_cast<uint32_t>(float_to_bf16_bits(t[0])) | (static_cast<uint32_t>(float_to_bf16_bits(t[16])) << 16);
+            wd.y = static_cast<uint32_t>(float_to_bf16_bits(t[32])) | (static_cast<uint32_t>(float_to_bf16_bits(t[48])) << 16);
+            *reinterpret_cast<uint2*>(o + dt * 16) = wd;
+        }
+        return;
+    }
+
     // ---- results: lane holds O^T[d = 16 dt + 4 G + r][row c]
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -248,13 +318,16 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
 template <int HDT, int NT>
 int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool, const int32_t* block_tables,
            int max_pages, const int32_t* items, int n_items, void* out, float* partials, int n_heads, int n_kv,
-           int page_size, int window, float scale, hipStream_t stream) {
+           int page_size, int window, float scale, int waves, hipStream_t stream) {
+    constexpr int MAXW = NT == 1 ? max_waves<HDT>() : 1;
     const int group = n_heads / n_kv;
     const int rows = 16 * NT;
     const int gh = group < rows ? group : rows;
     const int head_chunks = (group + gh - 1) / gh;
     const dim3 grid(n_items, n_kv * head_chunks);
-    attention_mfma_kernel<HDT, NT><<<grid, 64, 0, stream>>>(
+    if (waves < 1) waves = 1;
+    if (waves > MAXW) waves = MAXW;
+    attention_mfma_kernel<HDT, NT, MAXW><<<grid, 64 * waves, 0, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
         block_tables, max_pages, items, static_cast<bf16_t*>(out), partials, n_heads, n_kv, page_size, window, scale,
         gh, head_chunks);
@@ -263,6 +336,6 @@ int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_po
 }
 
 typedef int (*LaunchFn)(const void*, int64_t, const void*, const void*, const int32_t*, int, const int32_t*, int, void*,
-                        float*, int, int, int, int, float, hipStream_t);
+                        float*, int, int, int, int, float, int, hipStream_t);
 
 }  // namespace fsie_attn

@@ -237,12 +237,18 @@ def attention_mfma_rows(head_dim: int, large: bool) -> int:
     return 16 * load().fsie_attention_mfma_tiles(head_dim, int(large))
 
 
+def attention_mfma_max_waves(head_dim: int) -> int:
+    return load().fsie_attention_mfma_max_waves(head_dim)
+
+
 def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
                    block_tables: torch.Tensor, items: torch.Tensor, n_items: int, out: torch.Tensor,
                    partials: Optional[torch.Tensor], n_heads: int, n_kv: int, head_dim: int,
-                   window: Optional[int], scale: float, n_query_rows: int, large: bool) -> torch.Tensor:
+                   window: Optional[int], scale: float, n_query_rows: int, large: bool, waves: int = 1) -> torch.Tensor:
     """Attention of the work items over the paged cache on the matrix cores (bfloat16; head_dim a
-    multiple of 16; page size a multiple of 4).  ``items`` may be a view into a longer table."""
+    multiple of 16; page size a multiple of 4).  ``items`` may be a view into a longer table.
+    Small items (``large=False``) are worked on by ``waves`` waves of a workgroup that split the
+    keys and combine inside the workgroup."""
     if not q.is_cuda or q.dtype != torch.bfloat16:
         raise KernelError("attention_mfma q: must be bfloat16 on the GPU")
     _need(k_pool, "k_pool", dtype=q.dtype, ndim=4)
@@ -262,7 +268,7 @@ def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
     check(load().fsie_attention_mfma(q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                      block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(), n_items,
                                      out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim, page_size,
-                                     int(window or 0), float(scale), int(large), _stream()))
+                                     int(window or 0), float(scale), int(large), int(waves), _stream()))
     return out
 
 

@@ -22,9 +22,10 @@ class AttentionPlanner:
 
     A request's portion of n tokens at past length p becomes tiles of query tokens; a tile reads
     the keys from the start of its window to its last token.  A portion of at most
-    ``small_tokens`` tokens is one *small* item; if it reads more than ``split_keys`` keys
-    (decoding against a long context) it is split over the keys instead, ``split_keys`` per
-    item, and merged afterwards in the order of the splits.  Longer portions are cut into *large*
+    ``small_tokens`` tokens is one *small* item.  For the float32-arithmetic kernel a small item
+    that reads more than ``split_keys`` keys (decoding against a long context) is split over the
+    keys into several items and merged afterwards in the order of the splits; the matrix-core
+    kernel splits the keys among the waves of a workgroup instead (one wave per 128 keys).  Longer portions are cut into *large*
     tiles of ``large_tokens``.  Whether and how a portion is cut depends on the portion alone,
     never on what else is in the batch.  The item table lists the small items first.
 
@@ -45,7 +46,7 @@ class AttentionPlanner:
                 small = max(1, ops.attention_mfma_rows(self.head_dim, False) // min(group, 16))
                 rows = ops.attention_mfma_rows(self.head_dim, True)
                 large = max(1, rows // min(group, rows))
-                self._geometry[mfma] = (small, large, 128)
+                self._geometry[mfma] = (small, large, None)  # keys are split inside the workgroup
             else:
                 t = ops.attention_tile_tokens(self.n_heads, self.n_kv)
                 self._geometry[mfma] = (t, t, 256)
@@ -55,19 +56,32 @@ class AttentionPlanner:
         return (compute_dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.head_dim <= 256
                 and page_size % 4 == 0)
 
-    def graph_bucket(self, host) -> Optional[int]:
-        """Number of (small) work items, rounded up, that a captured graph of this step's shape
-        must launch; None if the step has portions that do not fit small items."""
+    @staticmethod
+    def _waves_for(keys: int, max_waves: int) -> int:
+        """Waves of a workgroup for an item of ``keys`` keys: one per 128 keys, a power of two."""
+        need = max(1, -(-keys // 128))
+        w = 1
+        while w < need and w < max_waves:
+            w *= 2
+        return min(w, max_waves)
+
+    def graph_bucket(self, host):
+        """What a captured graph of this step's shape must fix: the number of (small) work items
+        and the waves per item; None if the step has portions that do not fit small items."""
         mfma = self.uses_mfma(host.compute_dtype, host.page_size)
         small_tokens, _, split_keys = self.geometry(mfma)
-        n = 0
+        n, longest = 0, 1
         for s in range(host.n_seqs):
             if host.q_lens[s] > small_tokens:
                 return None
             first_key = max(0, host.past_lens[s] - self.window + 1) if self.window else 0
-            n += max(1, -(-(host.past_lens[s] + host.q_lens[s] - first_key) // split_keys))
+            keys = host.past_lens[s] + host.q_lens[s] - first_key
+            longest = max(longest, keys)
+            n += 1 if split_keys is None else max(1, -(-keys // split_keys))
+        if split_keys is None:
+            return (host.n_seqs, self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)))
         step = 4 * host.n_seqs
-        return -(-n // step) * step
+        return (-(-n // step) * step, 1)
 
     def plan(self, host) -> Dict[str, object]:
         mfma = self.uses_mfma(host.compute_dtype, host.page_size)
@@ -78,7 +92,7 @@ class AttentionPlanner:
             n, p, row0 = host.q_lens[s], host.past_lens[s], host.q_starts[s]
             first_key = max(0, p - self.window + 1) if self.window else 0
             total = p + n
-            if n <= small_tokens and total - first_key > split_keys:
+            if n <= small_tokens and split_keys is not None and total - first_key > split_keys:
                 n_splits = -(-(total - first_key) // split_keys)
                 base = n_partial
                 for i in range(n_splits):
@@ -95,20 +109,24 @@ class AttentionPlanner:
                     pos0 = p + t0
                     kb = max(0, pos0 - self.window + 1) if self.window else 0
                     (small if nq <= small_tokens else large).append((s, row0 + t0, nq, pos0, kb, pos0 + nq, -1, 0))
+        waves = 1
+        if mfma and small:
+            waves = self._waves_for(max(it[5] - it[4] for it in small), ops.attention_mfma_max_waves(self.head_dim))
         if getattr(host, "pad", None) is not None:
             # a captured graph launches fixed grids: pad with items and merges that do nothing
-            n_items = host.pad[self.key]
+            n_items, waves = host.pad[self.key]
             if large or len(small) > n_items:
                 raise RuntimeError("attention plan does not fit the captured graph")
             small += [(0, 0, 0, 0, 0, 0, -1, 0)] * (n_items - len(small))
-            merged = {m[0] for m in merges}
-            merges += [(row, 0, 0, 0) for row in range(host.n_tokens) if row not in merged]
-            n_partial = n_items * small_tokens
+            if split_keys is not None:
+                merged = {m[0] for m in merges}
+                merges += [(row, 0, 0, 0) for row in range(host.n_tokens) if row not in merged]
+                n_partial = n_items * small_tokens
         return {
             "items": np.asarray(small + large, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS),
             "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
             "n_small": len(small), "n_large": len(large), "n_merges": len(merges), "n_partial": n_partial,
-            "mfma": mfma,
+            "mfma": mfma, "waves": waves,
         }
 
 
@@ -176,7 +194,7 @@ class GQAttention(Mixer):
         if plan.mfma:
             if plan.n_small:
                 ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
-                                   plan.n_small, out, *args, large=False)
+                                   plan.n_small, out, *args, large=False, waves=plan.waves)
             if plan.n_large:
                 ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
                                    plan.items[plan.n_small:], plan.n_large, out, *args, large=True)

@@ -211,7 +211,7 @@ def run_attention(ops, case, heads, kv, hd, window=None):
     pools = (case["k_pool"].cuda(), case["v_pool"].cuda(), case["tables"].cuda())
     if plan["mfma"]:
         if plan["n_small"]:
-            ops.attention_mfma(q, heads * hd, *pools, items, plan["n_small"], *common, large=False)
+            ops.attention_mfma(q, heads * hd, *pools, items, plan["n_small"], *common, large=False, waves=plan["waves"])
         if plan["n_large"]:
             ops.attention_mfma(q, heads * hd, *pools, items[plan["n_small"]:], plan["n_large"], *common, large=True)
     else:
@@ -234,7 +234,7 @@ def run_attention(ops, case, heads, kv, hd, window=None):
 def test_attention_over_pages(ops, dtype, scalar, heads, kv, hd, page, window):
     # (past, new): the reference's (7, 5) and (19, 1), a long decode that is split, whole prompts,
     # portions starting mid-page, a two-token portion
-    seqs = [(7, 5), (19, 1), (600, 1), (0, 33), (300, 2), (123, 70), (0, 1), (40, 200)]
+    seqs = [(7, 5), (19, 1), (600, 1), (0, 33), (300, 2), (123, 70), (0, 1), (40, 200), (2500, 1)]
     case = paged_case(seqs, heads, kv, hd, page, dtype, seed=hd + heads, window=window, scalar=scalar)
     assert case["plan"]["mfma"] == (not scalar)
     out = run_attention(ops, case, heads, kv, hd, window)
