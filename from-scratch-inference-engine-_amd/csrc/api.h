@@ -50,7 +50,7 @@ int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, i
               int out_f32, int kind, hipStream_t stream);
 
 int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
-                          int out_f32, int waves, int blocks, hipStream_t stream);
+                          int out_f32, int waves, int blocks, int epilogue, hipStream_t stream);
 
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,

@@ -236,8 +236,10 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
 
     // ---- several waves: combine inside the workgroup (NT == 1)
     if (MAXW > 1 && NT == 1 && n_waves > 1) {
+        constexpr int kSlabFloats = 8192;              // 32 KB of LDS for the accumulators
+        constexpr int TP = kSlabFloats / (MAXW * 256); // head-dim tiles per phase (>= 1 for MAXW <= 16... 32)
         __shared__ float s_m[MAXW][16], s_l[MAXW][16];
-        __shared__ float s_o[MAXW > 1 ? HD * 16 : 1];
+        __shared__ float s_o[kSlabFloats];
         float l_w = l_run[0];
         l_w += __shfl_xor(l_w, 16, FSIE_WAVE);
         l_w += __shfl_xor(l_w, 32, FSIE_WAVE);
@@ -247,37 +249,40 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
         }
         __syncthreads();
         float m_all = -INFINITY;
-        for (int w = 0; w < n_waves; ++w) m_all = fmaxf(m_all, s_m[w][c]);
+        for (int w = 0; w < n_active; ++w) m_all = fmaxf(m_all, s_m[w][c]);
         float denom = 0.f;
-        for (int w = 0; w < n_waves; ++w) {
+        for (int w = 0; w < n_active; ++w) {
             const float mw = s_m[w][c];
             if (mw != -INFINITY) denom += s_l[w][c] * __builtin_amdgcn_exp2f(mw - m_all);
         }
         const float mine = (m_run[0] == -INFINITY || !(denom > 0.f)) ? 0.f
                            : __builtin_amdgcn_exp2f(m_run[0] - m_all) / denom;
-        // add the rescaled accumulators into one tile, wave after wave
-        for (int w = 0; w < n_waves; ++w) {
-            if (wave == w) {
+        // Each active wave lays its rescaled accumulators into a slab of its own, TP tiles of the
+        // head dimension at a time; then every thread sums the slabs for a few (d, row) places
+        // of its own column in the fixed order of the waves and writes them out.
+        bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[0]) * n_heads + rhead[0]) * HD;
+        const int n_threads = 64 * n_waves;
 #pragma unroll
-                for (int dt = 0; dt < HDT; ++dt)
+        for (int t0 = 0; t0 < HDT; t0 += TP) {
+            if (t0 > 0) __syncthreads();  // the slabs of the last phase have been read
+            if (wave < n_active) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        float* slot = &s_o[(dt * 16 + 4 * G + r) * 16 + c];
-                        const float v = acc[0][dt][r] * mine;
-                        *slot = (w == 0) ? v : *slot + v;
-                    }
+                for (int dt = t0; dt < t0 + TP && dt < HDT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        s_o[(wave * TP + (dt - t0)) * 256 + (4 * G + r) * 16 + c] = acc[0][dt][r] * mine;
             }
             __syncthreads();
-        }
-        if (wave != 0 || !rvalid[0]) return;
-        bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[0]) * n_heads + rhead[0]) * HD + 4 * G;
-#pragma unroll
-        for (int dt = 0; dt < HDT; ++dt) {
-            const float* t = &s_o[(dt * 16 + 4 * G) * 16 + c];
-            uint2 wd;
-            wd.x = static_cast<uint32_t>(float_to_bf16_bits(t[0])) | (static_cast<uint32_t>(float_to_bf16_bits(t[16])) << 16);
-            wd.y = static_cast<uint32_t>(float_to_bf16_bits(t[32])) | (static_cast<uint32_t>(float_to_bf16_bits(t[48])) << 16);
-            *reinterpret_cast<uint2*>(o + dt * 16) = wd;
+            const int n_out = (min(TP, HDT - t0)) * 256;  // (d, row) places of this phase
+            for (int idx = threadIdx.x; idx < n_out; idx += n_threads) {  // idx % 16 == c
+                const int tile = idx >> 8, within = idx & 255;
+                float sum = 0.f;
+                for (int w = 0; w < n_active; ++w) sum += s_o[(w * TP + tile) * 256 + within];
+                if (rvalid[0]) {
+                    const int d = (t0 + tile) * 16 + (within >> 4);
+                    o[d] = from_float<bf16_t>(sum);
+                }
+            }
         }
         return;
     }

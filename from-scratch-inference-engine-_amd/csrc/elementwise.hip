@@ -144,16 +144,24 @@ void launch_rmsnorm(float* residual, const void* delta, const float* weight, voi
     }
 }
 
-// out[t, j] = silu(x[t, j]) * x[t, inter + j]; x is [T, 2*inter] (gate columns, then up).
+// out[t, j] = silu(x[t, 2j]) * x[t, 2j + 1]; x is [T, 2*inter] with gate and up interleaved.
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t total, int inter) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total) return;
-    const int64_t t = i / inter;
-    const int j = static_cast<int>(i - t * inter);
-    const float g = to_float(x[t * 2 * inter + j]);
-    const float u = to_float(x[t * 2 * inter + inter + j]);
+    const float g = to_float(x[2 * i]);
+    const float u = to_float(x[2 * i + 1]);
     out[i] = from_float<T>((g / (1.0f + expf(-g))) * u);
+}
+
+// four outputs per thread: 8 inputs in 16 (bfloat16) or 32 (float32) bytes
+template <typename T>
+__global__ void swiglu_vec_kernel(const T* __restrict__ x, T* __restrict__ out, int64_t quads) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= quads) return;
+    const float4 a = Pack4<T>::load(x + 8 * i), b = Pack4<T>::load(x + 8 * i + 4);
+    Pack4<T>::store(out + 4 * i, float4{(a.x / (1.0f + expf(-a.x))) * a.y, (a.z / (1.0f + expf(-a.z))) * a.w,
+                                        (b.x / (1.0f + expf(-b.x))) * b.y, (b.z / (1.0f + expf(-b.z))) * b.w});
 }
 
 template <typename T>
@@ -207,11 +215,15 @@ extern "C" int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, in
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "swiglu: unknown dtype %d", dtype);
     const int64_t total = static_cast<int64_t>(n_tokens) * inter;
     if (total == 0) return 0;
-    const unsigned grid = static_cast<unsigned>(ceil_div64(total, kThreads));
+    const bool vec = total % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    const int64_t work = vec ? total / 4 : total;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(work, kThreads));
     if (dtype == FSIE_F32) {
-        swiglu_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(out), total, inter);
+        if (vec) swiglu_vec_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(out), work);
+        else swiglu_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), static_cast<float*>(out), total, inter);
     } else {
-        swiglu_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(out), total, inter);
+        if (vec) swiglu_vec_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(out), work);
+        else swiglu_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(out), total, inter);
     }
     FSIE_CHECK_LAUNCH("swiglu");
     return 0;

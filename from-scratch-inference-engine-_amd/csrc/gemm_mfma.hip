@@ -25,7 +25,9 @@ constexpr int kStep = 32;  // k per MFMA
 
 // MT = tiles of 16 rows of X, NB = blocks of 16 rows of W per workgroup (they share the X
 // fragments), WAVES = waves of the workgroup, which split K.
-template <int MT, int NB, int WAVES, typename OutT>
+// SWIGLU: the rows of W are gate and up interleaved; the output has N/2 columns,
+// y[m, j] = silu(d[2j]) * d[2j + 1], computed in float32 from the accumulators.
+template <int MT, int NB, int WAVES, typename OutT, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
     OutT* __restrict__ y, int M, int N, int K) {
@@ -112,6 +114,17 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         for (int t = 0; t < MT; ++t) {
             const int m = t * 16 + row;
             if (m >= M) continue;
+            if (SWIGLU) {
+#pragma unroll
+                for (int r = 0; r < 4; r += 2) {
+                    const int nn = n0 + nb * 16 + kg * 4 + r;  // even: a gate row, nn + 1 its up row
+                    if (nn + 1 < N) {
+                        const float g = acc[nb][t][r], u = acc[nb][t][r + 1];
+                        y[static_cast<int64_t>(m) * (N / 2) + nn / 2] = from_float<OutT>((g / (1.0f + expf(-g))) * u);
+                    }
+                }
+                continue;
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int nn = n0 + nb * 16 + kg * 4 + r;
@@ -123,49 +136,49 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         }
 }
 
-template <int MT, int NB, int WAVES, typename OutT>
+template <int MT, int NB, int WAVES, typename OutT, bool SWIGLU>
 int launch(const void* x, const void* w, const float* bias, void* y, int M, int N, int K, hipStream_t stream) {
     const unsigned grid = static_cast<unsigned>((N + 16 * NB - 1) / (16 * NB));
-    gemm_mfma_skinny_kernel<MT, NB, WAVES, OutT><<<grid, WAVES * FSIE_WAVE, 0, stream>>>(
+    gemm_mfma_skinny_kernel<MT, NB, WAVES, OutT, SWIGLU><<<grid, WAVES * FSIE_WAVE, 0, stream>>>(
         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias, static_cast<OutT*>(y), M, N, K);
     FSIE_CHECK_LAUNCH("gemm_mfma_skinny");
     return 0;
 }
 
-template <int MT, int NB, typename OutT>
+template <int MT, int NB, typename OutT, bool SWIGLU>
 int launch_waves(int waves, const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
                  hipStream_t stream) {
     switch (waves) {
-        case 1: return launch<MT, NB, 1, OutT>(x, w, bias, y, M, N, K, stream);
-        case 2: return launch<MT, NB, 2, OutT>(x, w, bias, y, M, N, K, stream);
-        case 4: return launch<MT, NB, 4, OutT>(x, w, bias, y, M, N, K, stream);
-        case 8: return launch<MT, NB, 8, OutT>(x, w, bias, y, M, N, K, stream);
+        case 1: return launch<MT, NB, 1, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
+        case 2: return launch<MT, NB, 2, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
+        case 4: return launch<MT, NB, 4, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
+        case 8: return launch<MT, NB, 8, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
         default:
-            if constexpr (MT * NB <= 4) return launch<MT, NB, 16, OutT>(x, w, bias, y, M, N, K, stream);
-            return launch<MT, NB, 8, OutT>(x, w, bias, y, M, N, K, stream);
+            if constexpr (MT * NB <= 4) return launch<MT, NB, 16, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
+            return launch<MT, NB, 8, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
     }
 }
 
-template <int MT, typename OutT>
+template <int MT, typename OutT, bool SWIGLU>
 int launch_blocks(int nb, int waves, const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
                   hipStream_t stream) {
     switch (nb) {
-        case 1: return launch_waves<MT, 1, OutT>(waves, x, w, bias, y, M, N, K, stream);
-        case 2: return launch_waves<MT, 2, OutT>(waves, x, w, bias, y, M, N, K, stream);
+        case 1: return launch_waves<MT, 1, OutT, SWIGLU>(waves, x, w, bias, y, M, N, K, stream);
+        case 2: return launch_waves<MT, 2, OutT, SWIGLU>(waves, x, w, bias, y, M, N, K, stream);
         default:
-            if constexpr (MT <= 2) return launch_waves<MT, 4, OutT>(waves, x, w, bias, y, M, N, K, stream);
-            return launch_waves<MT, 2, OutT>(waves, x, w, bias, y, M, N, K, stream);
+            if constexpr (MT <= 2) return launch_waves<MT, 4, OutT, SWIGLU>(waves, x, w, bias, y, M, N, K, stream);
+            return launch_waves<MT, 2, OutT, SWIGLU>(waves, x, w, bias, y, M, N, K, stream);
     }
 }
 
-template <typename OutT>
+template <typename OutT, bool SWIGLU>
 int launch_tiles(int mt, int nb, int waves, const void* x, const void* w, const float* bias, void* y, int M, int N,
                  int K, hipStream_t stream) {
     switch (mt) {
-        case 1: return launch_blocks<1, OutT>(nb, waves, x, w, bias, y, M, N, K, stream);
-        case 2: return launch_blocks<2, OutT>(nb, waves, x, w, bias, y, M, N, K, stream);
-        case 3: return launch_blocks<3, OutT>(nb, waves, x, w, bias, y, M, N, K, stream);
-        default: return launch_blocks<4, OutT>(nb, waves, x, w, bias, y, M, N, K, stream);
+        case 1: return launch_blocks<1, OutT, SWIGLU>(nb, waves, x, w, bias, y, M, N, K, stream);
+        case 2: return launch_blocks<2, OutT, SWIGLU>(nb, waves, x, w, bias, y, M, N, K, stream);
+        case 3: return launch_blocks<3, OutT, SWIGLU>(nb, waves, x, w, bias, y, M, N, K, stream);
+        default: return launch_blocks<4, OutT, SWIGLU>(nb, waves, x, w, bias, y, M, N, K, stream);
     }
 }
 
@@ -173,8 +186,12 @@ int launch_tiles(int mt, int nb, int waves, const void* x, const void* w, const 
 
 // bfloat16 only.  M <= 64, K a multiple of 8, x and w 16-byte aligned.
 // waves (K split inside a workgroup) and blocks (16-row blocks of W per workgroup): 0 = choose.
+// epilogue: 0 = y = d (+ bias); 1 = SiLU*up over interleaved gate/up rows (N even, no bias, y is [M, N/2]).
 extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
-                                     int out_f32, int waves, int blocks, hipStream_t stream) {
+                                     int out_f32, int waves, int blocks, int epilogue, hipStream_t stream) {
+    FSIE_REQUIRE(epilogue == 0 || epilogue == 1, "gemm_mfma_skinny: unknown epilogue %d", epilogue);
+    FSIE_REQUIRE(epilogue == 0 || (N % 2 == 0 && !bias && !out_f32),
+                 "gemm_mfma_skinny: the SiLU*up epilogue needs an even N, no bias and a bfloat16 result");
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_skinny: at most %d rows, got %d",
                  FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
@@ -202,6 +219,7 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
         while (waves > 1 && pairs < 2 * waves) waves /= 2;
     }
     if (mt * blocks > 4 && waves > 8) waves = 8;  // LDS of the reduction
-    return out_f32 ? launch_tiles<float>(mt, blocks, waves, x, w, bias, y, M, N, K, stream)
-                   : launch_tiles<bf16_t>(mt, blocks, waves, x, w, bias, y, M, N, K, stream);
+    if (epilogue == 1) return launch_tiles<bf16_t, true>(mt, blocks, waves, x, w, bias, y, M, N, K, stream);
+    return out_f32 ? launch_tiles<float, false>(mt, blocks, waves, x, w, bias, y, M, N, K, stream)
+                   : launch_tiles<bf16_t, false>(mt, blocks, waves, x, w, bias, y, M, N, K, stream);
 }

@@ -13,43 +13,57 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kMaxHalf = 256;  // head_dim <= 512
 
+// angle = position * inv_freq in float64, as the plain formula has it, reduced in float64 to
+// [-pi, pi]; there float32 sine and cosine are within a few 1e-7 of the float64 ones.
+__device__ __forceinline__ void rotation(double pos, double inv_freq, float* c, float* s) {
+    const double ang = pos * inv_freq;
+    const double turns = rint(ang * 0.15915494309189535);  // 1 / (2 pi)
+    const double red = fma(-turns, 6.283185307179586, ang) - turns * 2.4492935982947064e-16;  // 2 pi = hi + lo
+    sincosf(static_cast<float>(red), s, c);
+}
+
+// No LDS and no barrier: every thread rotates whole pairs, and a pair of a k head goes to the row
+// and to its cache slot from the same registers; the values are copied in a loop of their own.
 template <typename T>
-__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
-                                     const int32_t* __restrict__ slots, const double* __restrict__ inv_freq,
-                                     const float* __restrict__ bias, T* __restrict__ k_pool, T* __restrict__ v_pool, int n_heads, int n_kv,
-                                     int head_dim, int rotary_half, int page_size, int write_kv,
-                                     int64_t pool_slots) {
-    __shared__ float cs[kMaxHalf];
-    __shared__ float sn[kMaxHalf];
+__global__ __launch_bounds__(kThreads) void rope_kv_write_kernel(
+    T* __restrict__ qkv, const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+    const double* __restrict__ inv_freq, const float* __restrict__ bias, T* __restrict__ k_pool,
+    T* __restrict__ v_pool, int n_heads, int n_kv, int head_dim, int rotary_half, int page_size, int write_kv,
+    int64_t pool_slots) {
     const int t = blockIdx.x;
     const int q_dim = n_heads * head_dim;
     const int kv_dim = n_kv * head_dim;
     T* row = qkv + static_cast<int64_t>(t) * (q_dim + 2 * kv_dim);
-
-    // angle = position * inv_freq in float64, as the plain formula has it, reduced in float64 to
-    // [-pi, pi]; there float32 sine and cosine are within a few 1e-7 of the float64 ones.
-    const double pos = static_cast<double>(positions[t]);
-    for (int i = threadIdx.x; i < rotary_half; i += blockDim.x) {
-        const double ang = pos * inv_freq[i];
-        const double turns = rint(ang * 0.15915494309189535);  // 1 / (2 pi)
-        const double red = fma(-turns, 6.283185307179586, ang) - turns * 2.4492935982947064e-16;  // 2 pi = hi + lo
-        float s, c;
-        sincosf(static_cast<float>(red), &s, &c);
-        cs[i] = c;
-        sn[i] = s;
-    }
-    __syncthreads();
-
-    const int slot = (write_kv && slots) ? slots[t] : -1;
+    int slot = (write_kv && slots) ? slots[t] : -1;
+    if (slot >= pool_slots) slot = -1;
     const int64_t page = slot >= 0 ? slot / page_size : 0;
     const int off = slot >= 0 ? slot % page_size : 0;
 
-    // q and k heads: add the bias, then rotate the pairs (i, i + rotary_half) of the first
-    // 2*rotary_half dimensions in place; the remaining dimensions only take the bias.
-    const int n_rot_heads = n_heads + n_kv;  // k heads follow the q heads directly in a row
+    // values first: their loads do not wait for the position
+    if (slot >= 0) {
+        const T* v = row + q_dim + kv_dim;
+        for (int idx = threadIdx.x; idx < kv_dim; idx += blockDim.x) {
+            const int kvh = idx / head_dim;
+            const int d = idx - kvh * head_dim;
+            const int64_t head = (page * n_kv + kvh) * page_size * head_dim;
+            v_pool[head + static_cast<int64_t>(d) * page_size + off] =
+                bias ? from_float<T>(to_float(v[idx]) + bias[q_dim + kv_dim + idx]) : v[idx];
+        }
+    }
+
+    // q and k heads (k heads follow the q heads directly in a row): add the bias, rotate the
+    // pairs (i, i + rotary_half) of the first 2*rotary_half dimensions
+    const double pos = static_cast<double>(positions[t]);
+    const int n_rot_heads = n_heads + n_kv;
+    int have_i = -1;
+    float c = 1.f, s = 0.f;
     for (int idx = threadIdx.x; idx < n_rot_heads * rotary_half; idx += blockDim.x) {
         const int h = idx / rotary_half;
         const int i = idx - h * rotary_half;
+        if (i != have_i) {  // the same for every turn of the loop when blockDim is a multiple of rotary_half
+            rotation(pos, inv_freq[i], &c, &s);
+            have_i = i;
+        }
         T* head = row + h * head_dim;
         float x1 = to_float(head[i]);
         float x2 = to_float(head[i + rotary_half]);
@@ -57,30 +71,27 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const int32_t* __restr
             x1 += bias[h * head_dim + i];
             x2 += bias[h * head_dim + i + rotary_half];
         }
-        const float c = cs[i], s = sn[i];
-        head[i] = from_float<T>(x1 * c - x2 * s);
-        head[i + rotary_half] = from_float<T>(x2 * c + x1 * s);
+        const T r1 = from_float<T>(x1 * c - x2 * s);
+        const T r2 = from_float<T>(x2 * c + x1 * s);
+        head[i] = r1;
+        head[i + rotary_half] = r2;
+        if (h >= n_heads && slot >= 0) {
+            T* dst = k_pool + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+            dst[i] = r1;
+            dst[i + rotary_half] = r2;
+        }
     }
+    // dimensions beyond the rotary ones only take the bias
     const int rest = head_dim - 2 * rotary_half;
-    if (bias && rest > 0) {
+    if (rest > 0) {
         for (int idx = threadIdx.x; idx < n_rot_heads * rest; idx += blockDim.x) {
             const int h = idx / rest;
             const int d = 2 * rotary_half + (idx - h * rest);
             T* head = row + h * head_dim;
-            head[d] = from_float<T>(to_float(head[d]) + bias[h * head_dim + d]);
+            const T v = bias ? from_float<T>(to_float(head[d]) + bias[h * head_dim + d]) : head[d];
+            head[d] = v;
+            if (h >= n_heads && slot >= 0) k_pool[((page * n_kv + (h - n_heads)) * page_size + off) * head_dim + d] = v;
         }
-    }
-    if (slot < 0 || slot >= pool_slots) return;  // uniform over the block
-    __syncthreads();  // the k written above is read back below by other threads
-    const T* k = row + q_dim;
-    const T* v = row + q_dim + kv_dim;
-    for (int idx = threadIdx.x; idx < kv_dim; idx += blockDim.x) {
-        const int kvh = idx / head_dim;
-        const int d = idx - kvh * head_dim;
-        const int64_t head = (page * n_kv + kvh) * page_size * head_dim;
-        k_pool[head + static_cast<int64_t>(off) * head_dim + d] = k[idx];
-        v_pool[head + static_cast<int64_t>(d) * page_size + off] =
-            bias ? from_float<T>(to_float(v[idx]) + bias[q_dim + kv_dim + idx]) : v[idx];
     }
 }
 

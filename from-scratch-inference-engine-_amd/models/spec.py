@@ -46,12 +46,12 @@ class ModelSpec:
 
 
 def bind(bindings: List[ParamBinding], owner: Part, attr: str, sources: Sequence[TensorSpec]) -> None:
-    """Declare that ``owner.attr`` is the concatenation (dim 0) of the checkpoint tensors
-    ``sources``; checks the shapes against the part's own declaration."""
+    """Declare that ``owner.attr`` is made of the checkpoint tensors ``sources`` (joined along
+    dim 0 the way the part's declaration says); checks the shapes against that declaration."""
     decl = owner.param_decls()[attr]
     rows = sum(s.shape[0] for s in sources)
     tail = tuple(sources[0].shape[1:])
     if any(tuple(s.shape[1:]) != tail for s in sources) or (rows, *tail) != tuple(decl.shape):
         raise ValueError(f"{type(owner).__name__}.{attr}: sources {[s.shape for s in sources]} do not "
                          f"make up {decl.shape}")
-    bindings.append(ParamBinding(owner, attr, list(sources), decl.storage))
+    bindings.append(ParamBinding(owner, attr, list(sources), decl.storage, decl.layout))

@@ -83,7 +83,7 @@ def rmsnorm(residual: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype:
 
 
 def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """silu(x[:, :I]) * x[:, I:] for x [T, 2I]."""
+    """silu(x[:, 0::2]) * x[:, 1::2] for x [T, 2I] (gate and up interleaved)."""
     _need(x, "swiglu input", ndim=2)
     t, two_i = x.shape
     if two_i % 2:
@@ -172,8 +172,10 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = N
 
 def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      out_dtype: Optional[torch.dtype] = None, waves: int = 0, blocks: int = 0,
-                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The same product on the matrix cores for bfloat16 and at most 64 rows (K a multiple of 8)."""
+                     out: Optional[torch.Tensor] = None, epilogue: str = "plain") -> torch.Tensor:
+    """The same product on the matrix cores for bfloat16 and at most 64 rows (K a multiple of 8).
+    ``epilogue="swiglu"``: the rows of ``weight`` are gate and up interleaved and the result is
+    silu(gate) * up, [M, N/2]."""
     _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
     _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
     m, k = x.shape
@@ -185,11 +187,17 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     out_dtype = out_dtype or x.dtype
     if out_dtype not in (torch.bfloat16, torch.float32):
         raise KernelError(f"gemm: output {out_dtype} is not offered")
+    if epilogue not in ("plain", "swiglu"):
+        raise KernelError(f"gemm: unknown epilogue '{epilogue}'")
+    if epilogue == "swiglu" and n % 2:
+        raise KernelError(f"gemm: the swiglu epilogue needs an even number of weight rows, found {n}")
+    n_out = n // 2 if epilogue == "swiglu" else n
     if out is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    _need(out, "gemm out", dtype=out_dtype, shape=(m, n))
+        out = torch.empty((m, n_out), dtype=out_dtype, device=x.device)
+    _need(out, "gemm out", dtype=out_dtype, shape=(m, n_out))
     check(load().fsie_gemm_mfma_skinny(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
-                                       int(out_dtype == torch.float32), waves, blocks, _stream()))
+                                       int(out_dtype == torch.float32), waves, blocks, int(epilogue == "swiglu"),
+                                       _stream()))
     return out
 
 

@@ -29,11 +29,14 @@ import torch
 @dataclass(frozen=True)
 class ParamDecl:
     """A parameter of a part.  ``storage``: 'matrix' (compute dtype), 'vector' (float32) or
-    'int_table' (int32).  ``init`` names the random-weights distribution."""
+    'int_table' (int32).  ``init`` names the random-weights distribution.  ``layout`` says how
+    several checkpoint tensors make up the parameter: 'concat' (one after the other along dim
+    0) or 'interleave' (row i of every source in turn: a0, b0, a1, b1, ...)."""
 
     shape: Tuple[int, ...]
     storage: str = "matrix"
     init: str = "weight"
+    layout: str = "concat"
 
 
 class HiddenState:

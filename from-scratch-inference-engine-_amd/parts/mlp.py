@@ -8,13 +8,16 @@ import torch
 
 from .. import ops
 from .base import FeedForward, ParamDecl, register_part
+from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M
 from .linear import Linear
 
 
 @register_part("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
     """down(silu(gate(x)) * up(x)), no biases (src/model/model.cpp:134-138).  gate and up are one
-    matrix [2I, H] (gate rows first), so x is read once."""
+    matrix [2I, H] with their rows interleaved (gate_0, up_0, gate_1, up_1, ...): x is read once,
+    and the lane that holds gate_j also holds up_j, so that for a few rows (decoding) SiLU*up
+    happens in the product's epilogue and the [T, 2I] intermediate never reaches memory."""
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size = hidden_size
@@ -23,7 +26,7 @@ class SwiGLU(FeedForward):
         self.down = Linear(intermediate_size, hidden_size)
 
     def param_decls(self) -> Dict[str, ParamDecl]:
-        return {"gate_up_weight": ParamDecl((2 * self.intermediate_size, self.hidden_size)),
+        return {"gate_up_weight": ParamDecl((2 * self.intermediate_size, self.hidden_size), layout="interleave"),
                 "down_weight": ParamDecl((self.hidden_size, self.intermediate_size))}
 
     @property
@@ -43,4 +46,8 @@ class SwiGLU(FeedForward):
         self.down.weight = t
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        return self.down(ops.swiglu(self.gate_up(x)))
+        if (x.dtype == torch.bfloat16 and x.shape[0] <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 8 == 0):
+            act = ops.gemm_mfma_skinny(x, self.gate_up.weight, epilogue="swiglu")
+        else:
+            act = ops.swiglu(self.gate_up(x))
+        return self.down(act)

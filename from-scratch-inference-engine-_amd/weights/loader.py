@@ -44,12 +44,14 @@ class TensorSpec:
 
 @dataclass
 class ParamBinding:
-    """Parameter ``attr`` of ``owner`` = concat(sources, dim 0), kept as ``storage``."""
+    """Parameter ``attr`` of ``owner`` = the sources joined along dim 0 ('concat': one after the
+    other; 'interleave': row i of every source in turn), kept as ``storage``."""
 
     owner: Any
     attr: str
     sources: Sequence[TensorSpec]
     storage: str = "matrix"  # matrix | vector | int_table
+    layout: str = "concat"   # concat | interleave
 
 
 def expected_tensors(bindings: Sequence[ParamBinding]) -> Dict[str, TensorSpec]:
@@ -102,7 +104,7 @@ def fill_parts(bindings: Sequence[ParamBinding], get_tensor, compute_dtype: torc
     shared: Dict[Tuple, torch.Tensor] = {}
     total = 0
     for b in bindings:
-        key = (tuple(s.name for s in b.sources), b.storage)
+        key = (tuple(s.name for s in b.sources), b.storage, b.layout)
         if key not in shared:
             target = _to_storage(None, b.storage, compute_dtype)
             pieces = []
@@ -111,7 +113,16 @@ def fill_parts(bindings: Sequence[ParamBinding], get_tensor, compute_dtype: torc
                 if b.storage == "int_table" and t.dtype.is_floating_point:
                     raise WeightsError(f"tensor {s.name} must hold integers, found {t.dtype}")
                 pieces.append(t.to(device=device, dtype=target, non_blocking=False))
-            value = pieces[0] if len(pieces) == 1 else torch.cat(pieces, dim=0)
+            if len(pieces) == 1:
+                value = pieces[0]
+            elif b.layout == "interleave":
+                if any(p.shape != pieces[0].shape for p in pieces):
+                    raise WeightsError(f"{b.attr}: interleaved sources must have equal shapes")
+                value = torch.stack(pieces, dim=1).reshape(-1, *pieces[0].shape[1:])
+            elif b.layout == "concat":
+                value = torch.cat(pieces, dim=0)
+            else:
+                raise ValueError(f"unknown layout '{b.layout}'")
             value = value.contiguous()
             shared[key] = value
             total += value.numel() * value.element_size()

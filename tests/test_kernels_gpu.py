@@ -61,10 +61,11 @@ def test_rmsnorm_alone_fused_and_rows(ops, dtype, hidden, eps):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_swiglu_and_adds(ops, dtype):
-    x = rnd((5, 2 * 4864), 4, dtype, 3.0)
-    ref = plain.silu_mul(x.float()[:, :4864], x.float()[:, 4864:])
-    out = ops.swiglu(x.cuda()).float().cpu()
-    assert (out - ref).abs().max() <= tol(dtype, ref)
+    for inter in (4864, 333):  # gate and up interleaved: (g0, u0, g1, u1, ...)
+        x = rnd((5, 2 * inter), 4, dtype, 3.0)
+        ref = plain.silu_mul(x.float()[:, 0::2], x.float()[:, 1::2])
+        out = ops.swiglu(x.cuda()).float().cpu()
+        assert (out - ref).abs().max() <= tol(dtype, ref)
     res, d = rnd((3, 333), 5), rnd((3, 333), 6, dtype)
     assert torch.equal(ops.residual_add(res.clone().cuda(), d.cuda()).cpu(), res + d.float())
     y, b = rnd((4, 77), 7, dtype), rnd((77,), 8)
@@ -130,6 +131,16 @@ def test_gemm_mfma_skinny(ops, m, n, k, waves):
     out = ops.gemm_mfma_skinny(x.cuda(), w.cuda(), None, waves=waves).float().cpu()
     ref = plain.linear(x.float(), w.float())
     assert (out - ref).abs().max() <= tol(torch.bfloat16, ref)
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 9728, 896), (8, 352, 64), (13, 640, 192), (16, 37888, 3584)])
+def test_gemm_mfma_skinny_with_swiglu_epilogue(ops, m, n, k):
+    x, w = rnd((m, k), 17, torch.bfloat16), rnd((n, k), 18, torch.bfloat16, 0.05)
+    full = plain.linear(x.float(), w.float())
+    ref = plain.silu_mul(full[:, 0::2], full[:, 1::2])
+    out = ops.gemm_mfma_skinny(x.cuda(), w.cuda(), epilogue="swiglu")
+    assert out.shape == (m, n // 2)
+    assert (out.float().cpu() - ref).abs().max() <= tol(torch.bfloat16, ref)
 
 
 def test_refusals(ops):

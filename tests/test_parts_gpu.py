@@ -58,9 +58,10 @@ def test_feed_forward_part(dtype):
     ffn = make_part("feed_forward", "swiglu", hidden_size=96, intermediate_size=200)
     assert ffn.param_decls()["gate_up_weight"].shape == (400, 96)
     gate, up, down = rnd((200, 96), 4, dtype, 0.1), rnd((200, 96), 5, dtype, 0.1), rnd((96, 200), 6, dtype, 0.1)
-    ffn.gate_up_weight = torch.cat([gate, up]).cuda()
+    assert ffn.param_decls()["gate_up_weight"].layout == "interleave"
+    ffn.gate_up_weight = torch.stack([gate, up], dim=1).reshape(400, 96).cuda()  # g0, u0, g1, u1, ...
     ffn.down_weight = down.cuda()
-    for rows in (3, 40):  # the small-matrix kernel and the library product
+    for rows in (3, 40):  # the small-matrix kernel with its fused epilogue, and the library product
         x = rnd((rows, 96), 7, dtype)
         out = ffn.forward(x.cuda(), Ctx(dtype)).float().cpu()
         ref = plain.linear(plain.silu_mul(plain.linear(x.float(), gate.float()), plain.linear(x.float(), up.float())), down.float())

@@ -106,7 +106,8 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
 
 def test_storage_kinds_and_fusion(tmp_path):
     """Matrices take the compute dtype, vectors stay float32 whatever the file stores, q/k/v
-    and gate/up are concatenated in that order, a tied head shares the embedding's memory."""
+    are concatenated in that order, gate/up are interleaved row by row, a tied head shares the
+    embedding's memory."""
     cfg = helpers.TINY_A
     tensors = helpers.random_tensors(cfg, 3, torch.float32)
     d = helpers.make_model_dir(tmp_path / "m", cfg, 3, tensors=tensors)
@@ -119,7 +120,8 @@ def test_storage_kinds_and_fusion(tmp_path):
         assert mixer.qkv_weight.dtype == dtype and torch.equal(mixer.qkv_weight, want)
         assert mixer.qkv_bias.dtype == torch.float32
         assert torch.equal(mixer.qkv_bias, torch.cat([tensors[p + f"self_attn.{n}_proj.bias"] for n in "qkv"]))
-        assert torch.equal(ffn.gate_up_weight, torch.cat([tensors[p + "mlp.gate_proj.weight"], tensors[p + "mlp.up_proj.weight"]]).to(dtype))
+        gate, up = tensors[p + "mlp.gate_proj.weight"].to(dtype), tensors[p + "mlp.up_proj.weight"].to(dtype)
+        assert torch.equal(ffn.gate_up_weight[0::2], gate) and torch.equal(ffn.gate_up_weight[1::2], up)  # interleaved
         assert spec.layers[0].mixer_norm.weight.dtype == torch.float32
         assert torch.equal(spec.final_norm.weight, tensors["model.norm.weight"])
         assert spec.lm_head.weight.data_ptr() == spec.embedding.weight.data_ptr()
