@@ -18,12 +18,12 @@ extern "C" int fsie_attention_mfma_max_waves(int head_dim) {
 extern "C" int fsie_attention_mfma_tiles(int head_dim, int large) {
     if (head_dim <= 0 || head_dim % 16 || head_dim > 256) return 0;
     if (!large) return 1;
-    return head_dim <= 128 ? 4 : 2;
+    return 2;
 }
 
 // bfloat16 only; head_dim a multiple of 16 up to 256; page_size a multiple of 4.
-// large = 0: items of at most 16 rows (tokens x heads of a group), `waves` waves of a workgroup split
-// each item's keys; large = 1: up to 16 * tiles rows, one wave per item.
+// large = 0: items of at most 16 rows (tokens x heads of a group); large = 1: up to 16 * tiles rows.
+// `waves` waves of a workgroup split each item's keys (at most 4 for large items).
 extern "C" int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                                    const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
                                    void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,
@@ -43,5 +43,5 @@ extern "C" int fsie_attention_mfma(const void* q, int64_t q_stride, const void* 
                            : hdt <= 12 ? fsie_attn::table_c(hdt, large) : fsie_attn::table_d(hdt, large);
     FSIE_REQUIRE(fn != nullptr, "attention_mfma: no kernel for head_dim %d", head_dim);
     return fn(q, q_stride, k_pool, v_pool, block_tables, max_pages, items, n_items, out, partials, n_heads, n_kv,
-              page_size, window, scale, large ? 1 : waves, stream);
+              page_size, window, scale, waves, stream);
 }

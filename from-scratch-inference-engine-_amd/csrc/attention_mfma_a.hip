@@ -6,10 +6,10 @@ namespace fsie_attn {
 
 LaunchFn table_a(int hdt, int large) {
     switch (hdt) {
-        case 1: return large ? launch<1, 4> : launch<1, 1>;
-        case 2: return large ? launch<2, 4> : launch<2, 1>;
-        case 3: return large ? launch<3, 4> : launch<3, 1>;
-        case 4: return large ? launch<4, 4> : launch<4, 1>;
+        case 1: return large ? launch<1, 2> : launch<1, 1>;
+        case 2: return large ? launch<2, 2> : launch<2, 1>;
+        case 3: return large ? launch<3, 2> : launch<3, 1>;
+        case 4: return large ? launch<4, 2> : launch<4, 1>;
         default: return nullptr;
     }
 }

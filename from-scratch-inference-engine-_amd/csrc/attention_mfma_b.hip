@@ -6,10 +6,10 @@ namespace fsie_attn {
 
 LaunchFn table_b(int hdt, int large) {
     switch (hdt) {
-        case 5: return large ? launch<5, 4> : launch<5, 1>;
-        case 6: return large ? launch<6, 4> : launch<6, 1>;
-        case 7: return large ? launch<7, 4> : launch<7, 1>;
-        case 8: return large ? launch<8, 4> : launch<8, 1>;
+        case 5: return large ? launch<5, 2> : launch<5, 1>;
+        case 6: return large ? launch<6, 2> : launch<6, 1>;
+        case 7: return large ? launch<7, 2> : launch<7, 1>;
+        case 8: return large ? launch<8, 2> : launch<8, 1>;
         default: return nullptr;
     }
 }

@@ -20,7 +20,7 @@
 // HDT = head_dim / 16, NT = column tiles of 16 query rows per wave (rows = tokens x heads of the
 // kv head's group).  Keys are walked in blocks of 32.  Requires page_size % 4 == 0.
 //
-// A workgroup may have several waves (NT = 1 only, up to MAXW): they split the item's key range
+// A workgroup may have several waves (up to MAXW; 4 when NT > 1): they split the item's key range
 // into contiguous runs of blocks, and their partial results are combined inside the workgroup:
 // maxima and sums through LDS, then the rescaled accumulators are added into one LDS tile in the
 // fixed order of the waves.  Decoding against a long context therefore needs neither partial
@@ -114,9 +114,9 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
         const bf16_t* qp = q + static_cast<int64_t>(q_row0 + (rvalid[nt] ? tq : 0)) * q_stride +
                            static_cast<int64_t>(rvalid[nt] ? rhead[nt] : h_base) * HD;
 #pragma unroll
-        for (int s = 0; s < S32; ++s) qf[nt][s].raw = rvalid[nt] ? ld16(qp + s * 32 + 8 * G) : uint4{0, 0, 0, 0};
+        for (int s = 0; s < S32; ++s) qf[nt][s].raw = ld16(qp + s * 32 + 8 * G);  // a row that does not exist reads
 #pragma unroll
-        for (int s = 0; s < S16; ++s) qt[nt][s].raw = rvalid[nt] ? ld8(qp + s * 16 + 4 * G) : uint2{0, 0};
+        for (int s = 0; s < S16; ++s) qt[nt][s].raw = ld8(qp + s * 16 + 4 * G);   // the item's first row: masked later
     }
 
     float m_run[NT], l_run[NT];
@@ -133,44 +133,67 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
     // this wave's run of key blocks
     const int kb_first = key_begin & ~31;
     const int n_blocks = (key_end - kb_first + 31) >> 5;
-    // an item uses one wave per 4 blocks (128 keys) of its own, however many the launch has:
-    // how its keys are split depends on the item alone
-    const int n_active = min(n_waves, max(1, (n_blocks + 3) >> 2));
+    // an item uses one wave per 4 blocks (128 keys) of its own when it has one query tile, per 16
+    // blocks (512 keys) when it has several, however many waves the launch has: how its keys are
+    // split depends on the item alone
+    constexpr int kBlocksPerWave = NT == 1 ? 4 : 16;
+    const int n_active = min(n_waves, max(1, (n_blocks + kBlocksPerWave - 1) / kBlocksPerWave));
     const int per_wave = (n_blocks + n_active - 1) / n_active;
     const int kb_begin = kb_first + wave * per_wave * 32;
     const int kb_end = min(key_end, kb_begin + per_wave * 32);
-    for (int kb = kb_begin; kb < kb_end; kb += 32) {
-        // ---- keys (A operand of the scores) and values (A operand of the second product)
+    // the keys (A operand of the scores) and values (A operand of the second product) of a block
+    struct Block {
         F16B kf[2][S32A];
         F8B kt[2][S16A];
         F8B vf[2][HDT];
+    };
+    // Where the four runs of a block's keys lie: the two tiles of 16 keys of the scores (one key
+    // per lane, c) and the two runs of 4 consecutive keys per lane group of the second product
+    // (never across a page: page_size % 4 == 0).  A key without a page (past the end, or behind a
+    // window) points at page 0: what is read there is finite and its probability is zero.
+    struct Where {
+        int64_t k[2], v[2];  // element offsets into the pools
+    };
+    auto locate = [&](int kb, Where& at) {
+        int page[4], idx[4], key[4];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int key = kb + t * 16 + c;
-            const int idx = key / page_size;
-            const int page = (key < key_end && idx < max_pages) ? table[idx] : -1;
-            const bool ok = page >= 0;
-            const bf16_t* kp = k_pool + (static_cast<int64_t>(ok ? page : 0) * n_kv + kvh) * head_stride +
-                               static_cast<int64_t>(key - idx * page_size) * HD;
+            key[t] = kb + t * 16 + c;
+            key[2 + t] = kb + t * 16 + 4 * G;
+        }
 #pragma unroll
-            for (int s = 0; s < S32; ++s) kf[t][s].raw = ok ? ld16(kp + s * 32 + 8 * G) : uint4{0, 0, 0, 0};
+        for (int i = 0; i < 4; ++i) {  // the four table reads go out together
+            idx[i] = key[i] / page_size;
+            page[i] = table[min(idx[i], max_pages - 1)];
+        }
 #pragma unroll
-            for (int s = 0; s < S16; ++s) kt[t][s].raw = ok ? ld8(kp + s * 16 + 4 * G) : uint2{0, 0};
+        for (int i = 0; i < 4; ++i) {
+            const bool ok = key[i] < key_end && idx[i] < max_pages && page[i] >= 0;
+            const int64_t head = (static_cast<int64_t>(ok ? page[i] : 0) * n_kv + kvh) * head_stride;
+            const int off = ok ? key[i] - idx[i] * page_size : 0;
+            if (i < 2) at.k[i] = head + static_cast<int64_t>(off) * HD + (X32 ? 8 : 4) * G;
+            else at.v[i - 2] = head + off + static_cast<int64_t>(c) * page_size;
+        }
+    };
+    auto load_block = [&](const Where& at, Block& blk) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const bf16_t* kp = k_pool + at.k[t];
+#pragma unroll
+            for (int s = 0; s < S32; ++s) blk.kf[t][s].raw = ld16(kp + s * 32);
+#pragma unroll
+            for (int s = 0; s < S16; ++s) blk.kt[t][s].raw = ld8(kp + s * 16);
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int key0 = kb + t * 16 + 4 * G;  // 4 consecutive keys, never across a page (page_size % 4 == 0)
-            const int idx = key0 / page_size;
-            const int page = (key0 < key_end && idx < max_pages) ? table[idx] : -1;
-            const bool ok = page >= 0;
-            const bf16_t* vp = v_pool + (static_cast<int64_t>(ok ? page : 0) * n_kv + kvh) * head_stride +
-                               (key0 - idx * page_size);
+            const bf16_t* vp = v_pool + at.v[t];
 #pragma unroll
-            for (int dt = 0; dt < HDT; ++dt) {
-                vf[t][dt].raw = ok ? ld8(vp + static_cast<int64_t>(dt * 16 + c) * page_size) : uint2{0, 0};
-            }
+            for (int dt = 0; dt < HDT; ++dt) blk.vf[t][dt].raw = ld8(vp + static_cast<int64_t>(dt * 16) * page_size);
         }
-
+    };
+    auto compute_block = [&](int kb, const Block& blk) {
+        const bool full = kb >= key_begin && kb + 32 <= key_end && kb + 31 <= pos0 &&
+                          (window <= 0 || kb > pos0 + n_q - 1 - window);  // the same for the whole wave
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             // ---- S^T for 32 keys x 16 rows
@@ -180,24 +203,34 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
                 st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int s = 0; s < S32; ++s)
-                    st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][s].v, qf[nt][s].v, st[t], 0, 0, 0);
+                    st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kf[t][s].v, qf[nt][s].v, st[t], 0, 0, 0);
 #pragma unroll
                 for (int s = 0; s < S16; ++s)
-                    st[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kt[t][s].v, qt[nt][s].v, st[t], 0, 0, 0);
+                    st[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.kt[t][s].v, qt[nt][s].v, st[t], 0, 0, 0);
             }
-            // ---- mask, running maximum
+            // ---- mask, running maximum.  A block that every row of the item sees whole (below
+            // the diagonal, inside the key range and the window) needs no mask; in a long
+            // portion that is nearly every block.
             float sv[8];
             float m_loc = -INFINITY;
+            if (full) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int key = kb + t * 16 + 4 * G + r;
-                    const bool vis = rvalid[nt] && key >= key_begin && key < key_end && key <= rpos[nt] &&
-                                     (window <= 0 || key > rpos[nt] - window);
-                    sv[t * 4 + r] = vis ? st[t][r] * scale2 : -INFINITY;
-                    m_loc = fmaxf(m_loc, sv[t * 4 + r]);
+                for (int i = 0; i < 8; ++i) {
+                    sv[i] = st[i >> 2][i & 3] * scale2;
+                    m_loc = fmaxf(m_loc, sv[i]);
                 }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int key = kb + t * 16 + 4 * G + r;
+                        const bool vis = rvalid[nt] && key >= key_begin && key < key_end && key <= rpos[nt] &&
+                                         (window <= 0 || key > rpos[nt] - window);
+                        sv[t * 4 + r] = vis ? st[t][r] * scale2 : -INFINITY;
+                        m_loc = fmaxf(m_loc, sv[t * 4 + r]);
+                    }
+            }
             m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16, FSIE_WAVE));
             m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32, FSIE_WAVE));
             const float m_new = fmaxf(m_run[nt], m_loc);
@@ -214,73 +247,114 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
             F8B pb[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                pb[t].raw.x = static_cast<uint32_t>(float_to_bf16_bits(p[t * 4 + 0])) |
-                              (static_cast<uint32_t>(float_to_bf16_bits(p[t * 4 + 1])) << 16);
-                pb[t].raw.y = static_cast<uint32_t>(float_to_bf16_bits(p[t * 4 + 2])) |
-                              (static_cast<uint32_t>(float_to_bf16_bits(p[t * 4 + 3])) << 16);
+                pb[t].raw.x = pack2_bf16(p[t * 4 + 0], p[t * 4 + 1]);
+                pb[t].raw.y = pack2_bf16(p[t * 4 + 2], p[t * 4 + 3]);
+            }
+            // the accumulators shrink only when some row's maximum moved (rare after the first blocks)
+            if (__any(corr != 1.f)) {
+#pragma unroll
+                for (int dt = 0; dt < HDT; ++dt) {
+                    acc[nt][dt][0] *= corr;
+                    acc[nt][dt][1] *= corr;
+                    acc[nt][dt][2] *= corr;
+                    acc[nt][dt][3] *= corr;
+                }
             }
             // ---- O^T += V^T P^T
 #pragma unroll
             for (int dt = 0; dt < HDT; ++dt) {
                 floatx4 a = acc[nt][dt];
-                a[0] *= corr;
-                a[1] *= corr;
-                a[2] *= corr;
-                a[3] *= corr;
-                a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[0][dt].v, pb[0].v, a, 0, 0, 0);
-                a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[1][dt].v, pb[1].v, a, 0, 0, 0);
+                a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.vf[0][dt].v, pb[0].v, a, 0, 0, 0);
+                a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.vf[1][dt].v, pb[1].v, a, 0, 0, 0);
                 acc[nt][dt] = a;
+            }
+        }
+    };
+    // The table reads of a block go out one block ahead, so that its data reads never wait for
+    // an address.  One query tile and a moderate head size leave registers for a second block:
+    // its data is in flight while the matrix cores work on the present one (few waves run here,
+    // so occupancy does not hide the latency).
+    constexpr bool PREFETCH = NT == 1 && HDT <= 8;
+    if (kb_begin < kb_end) {
+        Where at;
+        locate(kb_begin, at);
+        if (PREFETCH) {
+            Block cur, nxt;
+            load_block(at, cur);
+            locate(kb_begin + 32, at);
+            for (int kb = kb_begin; kb < kb_end; kb += 32) {
+                if (kb + 32 < kb_end) {
+                    load_block(at, nxt);
+                    locate(kb + 64, at);
+                }
+                compute_block(kb, cur);
+                cur = nxt;
+            }
+        } else {
+            for (int kb = kb_begin; kb < kb_end; kb += 32) {
+                Block blk;
+                load_block(at, blk);
+                locate(kb + 32, at);
+                compute_block(kb, blk);
             }
         }
     }
 
-    // ---- several waves: combine inside the workgroup (NT == 1)
-    if (MAXW > 1 && NT == 1 && n_waves > 1) {
-        constexpr int kSlabFloats = 8192;              // 32 KB of LDS for the accumulators
-        constexpr int TP = kSlabFloats / (MAXW * 256); // head-dim tiles per phase (>= 1 for MAXW <= 16... 32)
-        __shared__ float s_m[MAXW][16], s_l[MAXW][16];
+    // ---- several waves: combine inside the workgroup
+    if (MAXW > 1 && n_waves > 1) {
+        constexpr int kSlabFloats = 8192;               // 32 KB of LDS for the accumulators
+        constexpr int TP = kSlabFloats / (MAXW * 256);  // head-dim tiles per phase
+        __shared__ float s_m[NT][MAXW][16], s_l[NT][MAXW][16];
         __shared__ float s_o[kSlabFloats];
-        float l_w = l_run[0];
-        l_w += __shfl_xor(l_w, 16, FSIE_WAVE);
-        l_w += __shfl_xor(l_w, 32, FSIE_WAVE);
-        if (G == 0) {
-            s_m[wave][c] = m_run[0];
-            s_l[wave][c] = l_w;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            float l_w = l_run[nt];
+            l_w += __shfl_xor(l_w, 16, FSIE_WAVE);
+            l_w += __shfl_xor(l_w, 32, FSIE_WAVE);
+            if (G == 0) {
+                s_m[nt][wave][c] = m_run[nt];
+                s_l[nt][wave][c] = l_w;
+            }
         }
         __syncthreads();
-        float m_all = -INFINITY;
-        for (int w = 0; w < n_active; ++w) m_all = fmaxf(m_all, s_m[w][c]);
-        float denom = 0.f;
-        for (int w = 0; w < n_active; ++w) {
-            const float mw = s_m[w][c];
-            if (mw != -INFINITY) denom += s_l[w][c] * __builtin_amdgcn_exp2f(mw - m_all);
-        }
-        const float mine = (m_run[0] == -INFINITY || !(denom > 0.f)) ? 0.f
-                           : __builtin_amdgcn_exp2f(m_run[0] - m_all) / denom;
-        // Each active wave lays its rescaled accumulators into a slab of its own, TP tiles of the
-        // head dimension at a time; then every thread sums the slabs for a few (d, row) places
-        // of its own column in the fixed order of the waves and writes them out.
-        bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[0]) * n_heads + rhead[0]) * HD;
         const int n_threads = 64 * n_waves;
+        bool first = true;
 #pragma unroll
-        for (int t0 = 0; t0 < HDT; t0 += TP) {
-            if (t0 > 0) __syncthreads();  // the slabs of the last phase have been read
-            if (wave < n_active) {
-#pragma unroll
-                for (int dt = t0; dt < t0 + TP && dt < HDT; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        s_o[(wave * TP + (dt - t0)) * 256 + (4 * G + r) * 16 + c] = acc[0][dt][r] * mine;
+        for (int nt = 0; nt < NT; ++nt) {
+            float m_all = -INFINITY;
+            for (int w = 0; w < n_active; ++w) m_all = fmaxf(m_all, s_m[nt][w][c]);
+            float denom = 0.f;
+            for (int w = 0; w < n_active; ++w) {
+                const float mw = s_m[nt][w][c];
+                if (mw != -INFINITY) denom += s_l[nt][w][c] * __builtin_amdgcn_exp2f(mw - m_all);
             }
-            __syncthreads();
-            const int n_out = (min(TP, HDT - t0)) * 256;  // (d, row) places of this phase
-            for (int idx = threadIdx.x; idx < n_out; idx += n_threads) {  // idx % 16 == c
-                const int tile = idx >> 8, within = idx & 255;
-                float sum = 0.f;
-                for (int w = 0; w < n_active; ++w) sum += s_o[(w * TP + tile) * 256 + within];
-                if (rvalid[0]) {
-                    const int d = (t0 + tile) * 16 + (within >> 4);
-                    o[d] = from_float<bf16_t>(sum);
+            const float mine = (m_run[nt] == -INFINITY || !(denom > 0.f)) ? 0.f
+                               : __builtin_amdgcn_exp2f(m_run[nt] - m_all) / denom;
+            // Each active wave lays its rescaled accumulators into a slab of its own, TP tiles of
+            // the head dimension at a time; then every thread sums the slabs for a few (d, row)
+            // places of its own column in the fixed order of the waves and writes them out.
+            bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[nt]) * n_heads + rhead[nt]) * HD;
+#pragma unroll
+            for (int t0 = 0; t0 < HDT; t0 += TP) {
+                if (!first) __syncthreads();  // the slabs of the last phase have been read
+                first = false;
+                if (wave < n_active) {
+#pragma unroll
+                    for (int dt = t0; dt < t0 + TP && dt < HDT; ++dt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            s_o[(wave * TP + (dt - t0)) * 256 + (4 * G + r) * 16 + c] = acc[nt][dt][r] * mine;
+                }
+                __syncthreads();
+                const int n_out = (min(TP, HDT - t0)) * 256;  // (d, row) places of this phase
+                for (int idx = threadIdx.x; idx < n_out; idx += n_threads) {  // idx % 16 == c
+                    const int tile = idx >> 8, within = idx & 255;
+                    float sum = 0.f;
+                    for (int w = 0; w < n_active; ++w) sum += s_o[(w * TP + tile) * 256 + within];
+                    if (rvalid[nt]) {
+                        const int d = (t0 + tile) * 16 + (within >> 4);
+                        o[d] = from_float<bf16_t>(sum);
+                    }
                 }
             }
         }
@@ -300,10 +374,8 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
 #pragma unroll
             for (int dt = 0; dt < HDT; ++dt) {
                 uint2 w;
-                w.x = static_cast<uint32_t>(float_to_bf16_bits(acc[nt][dt][0] * inv)) |
-                      (static_cast<uint32_t>(float_to_bf16_bits(acc[nt][dt][1] * inv)) << 16);
-                w.y = static_cast<uint32_t>(float_to_bf16_bits(acc[nt][dt][2] * inv)) |
-                      (static_cast<uint32_t>(float_to_bf16_bits(acc[nt][dt][3] * inv)) << 16);
+                w.x = pack2_bf16(acc[nt][dt][0] * inv, acc[nt][dt][1] * inv);
+                w.y = pack2_bf16(acc[nt][dt][2] * inv, acc[nt][dt][3] * inv);
                 *reinterpret_cast<uint2*>(o + dt * 16) = w;
             }
         } else {
@@ -324,7 +396,7 @@ template <int HDT, int NT>
 int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool, const int32_t* block_tables,
            int max_pages, const int32_t* items, int n_items, void* out, float* partials, int n_heads, int n_kv,
            int page_size, int window, float scale, int waves, hipStream_t stream) {
-    constexpr int MAXW = NT == 1 ? max_waves<HDT>() : 1;
+    constexpr int MAXW = NT == 1 ? max_waves<HDT>() : 4;
     const int group = n_heads / n_kv;
     const int rows = 16 * NT;
     const int gh = group < rows ? group : rows;

@@ -25,6 +25,16 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
     return static_cast<uint16_t>(u >> 16);
 }
 
+// Two floats to two bfloat16 in one register (low half first), round to nearest even: one
+// v_cvt_pk_bf16_f32 on gfx950.
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float floatx2_t __attribute__((ext_vector_type(2)));
+    const floatx2_t v = {lo, hi};
+    const bf16x2_t b = __builtin_convertvector(v, bf16x2_t);
+    return *reinterpret_cast<const uint32_t*>(&b);
+}
+
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(bf16_t v) { return bf16_bits_to_float(v.bits); }
 

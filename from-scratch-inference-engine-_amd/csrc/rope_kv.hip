@@ -55,30 +55,48 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_kernel(
     // pairs (i, i + rotary_half) of the first 2*rotary_half dimensions
     const double pos = static_cast<double>(positions[t]);
     const int n_rot_heads = n_heads + n_kv;
+    const int n_pairs = n_rot_heads * rotary_half;
     int have_i = -1;
     float c = 1.f, s = 0.f;
-    for (int idx = threadIdx.x; idx < n_rot_heads * rotary_half; idx += blockDim.x) {
-        const int h = idx / rotary_half;
-        const int i = idx - h * rotary_half;
-        if (i != have_i) {  // the same for every turn of the loop when blockDim is a multiple of rotary_half
-            rotation(pos, inv_freq[i], &c, &s);
-            have_i = i;
+    constexpr int PB = 8;  // pairs in flight per thread: all loads of a batch are issued before its stores
+    for (int base = threadIdx.x; base < n_pairs; base += blockDim.x * PB) {
+        float x1[PB], x2[PB];
+#pragma unroll
+        for (int u = 0; u < PB; ++u) {
+            const int idx = base + u * blockDim.x;
+            x1[u] = x2[u] = 0.f;
+            if (idx < n_pairs) {
+                const int h = idx / rotary_half;
+                const int i = idx - h * rotary_half;
+                const T* head = row + h * head_dim;
+                x1[u] = to_float(head[i]);
+                x2[u] = to_float(head[i + rotary_half]);
+                if (bias) {
+                    x1[u] += bias[h * head_dim + i];
+                    x2[u] += bias[h * head_dim + i + rotary_half];
+                }
+            }
         }
-        T* head = row + h * head_dim;
-        float x1 = to_float(head[i]);
-        float x2 = to_float(head[i + rotary_half]);
-        if (bias) {
-            x1 += bias[h * head_dim + i];
-            x2 += bias[h * head_dim + i + rotary_half];
-        }
-        const T r1 = from_float<T>(x1 * c - x2 * s);
-        const T r2 = from_float<T>(x2 * c + x1 * s);
-        head[i] = r1;
-        head[i + rotary_half] = r2;
-        if (h >= n_heads && slot >= 0) {
-            T* dst = k_pool + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
-            dst[i] = r1;
-            dst[i + rotary_half] = r2;
+#pragma unroll
+        for (int u = 0; u < PB; ++u) {
+            const int idx = base + u * blockDim.x;
+            if (idx >= n_pairs) continue;
+            const int h = idx / rotary_half;
+            const int i = idx - h * rotary_half;
+            if (i != have_i) {  // the same for the whole loop when blockDim is a multiple of rotary_half
+                rotation(pos, inv_freq[i], &c, &s);
+                have_i = i;
+            }
+            const T r1 = from_float<T>(x1[u] * c - x2[u] * s);
+            const T r2 = from_float<T>(x2[u] * c + x1[u] * s);
+            T* head = row + h * head_dim;
+            head[i] = r1;
+            head[i + rotary_half] = r2;
+            if (h >= n_heads && slot >= 0) {
+                T* dst = k_pool + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+                dst[i] = r1;
+                dst[i + rotary_half] = r2;
+            }
         }
     }
     // dimensions beyond the rotary ones only take the bias

@@ -255,8 +255,7 @@ def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
                    window: Optional[int], scale: float, n_query_rows: int, large: bool, waves: int = 1) -> torch.Tensor:
     """Attention of the work items over the paged cache on the matrix cores (bfloat16; head_dim a
     multiple of 16; page size a multiple of 4).  ``items`` may be a view into a longer table.
-    Small items (``large=False``) are worked on by ``waves`` waves of a workgroup that split the
-    keys and combine inside the workgroup."""
+    ``waves`` waves of a workgroup split each item's keys and combine inside the workgroup."""
     if not q.is_cuda or q.dtype != torch.bfloat16:
         raise KernelError("attention_mfma q: must be bfloat16 on the GPU")
     _need(k_pool, "k_pool", dtype=q.dtype, ndim=4)

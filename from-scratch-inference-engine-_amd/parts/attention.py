@@ -33,6 +33,11 @@ class AttentionPlanner:
     a multiple of 4) and the float32-arithmetic kernel for everything else; which one a step
     uses follows from the step's dtype and page size."""
 
+    # Keys above which a large tile is given four waves that split its keys.  Off: on MI355X a
+    # 2,048-token prefill at 28/4 heads of 128 took 235 us per layer with 512 against 176 us
+    # without (idle waves in the four-wave workgroups cost more than the balance gains).
+    long_keys: Optional[int] = None
+
     def __init__(self, n_heads: int, n_kv: int, head_dim: int, window: Optional[int]):
         self.n_heads, self.n_kv, self.head_dim, self.window = n_heads, n_kv, head_dim, window
         self.key = ("attention", n_heads, n_kv, head_dim, window)
@@ -122,11 +127,17 @@ class AttentionPlanner:
                 merged = {m[0] for m in merges}
                 merges += [(row, 0, 0, 0) for row in range(host.n_tokens) if row not in merged]
                 n_partial = n_items * small_tokens
+        n_long = 0
+        if mfma and self.long_keys is not None:
+            # large tiles that read more than ``long_keys`` keys go to workgroups of four waves
+            long_ones = [it for it in large if it[5] - it[4] > self.long_keys]
+            large = [it for it in large if it[5] - it[4] <= self.long_keys] + long_ones
+            n_long = len(long_ones)
         return {
             "items": np.asarray(small + large, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS),
             "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
-            "n_small": len(small), "n_large": len(large), "n_merges": len(merges), "n_partial": n_partial,
-            "mfma": mfma, "waves": waves,
+            "n_small": len(small), "n_large": len(large) - n_long, "n_long": n_long, "n_merges": len(merges),
+            "n_partial": n_partial, "mfma": mfma, "waves": waves,
         }
 
 
@@ -198,6 +209,10 @@ class GQAttention(Mixer):
             if plan.n_large:
                 ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
                                    plan.items[plan.n_small:], plan.n_large, out, *args, large=True)
+            if plan.n_long:
+                ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
+                                   plan.items[plan.n_small + plan.n_large:], plan.n_long, out, *args, large=True,
+                                   waves=4)
         else:
             ops.attention_scalar(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
                                  plan.n_small + plan.n_large, out, *args)

@@ -225,6 +225,9 @@ def run_attention(ops, case, heads, kv, hd, window=None):
             ops.attention_mfma(q, heads * hd, *pools, items, plan["n_small"], *common, large=False, waves=plan["waves"])
         if plan["n_large"]:
             ops.attention_mfma(q, heads * hd, *pools, items[plan["n_small"]:], plan["n_large"], *common, large=True)
+        if plan["n_long"]:
+            ops.attention_mfma(q, heads * hd, *pools, items[plan["n_small"] + plan["n_large"]:], plan["n_long"], *common,
+                               large=True, waves=4)
     else:
         ops.attention_scalar(q, heads * hd, *pools, items, plan["n_small"] + plan["n_large"], *common)
     if plan["n_merges"]:
@@ -245,7 +248,7 @@ def run_attention(ops, case, heads, kv, hd, window=None):
 def test_attention_over_pages(ops, dtype, scalar, heads, kv, hd, page, window):
     # (past, new): the reference's (7, 5) and (19, 1), a long decode that is split, whole prompts,
     # portions starting mid-page, a two-token portion
-    seqs = [(7, 5), (19, 1), (600, 1), (0, 33), (300, 2), (123, 70), (0, 1), (40, 200), (2500, 1)]
+    seqs = [(7, 5), (19, 1), (600, 1), (0, 33), (300, 2), (123, 70), (0, 1), (40, 200), (2500, 1), (900, 130)]
     case = paged_case(seqs, heads, kv, hd, page, dtype, seed=hd + heads, window=window, scalar=scalar)
     assert case["plan"]["mfma"] == (not scalar)
     out = run_attention(ops, case, heads, kv, hd, window)
@@ -299,6 +302,23 @@ def test_attention_finds_one_far_key_and_respects_edges(ops, dtype, scalar):
                 if i == 0:
                     assert (ref[i] - want).abs().max() < 1e-3
             row += n
+
+
+def test_attention_long_tiles_on_four_waves(ops, monkeypatch):
+    """Large tiles may be given four waves that split the keys and merge in the workgroup."""
+    from from_scratch_inference_engine_amd.parts.attention import AttentionPlanner
+
+    monkeypatch.setattr(AttentionPlanner, "long_keys", 96)
+    heads, kv, hd, page = 8, 2, 64, 8
+    seqs = [(500, 70), (0, 300), (37, 3)]
+    case = paged_case(seqs, heads, kv, hd, page, torch.bfloat16, seed=9)
+    assert case["plan"]["n_long"] > 0 and case["plan"]["n_large"] > 0
+    out = run_attention(ops, case, heads, kv, hd)
+    row = 0
+    for (p, n), q, k, v in zip(seqs, case["qs"], case["ks"], case["vs"]):
+        ref = plain.attention(q, k, v, heads, kv, hd, query_offset=p)
+        assert (out[row:row + n] - ref).abs().max() <= 2.0 ** -7 * ref.abs().max()
+        row += n
 
 
 def test_attention_does_not_depend_on_page_ids(ops):
