@@ -79,32 +79,50 @@ struct Pack4<bf16_t> {
     }
 };
 
-template <typename T, int ITERS>
+// four elements per thread, grid = (tokens, quads / threads): no loop, one load per thread
+template <typename T>
+__global__ void embedding_vec_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
+                                     float* __restrict__ out, int hidden, int vocab) {
+    const int t = blockIdx.x;
+    const int j = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+    if (j >= hidden) return;
+    const int id = ids[t];
+    const bool ok = id >= 0 && id < vocab;
+    const float4 v = Pack4<T>::load(table + static_cast<int64_t>(ok ? id : 0) * hidden + j);
+    Pack4<float>::store(out + static_cast<int64_t>(t) * hidden + j, ok ? v : float4{0.f, 0.f, 0.f, 0.f});
+}
+
+template <typename T, int ITERS, bool HAS_DELTA, bool WRITE_BACK>
 __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta,
                                                                const float* __restrict__ weight, T* __restrict__ out,
-                                                               const int32_t* __restrict__ rows, int hidden, float eps,
-                                                               int write_back) {
+                                                               const int32_t* __restrict__ rows, int hidden, float eps) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int64_t row = rows ? rows[r] : r;
     float* res = residual + row * hidden;
-    const T* del = delta ? delta + row * hidden : nullptr;
-    float4 v[ITERS];
+    const T* del = HAS_DELTA ? delta + row * hidden : nullptr;
+    // every load of the row goes out before anything waits: places past the end read the last
+    // quad again and are masked out of the sum and the stores
+    float4 v[ITERS], d[ITERS], w[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int j = min((it * kThreads + static_cast<int>(threadIdx.x)) * 4, hidden - 4);
+        v[it] = Pack4<float>::load(res + j);
+        if (HAS_DELTA) d[it] = Pack4<T>::load(del + j);
+        w[it] = Pack4<float>::load(weight + j);
+    }
     float sum_sq = 0.f;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int j = (it * kThreads + threadIdx.x) * 4;
-        v[it] = float4{0.f, 0.f, 0.f, 0.f};
+        if (HAS_DELTA) {
+            v[it].x += d[it].x;
+            v[it].y += d[it].y;
+            v[it].z += d[it].z;
+            v[it].w += d[it].w;
+        }
         if (j < hidden) {
-            v[it] = Pack4<float>::load(res + j);
-            if (del) {
-                const float4 d = Pack4<T>::load(del + j);
-                v[it].x += d.x;
-                v[it].y += d.y;
-                v[it].z += d.z;
-                v[it].w += d.w;
-            }
-            if (write_back) Pack4<float>::store(res + j, v[it]);
+            if (WRITE_BACK) Pack4<float>::store(res + j, v[it]);
             sum_sq += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
         }
     }
@@ -115,10 +133,21 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict
     for (int it = 0; it < ITERS; ++it) {
         const int j = (it * kThreads + threadIdx.x) * 4;
         if (j < hidden) {
-            const float4 w = Pack4<float>::load(weight + j);
-            Pack4<T>::store(dst + j, float4{(v[it].x * scale) * w.x, (v[it].y * scale) * w.y, (v[it].z * scale) * w.z,
-                                            (v[it].w * scale) * w.w});
+            Pack4<T>::store(dst + j, float4{(v[it].x * scale) * w[it].x, (v[it].y * scale) * w[it].y,
+                                            (v[it].z * scale) * w[it].z, (v[it].w * scale) * w[it].w});
         }
+    }
+}
+
+template <typename T, int ITERS>
+void launch_rmsnorm_vec(float* residual, const T* d, const float* weight, T* o, const int32_t* rows, int n_rows,
+                        int hidden, float eps, int write_back, hipStream_t stream) {
+    if (!d) {
+        rmsnorm_vec_kernel<T, ITERS, false, false><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps);
+    } else if (write_back) {
+        rmsnorm_vec_kernel<T, ITERS, true, true><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps);
+    } else {
+        rmsnorm_vec_kernel<T, ITERS, true, false><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps);
     }
 }
 
@@ -131,14 +160,14 @@ void launch_rmsnorm(float* residual, const void* delta, const float* weight, voi
                          reinterpret_cast<uintptr_t>(weight) % 16 == 0 && reinterpret_cast<uintptr_t>(delta) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(out) % 16 == 0;
     const int per_iter = kThreads * 4;
-    if (aligned && hidden <= per_iter) {
-        rmsnorm_vec_kernel<T, 1><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
-    } else if (aligned && hidden <= 2 * per_iter) {
-        rmsnorm_vec_kernel<T, 2><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
-    } else if (aligned && hidden <= 4 * per_iter) {
-        rmsnorm_vec_kernel<T, 4><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
-    } else if (aligned && hidden <= 8 * per_iter) {
-        rmsnorm_vec_kernel<T, 8><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
+    if (aligned && hidden >= 4 && hidden <= per_iter) {
+        launch_rmsnorm_vec<T, 1>(residual, d, weight, o, rows, n_rows, hidden, eps, write_back, stream);
+    } else if (aligned && hidden <= 2 * per_iter && hidden >= 4) {
+        launch_rmsnorm_vec<T, 2>(residual, d, weight, o, rows, n_rows, hidden, eps, write_back, stream);
+    } else if (aligned && hidden <= 4 * per_iter && hidden >= 4) {
+        launch_rmsnorm_vec<T, 4>(residual, d, weight, o, rows, n_rows, hidden, eps, write_back, stream);
+    } else if (aligned && hidden <= 8 * per_iter && hidden >= 4) {
+        launch_rmsnorm_vec<T, 8>(residual, d, weight, o, rows, n_rows, hidden, eps, write_back, stream);
     } else {
         rmsnorm_kernel<T><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
     }
@@ -184,10 +213,14 @@ extern "C" int fsie_embedding(const void* table, int dtype, const int32_t* ids, 
                  n_tokens, hidden, vocab);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "embedding: unknown dtype %d", dtype);
     if (n_tokens == 0) return 0;
+    const bool vec = hidden % 4 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    const dim3 vgrid(n_tokens, static_cast<unsigned>(ceil_div64(hidden / 4, kThreads)));
     if (dtype == FSIE_F32) {
-        embedding_kernel<float><<<n_tokens, kThreads, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab);
+        if (vec) embedding_vec_kernel<float><<<vgrid, kThreads, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab);
+        else embedding_kernel<float><<<n_tokens, kThreads, 0, stream>>>(static_cast<const float*>(table), ids, out, hidden, vocab);
     } else {
-        embedding_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, hidden, vocab);
+        if (vec) embedding_vec_kernel<bf16_t><<<vgrid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, hidden, vocab);
+        else embedding_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(static_cast<const bf16_t*>(table), ids, out, hidden, vocab);
     }
     FSIE_CHECK_LAUNCH("embedding");
     return 0;

@@ -24,7 +24,7 @@ __device__ __forceinline__ void rotation(double pos, double inv_freq, float* c, 
 
 // No LDS and no barrier: every thread rotates whole pairs, and a pair of a k head goes to the row
 // and to its cache slot from the same registers; the values are copied in a loop of their own.
-template <typename T>
+template <typename T, bool HAS_BIAS>
 __global__ __launch_bounds__(kThreads) void rope_kv_write_kernel(
     T* __restrict__ qkv, const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
     const double* __restrict__ inv_freq, const float* __restrict__ bias, T* __restrict__ k_pool,
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_kernel(
             const int d = idx - kvh * head_dim;
             const int64_t head = (page * n_kv + kvh) * page_size * head_dim;
             v_pool[head + static_cast<int64_t>(d) * page_size + off] =
-                bias ? from_float<T>(to_float(v[idx]) + bias[q_dim + kv_dim + idx]) : v[idx];
+                HAS_BIAS ? from_float<T>(to_float(v[idx]) + bias[q_dim + kv_dim + idx]) : v[idx];
         }
     }
 
@@ -56,39 +56,38 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_kernel(
     const double pos = static_cast<double>(positions[t]);
     const int n_rot_heads = n_heads + n_kv;
     const int n_pairs = n_rot_heads * rotary_half;
-    int have_i = -1;
-    float c = 1.f, s = 0.f;
-    constexpr int PB = 8;  // pairs in flight per thread: all loads of a batch are issued before its stores
+    constexpr int PB = 8;  // pairs in flight per thread
     for (int base = threadIdx.x; base < n_pairs; base += blockDim.x * PB) {
-        float x1[PB], x2[PB];
+        // loads only, from clamped places and without a branch, so that they all go out before
+        // the first of them is waited for
+        float x1[PB], x2[PB], b1[PB], b2[PB];
+        double freq[PB];
+        int which[PB];
 #pragma unroll
         for (int u = 0; u < PB; ++u) {
-            const int idx = base + u * blockDim.x;
-            x1[u] = x2[u] = 0.f;
-            if (idx < n_pairs) {
-                const int h = idx / rotary_half;
-                const int i = idx - h * rotary_half;
-                const T* head = row + h * head_dim;
-                x1[u] = to_float(head[i]);
-                x2[u] = to_float(head[i + rotary_half]);
-                if (bias) {
-                    x1[u] += bias[h * head_dim + i];
-                    x2[u] += bias[h * head_dim + i + rotary_half];
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < PB; ++u) {
-            const int idx = base + u * blockDim.x;
-            if (idx >= n_pairs) continue;
+            const int idx = min(base + u * static_cast<int>(blockDim.x), n_pairs - 1);
             const int h = idx / rotary_half;
             const int i = idx - h * rotary_half;
-            if (i != have_i) {  // the same for the whole loop when blockDim is a multiple of rotary_half
-                rotation(pos, inv_freq[i], &c, &s);
-                have_i = i;
-            }
-            const T r1 = from_float<T>(x1[u] * c - x2[u] * s);
-            const T r2 = from_float<T>(x2[u] * c + x1[u] * s);
+            const T* head = row + h * head_dim;
+            which[u] = i;
+            freq[u] = inv_freq[i];
+            x1[u] = to_float(head[i]);
+            x2[u] = to_float(head[i + rotary_half]);
+            b1[u] = HAS_BIAS ? bias[h * head_dim + i] : 0.f;
+            b2[u] = HAS_BIAS ? bias[h * head_dim + i + rotary_half] : 0.f;
+        }
+        float c = 1.f, s = 0.f;
+#pragma unroll
+        for (int u = 0; u < PB; ++u) {
+            const int idx = base + u * blockDim.x;
+            // the same angle for the whole batch when blockDim is a multiple of rotary_half
+            if (u == 0 || which[u] != which[u - 1]) rotation(pos, freq[u], &c, &s);
+            if (idx >= n_pairs) continue;
+            const int h = idx / rotary_half;
+            const int i = which[u];
+            const float a1 = x1[u] + b1[u], a2 = x2[u] + b2[u];
+            const T r1 = from_float<T>(a1 * c - a2 * s);
+            const T r2 = from_float<T>(a2 * c + a1 * s);
             T* head = row + h * head_dim;
             head[i] = r1;
             head[i + rotary_half] = r2;
@@ -106,7 +105,7 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_kernel(
             const int h = idx / rest;
             const int d = 2 * rotary_half + (idx - h * rest);
             T* head = row + h * head_dim;
-            const T v = bias ? from_float<T>(to_float(head[d]) + bias[h * head_dim + d]) : head[d];
+            const T v = HAS_BIAS ? from_float<T>(to_float(head[d]) + bias[h * head_dim + d]) : head[d];
             head[d] = v;
             if (h >= n_heads && slot >= 0) k_pool[((page * n_kv + (h - n_heads)) * page_size + off) * head_dim + d] = v;
         }
@@ -129,17 +128,16 @@ extern "C" int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int
     const int write_kv = (k_pool && v_pool && slots) ? 1 : 0;
     FSIE_REQUIRE(!write_kv || (page_size > 0 && pool_slots > 0), "rope_kv_write: bad page geometry");
     if (n_tokens == 0) return 0;
+#define FSIE_ROPE_LAUNCH(T, B)                                                                                   \
+    rope_kv_write_kernel<T, B><<<n_tokens, kThreads, 0, stream>>>(                                               \
+        static_cast<T*>(qkv), positions, slots, inv_freq, bias, static_cast<T*>(k_pool), static_cast<T*>(v_pool), \
+        n_heads, n_kv, head_dim, rotary_dim / 2, page_size, write_kv, pool_slots)
     if (dtype == FSIE_F32) {
-        rope_kv_write_kernel<float><<<n_tokens, kThreads, 0, stream>>>(
-            static_cast<float*>(qkv), positions, slots, inv_freq, bias, static_cast<float*>(k_pool),
-            static_cast<float*>(v_pool), n_heads, n_kv, head_dim, rotary_dim / 2, page_size, write_kv,
-            pool_slots);
+        if (bias) FSIE_ROPE_LAUNCH(float, true); else FSIE_ROPE_LAUNCH(float, false);
     } else {
-        rope_kv_write_kernel<bf16_t><<<n_tokens, kThreads, 0, stream>>>(
-            static_cast<bf16_t*>(qkv), positions, slots, inv_freq, bias, static_cast<bf16_t*>(k_pool),
-            static_cast<bf16_t*>(v_pool), n_heads, n_kv, head_dim, rotary_dim / 2, page_size, write_kv,
-            pool_slots);
+        if (bias) FSIE_ROPE_LAUNCH(bf16_t, true); else FSIE_ROPE_LAUNCH(bf16_t, false);
     }
+#undef FSIE_ROPE_LAUNCH
     FSIE_CHECK_LAUNCH("rope_kv_write");
     return 0;
 }

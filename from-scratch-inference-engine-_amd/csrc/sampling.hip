@@ -51,10 +51,35 @@ __device__ __forceinline__ Best better(Best a, Best b) {
 
 __device__ Best block_argmax(const float* row, int vocab, float* sval, int* sidx) {
     Best best{-INFINITY, 0x7fffffff};
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-        const float v = row[i];
+    auto take = [&](float v, int i) {
         if (best.index == 0x7fffffff || v > best.value) best = Best{v, i};  // strict: lowest index of a stripe wins
+    };
+    int done = 0;
+    if (reinterpret_cast<uintptr_t>(row) % 16 == 0) {
+        // 16-byte loads, four of them in flight per thread
+        const int quads = vocab / 4;
+        constexpr int U = 4;
+        for (int q0 = threadIdx.x; q0 < quads; q0 += blockDim.x * U) {
+            float4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int q = min(q0 + u * static_cast<int>(blockDim.x), quads - 1);
+                v[u] = *reinterpret_cast<const float4*>(row + 4 * q);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int q = q0 + u * blockDim.x;
+                if (q < quads) {
+                    take(v[u].x, 4 * q);
+                    take(v[u].y, 4 * q + 1);
+                    take(v[u].z, 4 * q + 2);
+                    take(v[u].w, 4 * q + 3);
+                }
+            }
+        }
+        done = quads * 4;
     }
+    for (int i = done + threadIdx.x; i < vocab; i += blockDim.x) take(row[i], i);
 #pragma unroll
     for (int off = FSIE_WAVE / 2; off > 0; off >>= 1) {
         Best other{__shfl_xor(best.value, off, FSIE_WAVE), __shfl_xor(best.index, off, FSIE_WAVE)};
