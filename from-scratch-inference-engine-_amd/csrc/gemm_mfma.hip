@@ -44,12 +44,10 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         wp[b] = w + static_cast<int64_t>(n) * K + kg * 8;
     }
     const bf16_t* xp[MT];
-    bool x_ok[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-        const int m = t * 16 + row;
-        x_ok[t] = m < M;
-        xp[t] = x + static_cast<int64_t>(x_ok[t] ? m : 0) * K + kg * 8;
+        // rows of X past the end read the last row again: their columns of D are never written
+        xp[t] = x + static_cast<int64_t>(min(t * 16 + row, M - 1)) * K + kg * 8;
     }
     floatx4 acc[NB][MT];
 #pragma unroll
@@ -59,31 +57,35 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
 
     // k steps of 32; a wave takes pairs of steps (128 bytes of every row), pairs interleaved over the waves
     const int n_pairs = (K + 2 * kStep - 1) / (2 * kStep);
-    constexpr int U = (NB * MT >= 8) ? 1 : 2;  // pairs in flight per wave
+    constexpr int U = (NB * MT >= 8) ? 1 : 2;  // pairs in flight per wave (more cost occupancy and lost 10-30 %)
     for (int p0 = wave; p0 < n_pairs; p0 += WAVES * U) {
+        // loads without branches, so that they all go out before the first wait: a step past the
+        // end of K reads step 0 again and its A fragments are zeroed afterwards
         Frag a[U][2][NB], b[U][2][MT];
+        bool ok[U][2];
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int k0 = ((p0 + u * WAVES) * 2 + h) * kStep;
-                const bool ok = k0 + kg * 8 < K;  // K is a multiple of 8: a lane's 8 values are all in or all out
+                ok[u][h] = k0 + kg * 8 < K;  // K is a multiple of 8: a lane's 8 values are all in or all out
+                const int k0c = ok[u][h] ? k0 : 0;
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-                    a[u][h][nb].raw = ok ? *reinterpret_cast<const uint4*>(wp[nb] + k0) : uint4{0, 0, 0, 0};
+                for (int nb = 0; nb < NB; ++nb) a[u][h][nb].raw = *reinterpret_cast<const uint4*>(wp[nb] + k0c);
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
-                    b[u][h][t].raw = (ok && x_ok[t]) ? *reinterpret_cast<const uint4*>(xp[t] + k0) : uint4{0, 0, 0, 0};
+                for (int t = 0; t < MT; ++t) b[u][h][t].raw = *reinterpret_cast<const uint4*>(xp[t] + k0c);
             }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
+                for (int nb = 0; nb < NB; ++nb) {
+                    if (!ok[u][h]) a[u][h][nb].raw = uint4{0, 0, 0, 0};
 #pragma unroll
                     for (int t = 0; t < MT; ++t)
                         acc[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][h][nb].v, b[u][h][t].v, acc[nb][t], 0, 0, 0);
+                }
     }
 
     if (WAVES > 1) {
