@@ -23,13 +23,26 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ x
     const int tid = threadIdx.x;
     const int tx = tid % 16, ty = tid / 16;
     const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
-    float acc[4][4];
+    // two levels of float32 sums: runs of kFlush products are added up on their own and then
+    // added to the total, so that the rounding error grows with sqrt(kFlush) + sqrt(K / kFlush)
+    // instead of sqrt(K) (K reaches 18944 in a 7B model)
+    constexpr int kFlush = 256;
+    float acc[4][4], total[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+        for (int j = 0; j < 4; ++j) acc[i][j] = total[i][j] = 0.f;
 
     for (int k0 = 0; k0 < K; k0 += TK) {
+        if (k0 > 0 && k0 % kFlush == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    total[i][j] += acc[i][j];
+                    acc[i][j] = 0.f;
+                }
+        }
         // 64 rows x 16 k per operand: 1024 elements, 4 per thread; k is the fast index in memory
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -63,7 +76,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ x
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
             if (n >= N) continue;
-            float v = acc[i][j];
+            float v = total[i][j] + acc[i][j];
             if (bias) v += bias[n];
             y[static_cast<int64_t>(m) * N + n] = from_float<OutT>(v);
         }
