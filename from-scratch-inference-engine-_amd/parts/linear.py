@@ -35,8 +35,9 @@ class Linear:
         wants_f32 = out_dtype is not None and out_dtype != x.dtype
         if self.in_features % 8 == 0 and m <= (GEMM_MFMA_SKINNY_MAX_M if wants_f32 else GEMM_MFMA_SKINNY_BEST_M):
             return ops.gemm_mfma_skinny(x, w, bias, out_dtype=out_dtype)
-        if m <= GEMM_SKINNY_MAX_M or wants_f32:
-            # odd inner sizes, and float32 results from bfloat16 operands (logits of many rows)
+        if m <= GEMM_SKINNY_MAX_M or wants_f32 or self.in_features % 8 or self.out_features % 8:
+            # few rows with an odd inner size; float32 results from bfloat16 operands (logits of
+            # many rows); and sizes whose rows are not 16-byte aligned, which the library is not given
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
         y = torch.mm(x, w.t())
         if bias is not None:
