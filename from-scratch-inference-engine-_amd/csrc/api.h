@@ -12,6 +12,7 @@
 #define FSIE_GEMM_SKINNY_MAX_M 8
 #define FSIE_GEMM_MFMA_SKINNY_MAX_M 64
 #define FSIE_GEMM_MFMA_SKINNY_BEST_M 16  // above this the library product is faster on MI355X
+#define FSIE_GEMM_MAX_SPLITS 8           // most slices of K a product may leave as partial sums
 
 // one attention work item = 8 int32
 #define FSIE_ATTN_ITEM_INTS 8
@@ -37,7 +38,8 @@ int fsie_device_info(char* arch_out, int arch_len, int* n_compute_units);
 int fsie_embedding(const void* table, int dtype, const int32_t* ids, float* out, int n_tokens, int hidden,
                    int vocab, hipStream_t stream);
 int fsie_rmsnorm(float* residual, const void* delta, const float* weight, void* out, const int32_t* rows,
-                 int n_rows, int hidden, float eps, int dtype, int write_back, hipStream_t stream);
+                 int n_rows, int hidden, float eps, int dtype, int write_back, int n_parts, int total_rows,
+                 hipStream_t stream);
 int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream);
 int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream);
 int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream);
@@ -50,7 +52,7 @@ int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, i
               int out_f32, int kind, hipStream_t stream);
 
 int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
-                          int out_f32, int waves, int blocks, int epilogue, hipStream_t stream);
+                          int out_f32, int waves, int blocks, int epilogue, int splits, hipStream_t stream);
 
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,

@@ -27,21 +27,31 @@ __global__ void embedding_kernel(const T* __restrict__ table, const int32_t* __r
 // One block per output row r; source row = rows ? rows[r] : r.
 //   v = residual[row] (+ delta[row]);  if write_back: residual[row] = v
 //   out[r] = (v * rsqrt(mean(v^2) + eps)) * weight
-// Sum of squares, scale and the residual sum are float32.
+// Sum of squares, scale and the residual sum are float32.  With n_parts > 0 the delta is the sum,
+// taken in order, of n_parts float32 arrays [total_rows, hidden] that lie one after the other
+// (partial sums of a matrix product whose inner dimension was cut).
 template <typename T>
 __global__ void rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
                                const float* __restrict__ weight, T* __restrict__ out,
                                const int32_t* __restrict__ rows, int hidden, float eps,
-                               int write_back) {
+                               int write_back, int n_parts, int64_t part_stride) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const int64_t row = rows ? rows[r] : r;
     float* res = residual + row * hidden;
-    const T* del = delta ? delta + row * hidden : nullptr;
+    const T* del = (delta && !n_parts) ? delta + row * hidden : nullptr;
+    const float* parts = n_parts ? reinterpret_cast<const float*>(delta) + row * hidden : nullptr;
+    auto delta_at = [&](int j) {
+        if (del) return to_float(del[j]);
+        float d = 0.f;
+        for (int s = 0; s < n_parts; ++s) d += parts[s * part_stride + j];
+        return d;
+    };
+    const bool has_delta = del || parts;
     float sum_sq = 0.f;
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
         float v = res[j];
-        if (del) v += to_float(del[j]);
+        if (has_delta) v += delta_at(j);
         if (write_back) res[j] = v;
         sum_sq += v * v;
     }
@@ -50,7 +60,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ residual, const T* __restrict
     T* dst = out + static_cast<int64_t>(r) * hidden;
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
         float v = res[j];
-        if (del && !write_back) v += to_float(del[j]);
+        if (has_delta && !write_back) v += delta_at(j);
         dst[j] = from_float<T>((v * scale) * weight[j]);
     }
 }
@@ -92,15 +102,19 @@ __global__ void embedding_vec_kernel(const T* __restrict__ table, const int32_t*
     Pack4<float>::store(out + static_cast<int64_t>(t) * hidden + j, ok ? v : float4{0.f, 0.f, 0.f, 0.f});
 }
 
-template <typename T, int ITERS, bool HAS_DELTA, bool WRITE_BACK>
+// DELTA: 0 = none, 1 = one array of T, 2 / 4 / 8 = that many float32 partial sums, added in order.
+template <typename T, int ITERS, int DELTA, bool WRITE_BACK>
 __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta,
                                                                const float* __restrict__ weight, T* __restrict__ out,
-                                                               const int32_t* __restrict__ rows, int hidden, float eps) {
+                                                               const int32_t* __restrict__ rows, int hidden, float eps,
+                                                               int64_t part_stride) {
     __shared__ float scratch[16];
+    constexpr bool HAS_DELTA = DELTA != 0;
     const int r = blockIdx.x;
     const int64_t row = rows ? rows[r] : r;
     float* res = residual + row * hidden;
-    const T* del = HAS_DELTA ? delta + row * hidden : nullptr;
+    const T* del = DELTA == 1 ? delta + row * hidden : nullptr;
+    const float* parts = DELTA > 1 ? reinterpret_cast<const float*>(delta) + row * hidden : nullptr;
     // every load of the row goes out before anything waits: places past the end read the last
     // quad again and are masked out of the sum and the stores
     float4 v[ITERS], d[ITERS], w[ITERS];
@@ -108,7 +122,20 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict
     for (int it = 0; it < ITERS; ++it) {
         const int j = min((it * kThreads + static_cast<int>(threadIdx.x)) * 4, hidden - 4);
         v[it] = Pack4<float>::load(res + j);
-        if (HAS_DELTA) d[it] = Pack4<T>::load(del + j);
+        if (DELTA == 1) d[it] = Pack4<T>::load(del + j);
+        if (DELTA > 1) {
+            float4 p[DELTA > 1 ? DELTA : 1];
+#pragma unroll
+            for (int s = 0; s < DELTA; ++s) p[s] = Pack4<float>::load(parts + s * part_stride + j);
+            d[it] = p[0];
+#pragma unroll
+            for (int s = 1; s < DELTA; ++s) {
+                d[it].x += p[s].x;
+                d[it].y += p[s].y;
+                d[it].z += p[s].z;
+                d[it].w += p[s].w;
+            }
+        }
         w[it] = Pack4<float>::load(weight + j);
     }
     float sum_sq = 0.f;
@@ -139,37 +166,63 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict
     }
 }
 
-template <typename T, int ITERS>
-void launch_rmsnorm_vec(float* residual, const T* d, const float* weight, T* o, const int32_t* rows, int n_rows,
-                        int hidden, float eps, int write_back, hipStream_t stream) {
-    if (!d) {
-        rmsnorm_vec_kernel<T, ITERS, false, false><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps);
-    } else if (write_back) {
-        rmsnorm_vec_kernel<T, ITERS, true, true><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps);
+struct NormCall {
+    float* residual;
+    const void* delta;
+    const float* weight;
+    void* out;
+    const int32_t* rows;
+    int n_rows, hidden;
+    float eps;
+    int write_back;
+    int n_parts;          // 0: delta (if any) is one array of the output's type
+    int64_t part_stride;  // elements between the partial sums
+    hipStream_t stream;
+};
+
+template <typename T, int ITERS, int DELTA>
+void launch_rmsnorm_delta(const NormCall& c) {
+    const T* d = static_cast<const T*>(c.delta);
+    T* o = static_cast<T*>(c.out);
+    if (c.write_back) {
+        rmsnorm_vec_kernel<T, ITERS, DELTA, DELTA != 0><<<c.n_rows, kThreads, 0, c.stream>>>(
+            c.residual, d, c.weight, o, c.rows, c.hidden, c.eps, c.part_stride);
     } else {
-        rmsnorm_vec_kernel<T, ITERS, true, false><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps);
+        rmsnorm_vec_kernel<T, ITERS, DELTA, false><<<c.n_rows, kThreads, 0, c.stream>>>(
+            c.residual, d, c.weight, o, c.rows, c.hidden, c.eps, c.part_stride);
+    }
+}
+
+template <typename T, int ITERS>
+void launch_rmsnorm_vec(const NormCall& c) {
+    if (!c.delta) return launch_rmsnorm_delta<T, ITERS, 0>(c);
+    switch (c.n_parts) {
+        case 0: return launch_rmsnorm_delta<T, ITERS, 1>(c);
+        case 2: return launch_rmsnorm_delta<T, ITERS, 2>(c);
+        case 4: return launch_rmsnorm_delta<T, ITERS, 4>(c);
+        default: return launch_rmsnorm_delta<T, ITERS, 8>(c);
     }
 }
 
 template <typename T>
-void launch_rmsnorm(float* residual, const void* delta, const float* weight, void* out, const int32_t* rows, int n_rows,
-                    int hidden, float eps, int write_back, hipStream_t stream) {
-    const T* d = static_cast<const T*>(delta);
-    T* o = static_cast<T*>(out);
-    const bool aligned = hidden % 4 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(weight) % 16 == 0 && reinterpret_cast<uintptr_t>(delta) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(out) % 16 == 0;
+void launch_rmsnorm(const NormCall& c) {
+    const bool aligned = c.hidden % 4 == 0 && reinterpret_cast<uintptr_t>(c.residual) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(c.weight) % 16 == 0 && reinterpret_cast<uintptr_t>(c.delta) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(c.out) % 16 == 0 && c.part_stride % 4 == 0 &&
+                         (c.n_parts == 0 || c.n_parts == 2 || c.n_parts == 4 || c.n_parts == 8);
     const int per_iter = kThreads * 4;
-    if (aligned && hidden >= 4 && hidden <= per_iter) {
-        launch_rmsnorm_vec<T, 1>(residual, d, weight, o, rows, n_rows, hidden, eps, write_back, stream);
-    } else if (aligned && hidden <= 2 * per_iter && hidden >= 4) {
-        launch_rmsnorm_vec<T, 2>(residual, d, weight, o, rows, n_rows, hidden, eps, write_back, stream);
-    } else if (aligned && hidden <= 4 * per_iter && hidden >= 4) {
-        launch_rmsnorm_vec<T, 4>(residual, d, weight, o, rows, n_rows, hidden, eps, write_back, stream);
-    } else if (aligned && hidden <= 8 * per_iter && hidden >= 4) {
-        launch_rmsnorm_vec<T, 8>(residual, d, weight, o, rows, n_rows, hidden, eps, write_back, stream);
+    if (aligned && c.hidden >= 4 && c.hidden <= per_iter) {
+        launch_rmsnorm_vec<T, 1>(c);
+    } else if (aligned && c.hidden <= 2 * per_iter && c.hidden >= 4) {
+        launch_rmsnorm_vec<T, 2>(c);
+    } else if (aligned && c.hidden <= 4 * per_iter && c.hidden >= 4) {
+        launch_rmsnorm_vec<T, 4>(c);
+    } else if (aligned && c.hidden <= 8 * per_iter && c.hidden >= 4) {
+        launch_rmsnorm_vec<T, 8>(c);
     } else {
-        rmsnorm_kernel<T><<<n_rows, kThreads, 0, stream>>>(residual, d, weight, o, rows, hidden, eps, write_back);
+        rmsnorm_kernel<T><<<c.n_rows, kThreads, 0, c.stream>>>(c.residual, static_cast<const T*>(c.delta), c.weight,
+                                                             static_cast<T*>(c.out), c.rows, c.hidden, c.eps,
+                                                             c.write_back, c.n_parts, c.part_stride);
     }
 }
 
@@ -226,18 +279,25 @@ extern "C" int fsie_embedding(const void* table, int dtype, const int32_t* ids, 
     return 0;
 }
 
+// n_parts > 0: delta is n_parts float32 arrays [total_rows, hidden], one after the other, whose sum
+// (taken in order) is the delta; total_rows is the number of rows of the residual.
 extern "C" int fsie_rmsnorm(float* residual, const void* delta, const float* weight, void* out,
                             const int32_t* rows, int n_rows, int hidden, float eps, int dtype,
-                            int write_back, hipStream_t stream) {
+                            int write_back, int n_parts, int total_rows, hipStream_t stream) {
+    FSIE_REQUIRE(n_parts >= 0 && n_parts <= FSIE_GEMM_MAX_SPLITS && n_parts != 1,
+                 "rmsnorm: the delta comes whole or in 2..%d parts, not %d", FSIE_GEMM_MAX_SPLITS, n_parts);
+    FSIE_REQUIRE(n_parts == 0 || (delta && total_rows > 0), "rmsnorm: parts without a delta or a row count");
     FSIE_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, hidden);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "rmsnorm: unknown dtype %d", dtype);
     FSIE_REQUIRE(!(write_back && rows), "rmsnorm: write_back cannot be combined with a row list");
     FSIE_REQUIRE(!(write_back && !delta), "rmsnorm: write_back without a delta");
     if (n_rows == 0) return 0;
+    const NormCall call{residual, delta, weight, out, rows, n_rows, hidden, eps, write_back, n_parts,
+                        static_cast<int64_t>(total_rows) * hidden, stream};
     if (dtype == FSIE_F32) {
-        launch_rmsnorm<float>(residual, delta, weight, out, rows, n_rows, hidden, eps, write_back, stream);
+        launch_rmsnorm<float>(call);
     } else {
-        launch_rmsnorm<bf16_t>(residual, delta, weight, out, rows, n_rows, hidden, eps, write_back, stream);
+        launch_rmsnorm<bf16_t>(call);
     }
     FSIE_CHECK_LAUNCH("rmsnorm");
     return 0;

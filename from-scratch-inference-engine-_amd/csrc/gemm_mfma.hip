@@ -27,10 +27,13 @@ constexpr int kStep = 32;  // k per MFMA
 // fragments), WAVES = waves of the workgroup, which split K.
 // SWIGLU: the rows of W are gate and up interleaved; the output has N/2 columns,
 // y[m, j] = silu(d[2j]) * d[2j + 1], computed in float32 from the accumulators.
+// blockIdx.y selects a slice of K of `k_slice` values (a multiple of 64); with more than one slice
+// the kernel writes float32 partial sums y[slice][m][n] without bias, for the consumer to add up
+// in the order of the slices.
 template <int MT, int NB, int WAVES, typename OutT, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    OutT* __restrict__ y, int M, int N, int K) {
+    OutT* __restrict__ y, int M, int N, int K, int k_slice) {
     __shared__ float red[WAVES > 1 ? (WAVES - 1) * NB * MT * FSIE_WAVE * 4 : 1];
     const int lane = threadIdx.x & (FSIE_WAVE - 1);
     const int wave = threadIdx.x / FSIE_WAVE;
@@ -56,7 +59,9 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         for (int t = 0; t < MT; ++t) acc[b][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     // k steps of 32; a wave takes pairs of steps (128 bytes of every row), pairs interleaved over the waves
-    const int n_pairs = (K + 2 * kStep - 1) / (2 * kStep);
+    const int k_begin = blockIdx.y * k_slice;
+    const int k_end = min(K, k_begin + k_slice);
+    const int n_pairs = (k_end - k_begin + 2 * kStep - 1) / (2 * kStep);
     constexpr int U = (NB * MT >= 8) ? 1 : 2;  // pairs in flight per wave (more cost occupancy and lost 10-30 %)
     for (int p0 = wave; p0 < n_pairs; p0 += WAVES * U) {
         // loads without branches, so that they all go out before the first wait: a step past the
@@ -67,8 +72,8 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const int k0 = ((p0 + u * WAVES) * 2 + h) * kStep;
-                ok[u][h] = k0 + kg * 8 < K;  // K is a multiple of 8: a lane's 8 values are all in or all out
+                const int k0 = k_begin + ((p0 + u * WAVES) * 2 + h) * kStep;
+                ok[u][h] = k0 + kg * 8 < k_end;  // K is a multiple of 8: a lane's 8 values are all in or all out
                 const int k0c = ok[u][h] ? k0 : 0;
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) a[u][h][nb].raw = *reinterpret_cast<const uint4*>(wp[nb] + k0c);
@@ -116,6 +121,15 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         for (int t = 0; t < MT; ++t) {
             const int m = t * 16 + row;
             if (m >= M) continue;
+            if (gridDim.y > 1) {
+                float* part = reinterpret_cast<float*>(y) + (static_cast<int64_t>(blockIdx.y) * M + m) * N;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int nn = n0 + nb * 16 + kg * 4 + r;
+                    if (nn < N) part[nn] = acc[nb][t][r];
+                }
+                continue;
+            }
             if (SWIGLU) {
 #pragma unroll
                 for (int r = 0; r < 4; r += 2) {
@@ -138,49 +152,57 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         }
 }
 
+struct Call {
+    const void* x;
+    const void* w;
+    const float* bias;
+    void* y;
+    int M, N, K;
+    int splits;  // slices of K, each a workgroup row of its own (partial sums out) when > 1
+    hipStream_t stream;
+};
+
 template <int MT, int NB, int WAVES, typename OutT, bool SWIGLU>
-int launch(const void* x, const void* w, const float* bias, void* y, int M, int N, int K, hipStream_t stream) {
-    const unsigned grid = static_cast<unsigned>((N + 16 * NB - 1) / (16 * NB));
-    gemm_mfma_skinny_kernel<MT, NB, WAVES, OutT, SWIGLU><<<grid, WAVES * FSIE_WAVE, 0, stream>>>(
-        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias, static_cast<OutT*>(y), M, N, K);
+int launch(const Call& c) {
+    const int k_slice = c.splits > 1 ? ((c.K + c.splits - 1) / c.splits + 63) / 64 * 64 : c.K;
+    const dim3 grid(static_cast<unsigned>((c.N + 16 * NB - 1) / (16 * NB)),
+                    static_cast<unsigned>(c.splits > 1 ? c.splits : 1));
+    gemm_mfma_skinny_kernel<MT, NB, WAVES, OutT, SWIGLU><<<grid, WAVES * FSIE_WAVE, 0, c.stream>>>(
+        static_cast<const bf16_t*>(c.x), static_cast<const bf16_t*>(c.w), c.bias, static_cast<OutT*>(c.y), c.M, c.N,
+        c.K, k_slice);
     FSIE_CHECK_LAUNCH("gemm_mfma_skinny");
     return 0;
 }
 
 template <int MT, int NB, typename OutT, bool SWIGLU>
-int launch_waves(int waves, const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
-                 hipStream_t stream) {
+int launch_waves(int waves, const Call& c) {
     switch (waves) {
-        case 1: return launch<MT, NB, 1, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
-        case 2: return launch<MT, NB, 2, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
-        case 4: return launch<MT, NB, 4, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
-        case 8: return launch<MT, NB, 8, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
+        case 1: return launch<MT, NB, 1, OutT, SWIGLU>(c);
+        case 2: return launch<MT, NB, 2, OutT, SWIGLU>(c);
+        case 4: return launch<MT, NB, 4, OutT, SWIGLU>(c);
+        case 8: return launch<MT, NB, 8, OutT, SWIGLU>(c);
         default:
-            if constexpr (MT * NB <= 4) return launch<MT, NB, 16, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
-            return launch<MT, NB, 8, OutT, SWIGLU>(x, w, bias, y, M, N, K, stream);
+            if constexpr (MT * NB <= 4) return launch<MT, NB, 16, OutT, SWIGLU>(c);
+            return launch<MT, NB, 8, OutT, SWIGLU>(c);
     }
 }
 
 template <int MT, typename OutT, bool SWIGLU>
-int launch_blocks(int nb, int waves, const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
-                  hipStream_t stream) {
+int launch_blocks(int nb, int waves, const Call& c) {
     switch (nb) {
-        case 1: return launch_waves<MT, 1, OutT, SWIGLU>(waves, x, w, bias, y, M, N, K, stream);
-        case 2: return launch_waves<MT, 2, OutT, SWIGLU>(waves, x, w, bias, y, M, N, K, stream);
-        default:
-            if constexpr (MT <= 2) return launch_waves<MT, 4, OutT, SWIGLU>(waves, x, w, bias, y, M, N, K, stream);
-            return launch_waves<MT, 2, OutT, SWIGLU>(waves, x, w, bias, y, M, N, K, stream);
+        case 1: return launch_waves<MT, 1, OutT, SWIGLU>(waves, c);
+        case 2: return launch_waves<MT, 2, OutT, SWIGLU>(waves, c);
+        default: return launch_waves<MT, 4, OutT, SWIGLU>(waves, c);
     }
 }
 
 template <typename OutT, bool SWIGLU>
-int launch_tiles(int mt, int nb, int waves, const void* x, const void* w, const float* bias, void* y, int M, int N,
-                 int K, hipStream_t stream) {
+int launch_tiles(int mt, int nb, int waves, const Call& c) {
     switch (mt) {
-        case 1: return launch_blocks<1, OutT, SWIGLU>(nb, waves, x, w, bias, y, M, N, K, stream);
-        case 2: return launch_blocks<2, OutT, SWIGLU>(nb, waves, x, w, bias, y, M, N, K, stream);
-        case 3: return launch_blocks<3, OutT, SWIGLU>(nb, waves, x, w, bias, y, M, N, K, stream);
-        default: return launch_blocks<4, OutT, SWIGLU>(nb, waves, x, w, bias, y, M, N, K, stream);
+        case 1: return launch_blocks<1, OutT, SWIGLU>(nb, waves, c);
+        case 2: return launch_blocks<2, OutT, SWIGLU>(nb, waves, c);
+        case 3: return launch_blocks<3, OutT, SWIGLU>(nb, waves, c);
+        default: return launch_blocks<4, OutT, SWIGLU>(nb, waves, c);
     }
 }
 
@@ -189,8 +211,18 @@ int launch_tiles(int mt, int nb, int waves, const void* x, const void* w, const 
 // bfloat16 only.  M <= 64, K a multiple of 8, x and w 16-byte aligned.
 // waves (K split inside a workgroup) and blocks (16-row blocks of W per workgroup): 0 = choose.
 // epilogue: 0 = y = d (+ bias); 1 = SiLU*up over interleaved gate/up rows (N even, no bias, y is [M, N/2]).
+// splits > 1: K is cut into that many slices, each summed by workgroups of its own; y is then
+// float32 [splits, M, N], partial sums without bias, which the consumer adds in the order of the slices
+// (fsie_rmsnorm takes them as its delta).  Every slice must hold at least 64 values of K.
 extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
-                                     int out_f32, int waves, int blocks, int epilogue, hipStream_t stream) {
+                                     int out_f32, int waves, int blocks, int epilogue, int splits,
+                                     hipStream_t stream) {
+    FSIE_REQUIRE(splits >= 1 && splits <= FSIE_GEMM_MAX_SPLITS, "gemm_mfma_skinny: splits must be 1..%d, got %d",
+                 FSIE_GEMM_MAX_SPLITS, splits);
+    FSIE_REQUIRE(splits == 1 || (epilogue == 0 && !bias && out_f32),
+                 "gemm_mfma_skinny: partial sums are float32, without bias or epilogue");
+    FSIE_REQUIRE(splits == 1 || ((K + splits - 1) / splits + 63) / 64 * 64 * (splits - 1) < K,
+                 "gemm_mfma_skinny: K=%d is too short for %d slices", K, splits);
     FSIE_REQUIRE(epilogue == 0 || epilogue == 1, "gemm_mfma_skinny: unknown epilogue %d", epilogue);
     FSIE_REQUIRE(epilogue == 0 || (N % 2 == 0 && !bias && !out_f32),
                  "gemm_mfma_skinny: the SiLU*up epilogue needs an even N, no bias and a bfloat16 result");
@@ -205,23 +237,24 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
     FSIE_REQUIRE(blocks == 0 || blocks == 1 || blocks == 2 || blocks == 4, "gemm_mfma_skinny: blocks must be 0, 1, 2 or 4");
     if (M == 0) return 0;
     const int mt = (M + 15) / 16;
-    const int pairs = (K + 2 * kStep - 1) / (2 * kStep);
+    const int pairs = ((K + splits - 1) / splits + 2 * kStep - 1) / (2 * kStep);
     if (blocks == 0) {
         // more than a few rows of X: two blocks of W share each X fragment where N still leaves
         // enough workgroups for the chip (measured on MI355X: 5.2 against 4.4 TB/s at N = 37888)
-        blocks = (M > 4 && N >= 16384) ? 2 : 1;
+        blocks = (M > 4 && static_cast<int64_t>(N) * splits >= 14336) ? 2 : 1;
     }
     if (waves == 0) {
         // split K inside the workgroup until about a thousand waves stream W; a single row of X
         // gains from more loads in flight even at large N
-        const int groups = (N + 16 * blocks - 1) / (16 * blocks);
+        const int groups = (N + 16 * blocks - 1) / (16 * blocks) * splits;
         waves = 1;
         while (waves < 16 && groups * waves < 1024) waves *= 2;
         if (M <= 4 && waves < 8) waves = 8;
         while (waves > 1 && pairs < 2 * waves) waves /= 2;
     }
     if (mt * blocks > 4 && waves > 8) waves = 8;  // LDS of the reduction
-    if (epilogue == 1) return launch_tiles<bf16_t, true>(mt, blocks, waves, x, w, bias, y, M, N, K, stream);
-    return out_f32 ? launch_tiles<float, false>(mt, blocks, waves, x, w, bias, y, M, N, K, stream)
-                   : launch_tiles<bf16_t, false>(mt, blocks, waves, x, w, bias, y, M, N, K, stream);
+    const Call call{x, w, bias, y, M, N, K, splits, stream};
+    if (epilogue == 1) return launch_tiles<bf16_t, true>(mt, blocks, waves, call);
+    return out_f32 ? launch_tiles<float, false>(mt, blocks, waves, call)
+                   : launch_tiles<bf16_t, false>(mt, blocks, waves, call);
 }

@@ -124,6 +124,8 @@ class StepContext:
         self.n_seqs = host.n_seqs
         self.token_ids = self.positions = self.want_rows = None
         self.seq_slots = self.q_starts = self.past_lens = None
+        # set by the model: every norm can add up a delta that comes as float32 partial sums
+        self.partial_sums_ok = False
         self.block_tables: List[torch.Tensor] = []
         self.slots: List[torch.Tensor] = []
         self._plans: Dict[Hashable, SimpleNamespace] = {}

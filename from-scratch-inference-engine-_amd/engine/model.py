@@ -119,8 +119,10 @@ class Model:
         return model
 
     def _prepare(self) -> None:
+        from ..parts.base import Norm
         for part in self.spec.all_parts():
             part.prepare(self.device, self.dtype)
+        self.partial_sums_ok = all(p.adds_partial_sums for p in self.spec.all_parts() if isinstance(p, Norm))
 
     # ---------------------------------------------------------------- cache
     def make_cache(self, page_size: int, num_pages: int, max_requests: int):
@@ -137,6 +139,7 @@ class Model:
     def forward(self, ctx: StepContext, storage: CacheStorage) -> torch.Tensor:
         """float32 logits [wanted, vocab] for the step described by ``ctx``."""
         spec = self.spec
+        ctx.partial_sums_ok = self.partial_sums_ok
         hidden = HiddenState(spec.embedding.forward(ctx.token_ids))
         for i, call in enumerate(spec.schedule):
             cid = self.call_cache[i]

@@ -137,9 +137,16 @@ class Scheduler:
             self.running.append(seq.id)
             self.waiting.popleft()
 
-    def _fit_tokens(self, reserved, seq: Sequence, n: int) -> int:
-        """Largest n' <= n such that the step can still reserve n' tokens for ``seq``."""
-        while n > 0 and not self.manager.can_reserve(reserved + [(seq.cache, n)]):
+    def _fit_tokens(self, taken: List[int], seq: Sequence, n: int) -> int:
+        """Largest n' <= n such that the step can still reserve n' tokens for ``seq`` beside the
+        pages per group that its other items have ``taken``."""
+        manager = self.manager
+
+        def fits(k: int) -> bool:
+            need = manager.new_pages_needed(seq.cache, k)
+            return all(need[g] + taken[g] <= manager.free_pages(g) for g in range(len(taken)))
+
+        while n > 0 and not fits(n):
             # cut back to the last page boundary below n (what is free in the last held page
             # always fits), then page by page
             filled = seq.computed + n
@@ -148,7 +155,7 @@ class Scheduler:
 
     def _build(self) -> List[ScheduledItem]:
         items: List[ScheduledItem] = []
-        reserved = []
+        taken = [0] * len(self.manager.groups)
         budget = self.max_tokens_per_step
         seqs = [self.sequences[i] for i in self.running]
         for decode_pass in (True, False):
@@ -157,13 +164,14 @@ class Scheduler:
                 if decoding != decode_pass or budget <= 0:
                     continue
                 n = min(seq.remaining, budget) if decode_pass else min(seq.remaining, self.prefill_chunk, budget)
-                n = self._fit_tokens(reserved, seq, n)
+                n = self._fit_tokens(taken, seq, n)
                 if n <= 0:
                     continue
                 ctx = seq.context
                 tokens = ctx[seq.computed:seq.computed + n]
                 items.append(ScheduledItem(seq, tokens, seq.computed + n == len(ctx)))
-                reserved.append((seq.cache, n))
+                for g, k in enumerate(self.manager.new_pages_needed(seq.cache, n)):
+                    taken[g] += k
                 budget -= n
         return items
 

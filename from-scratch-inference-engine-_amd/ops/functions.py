@@ -14,6 +14,7 @@ ATTN_MERGE_INTS = 4
 GEMM_SKINNY_MAX_M = 8
 GEMM_MFMA_SKINNY_MAX_M = 64
 GEMM_MFMA_SKINNY_BEST_M = 16
+GEMM_SPLITS = (2, 4, 8)  # slices of K that a product may leave as partial sums
 GEMM_AUTO, GEMM_TILED, GEMM_SKINNY = 0, 1, 2
 
 
@@ -63,12 +64,19 @@ def embedding(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor
 def rmsnorm(residual: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
             write_back: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """RMSNorm of ``residual (+ delta)`` (float32 stream, delta in ``out_dtype``) times ``weight``
-    (float32).  ``write_back`` stores the sum into ``residual``; ``rows`` (int32) selects rows."""
+    """RMSNorm of ``residual (+ delta)`` (float32 stream) times ``weight`` (float32).  ``delta``
+    is [T, H] in ``out_dtype``, or float32 [S, T, H] with S in (2, 4, 8): partial sums that are
+    added in order.  ``write_back`` stores the sum into ``residual``; ``rows`` (int32) selects rows."""
     _need(residual, "rmsnorm residual", dtype=torch.float32, ndim=2)
     t, h = residual.shape
     _need(weight, "rmsnorm weight", dtype=torch.float32, shape=(h,))
-    if delta is not None:
+    n_parts = 0
+    if delta is not None and delta.ndim == 3:
+        n_parts = delta.shape[0]
+        _need(delta, "rmsnorm delta parts", dtype=torch.float32, shape=(n_parts, t, h))
+        if n_parts not in GEMM_SPLITS:
+            raise KernelError(f"rmsnorm: {n_parts} partial sums; offered are {GEMM_SPLITS}")
+    elif delta is not None:
         _need(delta, "rmsnorm delta", dtype=out_dtype, shape=(t, h))
     n_rows = t
     if rows is not None:
@@ -78,7 +86,7 @@ def rmsnorm(residual: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype:
         out = torch.empty((n_rows, h), dtype=out_dtype, device=residual.device)
     _need(out, "rmsnorm out", dtype=out_dtype, shape=(n_rows, h))
     check(load().fsie_rmsnorm(residual.data_ptr(), _ptr(delta), weight.data_ptr(), out.data_ptr(), _ptr(rows),
-                              n_rows, h, float(eps), dtype_code(out_dtype), int(write_back), _stream()))
+                              n_rows, h, float(eps), dtype_code(out_dtype), int(write_back), n_parts, t, _stream()))
     return out
 
 
@@ -172,10 +180,11 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = N
 
 def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      out_dtype: Optional[torch.dtype] = None, waves: int = 0, blocks: int = 0,
-                     out: Optional[torch.Tensor] = None, epilogue: str = "plain") -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, epilogue: str = "plain", splits: int = 1) -> torch.Tensor:
     """The same product on the matrix cores for bfloat16 and at most 64 rows (K a multiple of 8).
     ``epilogue="swiglu"``: the rows of ``weight`` are gate and up interleaved and the result is
-    silu(gate) * up, [M, N/2]."""
+    silu(gate) * up, [M, N/2].  ``splits`` in (2, 4, 8): K is cut into that many slices and the
+    result is their float32 partial sums [splits, M, N] (no bias), for ``rmsnorm`` to add up."""
     _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
     _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
     m, k = x.shape
@@ -192,12 +201,17 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     if epilogue == "swiglu" and n % 2:
         raise KernelError(f"gemm: the swiglu epilogue needs an even number of weight rows, found {n}")
     n_out = n // 2 if epilogue == "swiglu" else n
+    shape = (m, n_out)
+    if splits != 1:
+        if splits not in GEMM_SPLITS or epilogue != "plain" or bias is not None:
+            raise KernelError(f"gemm: partial sums come in {GEMM_SPLITS} slices, without bias or epilogue")
+        out_dtype, shape = torch.float32, (splits, m, n)
     if out is None:
-        out = torch.empty((m, n_out), dtype=out_dtype, device=x.device)
-    _need(out, "gemm out", dtype=out_dtype, shape=(m, n_out))
+        out = torch.empty(shape, dtype=out_dtype, device=x.device)
+    _need(out, "gemm out", dtype=out_dtype, shape=shape)
     check(load().fsie_gemm_mfma_skinny(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k,
                                        int(out_dtype == torch.float32), waves, blocks, int(epilogue == "swiglu"),
-                                       _stream()))
+                                       splits, _stream()))
     return out
 
 

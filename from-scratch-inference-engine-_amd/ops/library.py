@@ -26,14 +26,14 @@ _SIGNATURES = {
     "fsie_version": ([], c_int),
     "fsie_device_info": ([c_char_p, c_int, ctypes.POINTER(c_int)], c_int),
     "fsie_embedding": ([_P, c_int, _P, _P, c_int, c_int, c_int, _P], c_int),
-    "fsie_rmsnorm": ([_P, _P, _P, _P, _P, c_int, c_int, c_float, c_int, c_int, _P], c_int),
+    "fsie_rmsnorm": ([_P, _P, _P, _P, _P, c_int, c_int, c_float, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_swiglu": ([_P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_residual_add": ([_P, _P, c_int64, c_int, _P], c_int),
     "fsie_bias_add": ([_P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_rope_kv_write": ([_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
                             c_int, _P], c_int),
     "fsie_gemm": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
-    "fsie_gemm_mfma_skinny": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_gemm_mfma_skinny": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_attention_scalar": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
                                c_int, c_int, c_float, c_int, _P], c_int),
     "fsie_attention_mfma": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,

@@ -218,4 +218,4 @@ class GQAttention(Mixer):
                                  plan.n_small + plan.n_large, out, *args)
         if plan.n_merges:
             ops.attention_merge(partials, plan.merges, plan.n_merges, out, self.n_heads, self.head_dim)
-        return self.o(out)
+        return self.o.for_residual(out, ctx)

@@ -40,8 +40,10 @@ class ParamDecl:
 
 
 class HiddenState:
-    """The residual stream of a step: ``residual`` float32 [T, H] and a pending ``delta``
-    [T, H] in the compute dtype that has not been added yet."""
+    """The residual stream of a step: ``residual`` float32 [T, H] and a pending ``delta`` that has
+    not been added yet: [T, H] in the compute dtype, or (only if every norm of the model sets
+    ``adds_partial_sums``, which the step's context then says in ``partial_sums_ok``) float32
+    [S, T, H], partial sums of a matrix product to be added in order."""
 
     __slots__ = ("residual", "delta")
 
@@ -62,6 +64,8 @@ class Part:
 
 class Norm(Part):
     kind = "norm"
+    # True if the norm also takes a pending delta that comes as float32 partial sums [S, T, H]
+    adds_partial_sums = False
 
     def __call__(self, hidden: HiddenState, out_dtype: torch.dtype) -> torch.Tensor:
         raise NotImplementedError

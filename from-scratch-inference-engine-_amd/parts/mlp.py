@@ -50,4 +50,4 @@ class SwiGLU(FeedForward):
             act = ops.gemm_mfma_skinny(x, self.gate_up.weight, epilogue="swiglu")
         else:
             act = ops.swiglu(self.gate_up(x))
-        return self.down(act)
+        return self.down.for_residual(act, ctx)

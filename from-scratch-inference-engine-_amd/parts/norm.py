@@ -16,6 +16,8 @@ class RMSNorm(Norm):
     eps inside the square root, the weight multiplied last, plain w (the reference's rms_norm,
     src/model/nn.cpp:45-72, which sums in float64)."""
 
+    adds_partial_sums = True
+
     def __init__(self, hidden_size: int, eps: float):
         self.hidden_size = hidden_size
         self.eps = float(eps)

@@ -205,6 +205,43 @@ def test_graph_replays_equal_eager_steps(model_dirs):
     assert g.captures + g.replays == before
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_decoding_with_partial_sums_in_the_residual_stream(model_dirs, name, monkeypatch):
+    """The tiny models are too narrow for the projections to cut K by themselves, so the cut is
+    forced: the output and down projections then leave float32 partial sums that the next norm
+    (and the model's last one, on chosen rows) adds up.  Decoded in a batch, eagerly and through
+    graphs, against the plain implementation."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+    from from_scratch_inference_engine_amd.parts.linear import Linear
+
+    used = []
+
+    def two_if_it_fits(self, m):
+        fits = -(-(-(-self.in_features // 2)) // 64) * 64 < self.in_features
+        used.append(fits)
+        return 2 if fits else 1
+
+    monkeypatch.setattr(Linear, "residual_splits", two_if_it_fits)
+    model = load_model(model_dirs[name], dtype="bfloat16")
+    assert model.partial_sums_ok
+    vocab = plain.read_config(model_dirs[name])["vocab_size"]
+    seqs = [helpers.token_ids(vocab, 21 + 9 * i, 700 + i) for i in range(3)]
+    ref = [plain.forward_dir(model_dirs[name], ids).numpy() for ids in seqs]
+    for graphs in (False, True):
+        runner = Runner(model, page_size=4, num_pages=64, max_requests=4, use_graphs=graphs)
+        caches = [runner.manager.open(i) for i in range(3)]
+        n_pre = [len(ids) - 8 for ids in seqs]
+        runner.step([StepEntry(c, ids[:n], []) for c, ids, n in zip(caches, seqs, n_pre)])
+        for t in range(8):
+            out = runner.step([StepEntry(c, [ids[n + t]], [0]) for c, ids, n in zip(caches, seqs, n_pre)]).float().cpu()
+            for i in range(3):
+                helpers.assert_close_to_plain(out[i:i + 1].numpy(), ref[i][n_pre[i] + t:n_pre[i] + t + 1], "bfloat16",
+                                              f"{name} graphs={graphs} request {i} token {t}")
+    assert any(used)
+
+
 ODD = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
     "hidden_size": 72, "num_hidden_layers": 2, "num_attention_heads": 3, "num_key_value_heads": 3, "head_dim": 24,

@@ -133,6 +133,50 @@ def test_gemm_mfma_skinny(ops, m, n, k, waves):
     assert (out - ref).abs().max() <= tol(torch.bfloat16, ref)
 
 
+@pytest.mark.parametrize("m, n, k, splits, waves", [(1, 896, 4864, 2, 0), (8, 3584, 18944, 8, 0), (16, 100, 1032, 4, 2),
+                                                     (5, 48, 136, 2, 1), (13, 1000, 1000, 8, 4)])
+def test_gemm_mfma_skinny_partial_sums_feed_the_norm(ops, m, n, k, splits, waves):
+    """K cut into slices: the partial sums add up to the product, and the norm that takes them
+    as its delta gives what it gives for the whole product."""
+    x, w = rnd((m, k), 24, torch.bfloat16), rnd((n, k), 25, torch.bfloat16, 0.05)
+    ref = plain.linear(x.float(), w.float())
+    parts = ops.gemm_mfma_skinny(x.cuda(), w.cuda(), splits=splits, waves=waves)
+    assert parts.shape == (splits, m, n) and parts.dtype == torch.float32
+    total = parts.cpu().double().sum(0).float()
+    assert (total - ref).abs().max() <= 2e-5 * ref.abs().max()
+    # a slice holds only its own part of K (a slice that read beyond its end would not)
+    k_slice = -(-(-(-k // splits)) // 64) * 64
+    first = plain.linear(x[:, :k_slice].float(), w[:, :k_slice].float())
+    assert (parts[0].cpu() - first).abs().max() <= 2e-5 * ref.abs().max()
+    if n % 4:
+        return
+    res0, g, eps = rnd((m, n), 26), rnd((n,), 27) + 1.0, 1e-6
+    for dtype in DTYPES:
+        res = res0.clone().cuda()
+        out = ops.rmsnorm(res, g.cuda(), eps, dtype, delta=parts, write_back=True).float().cpu()
+        summed = res0 + total
+        assert (res.cpu() - summed).abs().max() <= 1e-5 * summed.abs().max()
+        want = plain.rms_norm(summed, g, eps)
+        assert (out - want).abs().max() <= tol(dtype, want)
+        rows = torch.tensor([m - 1, 0], dtype=torch.int32)
+        res = res0.clone().cuda()
+        out = ops.rmsnorm(res, g.cuda(), eps, dtype, delta=parts, rows=rows.cuda()).float().cpu()
+        assert torch.equal(res.cpu(), res0) and (out - want[rows.long()]).abs().max() <= tol(dtype, want)
+
+
+def test_rmsnorm_adds_partial_sums_at_odd_sizes(ops):
+    """Sizes the vector kernel does not take: hidden not a multiple of 4 and larger than its registers hold."""
+    for hidden, n_parts in [(102, 2), (9001 * 4, 4), (4099, 8)]:
+        x, g = rnd((3, hidden), 28), rnd((hidden,), 29) + 1.0
+        parts = rnd((n_parts, 3, hidden), 30)
+        summed = x + parts.double().sum(0).float()
+        want = plain.rms_norm(summed, g, 1e-5)
+        res = x.clone().cuda()
+        out = ops.rmsnorm(res, g.cuda(), 1e-5, torch.float32, delta=parts.cuda(), write_back=True).cpu()
+        assert (res.cpu() - summed).abs().max() <= 1e-5 * summed.abs().max()
+        assert (out - want).abs().max() <= tol(torch.float32, want)
+
+
 @pytest.mark.parametrize("m, n, k", [(1, 9728, 896), (8, 352, 64), (13, 640, 192), (16, 37888, 3584)])
 def test_gemm_mfma_skinny_with_swiglu_epilogue(ops, m, n, k):
     x, w = rnd((m, k), 17, torch.bfloat16), rnd((n, k), 18, torch.bfloat16, 0.05)
@@ -151,6 +195,10 @@ def test_refusals(ops):
         ops.gemm_mfma_skinny(x, w)
     with pytest.raises(KernelError, match="multiple of 8"):
         ops.gemm_mfma_skinny(x[:4, :60].contiguous(), w[:, :60].contiguous())
+    with pytest.raises(KernelError, match="too short for 2 slices"):
+        ops.gemm_mfma_skinny(x[:4], w, splits=2)
+    with pytest.raises(KernelError, match="partial sums come in"):
+        ops.gemm_mfma_skinny(x[:4], w, splits=3)
     with pytest.raises(KernelError, match="inner size"):
         ops.gemm(x, w[:, :32].contiguous())
     with pytest.raises(KernelError, match="contiguous"):
