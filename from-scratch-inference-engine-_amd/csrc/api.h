@@ -54,6 +54,11 @@ int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, i
 int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
                           int out_f32, int waves, int blocks, int epilogue, int splits, hipStream_t stream);
 
+int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const float* bias, void* y, int M, int K,
+                               const int32_t* positions, const int32_t* slots, const double* inv_freq, void* k_pool,
+                               void* v_pool, int n_heads, int n_kv, int head_dim, int page_size, int64_t pool_slots,
+                               hipStream_t stream);
+
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
                           void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,

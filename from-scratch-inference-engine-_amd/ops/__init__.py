@@ -6,9 +6,9 @@ computes with torch; a missing kernel library is an error, not a reason to fall 
 """
 
 from .functions import (bias_add, attention_merge, attention_mfma, attention_mfma_max_waves, attention_mfma_rows, attention_scalar, attention_tile_tokens, dtype_code,
-                        embedding, gemm, gemm_mfma_skinny, residual_add, rmsnorm, rope_kv_write, sample, swiglu)
+                        embedding, gemm, gemm_mfma_skinny, gemm_mfma_skinny_rope, residual_add, rmsnorm, rope_kv_write, sample, swiglu)
 from .library import KernelError, KernelLibraryMissing, load
 
 __all__ = ["KernelError", "KernelLibraryMissing", "attention_merge", "attention_mfma", "attention_mfma_max_waves", "attention_mfma_rows", "attention_scalar", "bias_add",
-           "attention_tile_tokens", "dtype_code", "embedding", "gemm", "gemm_mfma_skinny", "load", "residual_add",
+           "attention_tile_tokens", "dtype_code", "embedding", "gemm", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "load", "residual_add",
            "rmsnorm", "rope_kv_write", "sample", "swiglu"]

@@ -215,6 +215,44 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     return out
 
 
+def gemm_mfma_skinny_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                          positions: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
+                          inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor] = None,
+                          k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None,
+                          page_size: int = 0) -> torch.Tensor:
+    """The fused q/k/v projection x [M, K] . weight [(n_heads + 2 n_kv) head_dim, K]^T of at most 64
+    rows (bfloat16) with the position encoding in its epilogue: bias, rotation of the q and k
+    heads over the whole head (``inv_freq``: float64 [head_dim / 2], ``None`` = none) and the
+    write of k and v into the cache pools at ``slots``.  Returns [M, N] whose q columns are
+    filled; the k and v columns are not written."""
+    _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
+    _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
+    m, k = x.shape
+    n = (n_heads + 2 * n_kv) * head_dim
+    if tuple(weight.shape) != (n, k):
+        raise KernelError(f"gemm: weight shape {tuple(weight.shape)} is not [{n}, {k}]")
+    if bias is not None:
+        _need(bias, "qkv bias", dtype=torch.float32, shape=(n,))
+    _need(positions, "positions", dtype=torch.int32, shape=(m,))
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", dtype=torch.float64, shape=(head_dim // 2,))
+    pool_slots = 0
+    if k_pool is not None:
+        if v_pool is None or slots is None:
+            raise KernelError("gemm_mfma_skinny_rope: k_pool needs v_pool and slots")
+        _need(slots, "slots", dtype=torch.int32, shape=(m,))
+        _need(k_pool, "k_pool", dtype=torch.bfloat16, ndim=4)
+        _need(v_pool, "v_pool", dtype=torch.bfloat16, shape=(k_pool.shape[0], n_kv, head_dim, page_size))
+        if tuple(k_pool.shape[1:]) != (n_kv, page_size, head_dim):
+            raise KernelError(f"k_pool: shape {tuple(k_pool.shape)} is not [pages, {n_kv}, {page_size}, {head_dim}]")
+        pool_slots = k_pool.shape[0] * page_size
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    check(load().fsie_gemm_mfma_skinny_rope(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, k,
+                                            positions.data_ptr(), _ptr(slots), _ptr(inv_freq), _ptr(k_pool),
+                                            _ptr(v_pool), n_heads, n_kv, head_dim, page_size, pool_slots, _stream()))
+    return out
+
+
 def attention_tile_tokens(n_heads: int, n_kv: int) -> int:
     n = load().fsie_attention_scalar_tile_tokens(n_heads, n_kv)
     if n <= 0:

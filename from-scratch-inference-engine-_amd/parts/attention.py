@@ -191,9 +191,12 @@ class GQAttention(Mixer):
 
     # compute ----------------------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
-        qkv = self.qkv(x, skip_bias=True)
         store = KVStore(cache.k_pool, cache.v_pool, cache.slots, cache.page_size) if cache.writes else None
-        self.position.apply(qkv, self.n_heads, self.n_kv, self.head_dim, ctx, store, bias=self.qkv.bias)
+        qkv = self.position.project(x, self.qkv.weight, self.qkv.bias, self.n_heads, self.n_kv, self.head_dim, ctx,
+                                    store)
+        if qkv is None:
+            qkv = self.qkv(x, skip_bias=True)
+            self.position.apply(qkv, self.n_heads, self.n_kv, self.head_dim, ctx, store, bias=self.qkv.bias)
         plan = ctx.plan(self.planner())
         t = x.shape[0]
         out = torch.empty((t, self.q_dim), dtype=x.dtype, device=x.device)

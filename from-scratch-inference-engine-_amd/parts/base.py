@@ -104,6 +104,14 @@ class PositionEncoding(Part):
               bias: Optional[torch.Tensor] = None) -> None:
         raise NotImplementedError
 
+    def project(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], n_heads: int,
+                n_kv: int, head_dim: int, ctx, store) -> Optional[torch.Tensor]:
+        """Optional: the fused q/k/v projection of ``x`` and ``apply`` in one kernel.  Returns
+        the [T, (n_heads + 2 n_kv) head_dim] result of which the mixer reads only the q columns,
+        or None if this encoding (or these sizes) has no such kernel: the mixer then projects
+        by itself and calls ``apply``."""
+        return None
+
 
 class Block(Part):
     kind = "block"

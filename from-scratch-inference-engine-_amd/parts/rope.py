@@ -8,6 +8,7 @@ import numpy as np
 import torch
 
 from .. import ops
+from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M
 from .base import PositionEncoding, register_part
 
 
@@ -46,6 +47,17 @@ class RotaryEncoding(PositionEncoding):
         else:
             ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, slots=store.slots,
                               k_pool=store.k_pool, v_pool=store.v_pool, page_size=store.page_size, bias=bias)
+
+    def project(self, x, weight, bias, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore]):
+        """For a few rows of bfloat16 (decoding) the projection's own epilogue rotates and stores."""
+        if (x.dtype != torch.bfloat16 or not 0 < x.shape[0] <= GEMM_MFMA_SKINNY_BEST_M or x.shape[1] % 8
+                or head_dim % 16 or self.rotary_dim != head_dim):
+            return None
+        if store is None:
+            return ops.gemm_mfma_skinny_rope(x, weight, bias, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq)
+        return ops.gemm_mfma_skinny_rope(x, weight, bias, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq,
+                                         slots=store.slots, k_pool=store.k_pool, v_pool=store.v_pool,
+                                         page_size=store.page_size)
 
 
 @register_part("position", "none")

@@ -177,6 +177,47 @@ def test_rmsnorm_adds_partial_sums_at_odd_sizes(ops):
         assert (out - want).abs().max() <= tol(torch.float32, want)
 
 
+@pytest.mark.parametrize("m, heads, kv, hd, k, theta, use_bias", [
+    (1, 14, 2, 64, 896, 1e6, True), (9, 3, 3, 48, 72, 1e4, True), (16, 5, 1, 256, 320, 5e5, False),
+    (7, 28, 4, 128, 3584, 1e6, True), (33, 2, 1, 16, 64, 1e4, True)])
+def test_projection_with_rotary_epilogue(ops, m, heads, kv, hd, k, theta, use_bias):
+    """q/k/v projection, bias, rotation and cache write in one kernel, against the plain formulas
+    on the float32 product (one rounding to bfloat16, after the rotation)."""
+    page, pages = 4, 24
+    n = (heads + 2 * kv) * hd
+    x, w = rnd((m, k), 40, torch.bfloat16), rnd((n, k), 41, torch.bfloat16, 0.05)
+    bias = rnd((n,), 42) if use_bias else None
+    g = torch.Generator().manual_seed(43)
+    pos = torch.randint(0, 5000, (m,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(pages * page, generator=g)[:m].to(torch.int32)
+    slots[m // 2] = -1  # this token is not stored
+    inv = torch.tensor([theta ** (-2.0 * i / hd) for i in range(hd // 2)], dtype=torch.float64)
+    dk = torch.zeros((pages, kv, page, hd), dtype=torch.bfloat16).cuda()
+    dv = torch.zeros((pages, kv, hd, page), dtype=torch.bfloat16).cuda()
+    got = ops.gemm_mfma_skinny_rope(x.cuda(), w.cuda(), None if bias is None else bias.cuda(), pos.cuda(), heads, kv,
+                                    hd, inv.cuda(), slots=slots.cuda(), k_pool=dk, v_pool=dv, page_size=page)
+    full = plain.linear(x.float(), w.float(), bias)
+    q_ref = plain.rope(full[:, :heads * hd], heads, hd, theta, pos.tolist())
+    k_ref = plain.rope(full[:, heads * hd:(heads + kv) * hd], kv, hd, theta, pos.tolist())
+    v_ref = full[:, (heads + kv) * hd:]
+    bf = torch.bfloat16
+    assert (got.float().cpu()[:, :heads * hd] - q_ref).abs().max() <= tol(bf, q_ref)
+    kp, vp = dk.float().cpu(), dv.float().cpu()
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for i, s in enumerate(slots.tolist()):
+        if s < 0:
+            continue
+        written[s] = True
+        assert (kp[s // page, :, s % page, :].reshape(-1) - k_ref[i]).abs().max() <= tol(bf, k_ref), f"k of token {i}"
+        assert (vp[s // page, :, :, s % page].reshape(-1) - v_ref[i]).abs().max() <= tol(bf, v_ref), f"v of token {i}"
+    untouched = ~written.reshape(pages, 1, page, 1).expand_as(kp)
+    assert kp[untouched].abs().max() == 0 and vp.transpose(2, 3)[untouched].abs().max() == 0
+    # the same without a cache and without rotation: q is the product plus bias
+    got = ops.gemm_mfma_skinny_rope(x.cuda(), w.cuda(), None if bias is None else bias.cuda(), pos.cuda(), heads, kv,
+                                    hd, None)
+    assert (got.float().cpu()[:, :heads * hd] - full[:, :heads * hd]).abs().max() <= tol(bf, full)
+
+
 @pytest.mark.parametrize("m, n, k", [(1, 9728, 896), (8, 352, 64), (13, 640, 192), (16, 37888, 3584)])
 def test_gemm_mfma_skinny_with_swiglu_epilogue(ops, m, n, k):
     x, w = rnd((m, k), 17, torch.bfloat16), rnd((n, k), 18, torch.bfloat16, 0.05)
