@@ -22,8 +22,8 @@
 //
 // A workgroup may have several waves (up to MAXW; 4 when NT > 1): they split the item's key range
 // into contiguous runs of blocks, and their partial results are combined inside the workgroup:
-// maxima and sums through LDS, then the rescaled accumulators are added into one LDS tile in the
-// fixed order of the waves.  Decoding against a long context therefore needs neither partial
+// maxima and sums through LDS, then the first wave adds the others' rescaled accumulators to its
+// own in the fixed order of the waves.  Decoding against a long context therefore needs neither partial
 // records in memory nor a second kernel, and the result does not depend on timing.
 #pragma once
 
@@ -300,25 +300,30 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
         }
     }
 
-    // ---- several waves: combine inside the workgroup
-    if (MAXW > 1 && n_waves > 1) {
-        constexpr int kSlabFloats = 8192;               // 32 KB of LDS for the accumulators
-        constexpr int TP = kSlabFloats / (MAXW * 256);  // head-dim tiles per phase
-        __shared__ float s_m[NT][MAXW][16], s_l[NT][MAXW][16];
-        __shared__ float s_o[kSlabFloats];
+    // ---- the denominator and maximum of every query row; several waves combine inside the
+    // workgroup: maxima and sums through LDS, then the waves after the first lay their
+    // accumulators, rescaled to the common maximum, into LDS, and the first wave adds them to its
+    // own in the fixed order of the waves and writes the result (two barriers, no atomics)
+    float l_tot[NT], m_fin[NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            float l_w = l_run[nt];
-            l_w += __shfl_xor(l_w, 16, FSIE_WAVE);
-            l_w += __shfl_xor(l_w, 32, FSIE_WAVE);
-            if (G == 0) {
+    for (int nt = 0; nt < NT; ++nt) {
+        float l_w = l_run[nt];
+        l_w += __shfl_xor(l_w, 16, FSIE_WAVE);
+        l_w += __shfl_xor(l_w, 32, FSIE_WAVE);
+        l_tot[nt] = l_w;
+        m_fin[nt] = m_run[nt];
+    }
+    if (MAXW > 1 && n_waves > 1) {
+        __shared__ float s_m[NT][MAXW][16], s_l[NT][MAXW][16];
+        __shared__ floatx4 s_o[(MAXW - 1) * NT * HDT * 64];
+        if (G == 0) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
                 s_m[nt][wave][c] = m_run[nt];
-                s_l[nt][wave][c] = l_w;
+                s_l[nt][wave][c] = l_tot[nt];
             }
         }
         __syncthreads();
-        const int n_threads = 64 * n_waves;
-        bool first = true;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             float m_all = -INFINITY;
@@ -328,48 +333,43 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
                 const float mw = s_m[nt][w][c];
                 if (mw != -INFINITY) denom += s_l[nt][w][c] * __builtin_amdgcn_exp2f(mw - m_all);
             }
-            const float mine = (m_run[nt] == -INFINITY || !(denom > 0.f)) ? 0.f
-                               : __builtin_amdgcn_exp2f(m_run[nt] - m_all) / denom;
-            // Each active wave lays its rescaled accumulators into a slab of its own, TP tiles of
-            // the head dimension at a time; then every thread sums the slabs for a few (d, row)
-            // places of its own column in the fixed order of the waves and writes them out.
-            bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[nt]) * n_heads + rhead[nt]) * HD;
+            const float mine = (m_run[nt] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_run[nt] - m_all);
 #pragma unroll
-            for (int t0 = 0; t0 < HDT; t0 += TP) {
-                if (!first) __syncthreads();  // the slabs of the last phase have been read
-                first = false;
-                if (wave < n_active) {
-#pragma unroll
-                    for (int dt = t0; dt < t0 + TP && dt < HDT; ++dt)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            s_o[(wave * TP + (dt - t0)) * 256 + (4 * G + r) * 16 + c] = acc[nt][dt][r] * mine;
-                }
-                __syncthreads();
-                const int n_out = (min(TP, HDT - t0)) * 256;  // (d, row) places of this phase
-                for (int idx = threadIdx.x; idx < n_out; idx += n_threads) {  // idx % 16 == c
-                    const int tile = idx >> 8, within = idx & 255;
-                    float sum = 0.f;
-                    for (int w = 0; w < n_active; ++w) sum += s_o[(w * TP + tile) * 256 + within];
-                    if (rvalid[nt]) {
-                        const int d = (t0 + tile) * 16 + (within >> 4);
-                        o[d] = from_float<bf16_t>(sum);
-                    }
-                }
+            for (int dt = 0; dt < HDT; ++dt) {
+                acc[nt][dt][0] *= mine;
+                acc[nt][dt][1] *= mine;
+                acc[nt][dt][2] *= mine;
+                acc[nt][dt][3] *= mine;
             }
+            if (wave > 0 && wave < n_active) {
+#pragma unroll
+                for (int dt = 0; dt < HDT; ++dt) s_o[(((wave - 1) * NT + nt) * HDT + dt) * 64 + lane] = acc[nt][dt];
+            }
+            l_tot[nt] = denom;
+            m_fin[nt] = m_all;
         }
-        return;
+        __syncthreads();
+        if (wave > 0) return;
+        for (int w = 1; w < n_active; ++w) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int dt = 0; dt < HDT; ++dt) {
+                    const floatx4 v = s_o[(((w - 1) * NT + nt) * HDT + dt) * 64 + lane];
+                    acc[nt][dt][0] += v[0];
+                    acc[nt][dt][1] += v[1];
+                    acc[nt][dt][2] += v[2];
+                    acc[nt][dt][3] += v[3];
+                }
+        }
     }
 
-    // ---- results: lane holds O^T[d = 16 dt + 4 G + r][row c]
+    // ---- results: lane holds O^T[d = 16 dt + 4 G + r][row c], relative to the maximum m_fin
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        float l_tot = l_run[nt];
-        l_tot += __shfl_xor(l_tot, 16, FSIE_WAVE);
-        l_tot += __shfl_xor(l_tot, 32, FSIE_WAVE);
         if (!rvalid[nt]) continue;
         if (partial_base < 0) {
-            const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+            const float inv = l_tot[nt] > 0.f ? 1.0f / l_tot[nt] : 0.f;
             bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[nt]) * n_heads + rhead[nt]) * HD + 4 * G;
 #pragma unroll
             for (int dt = 0; dt < HDT; ++dt) {
@@ -379,14 +379,16 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
                 *reinterpret_cast<uint2*>(o + dt * 16) = w;
             }
         } else {
+            // the item is one of several that share a query's keys: unnormalised sums, their
+            // maximum (in natural units) and denominator, for attention_merge
             float* rec = partials + (static_cast<int64_t>(partial_base + rtok[nt]) * n_heads + rhead[nt]) * (HD + 2);
 #pragma unroll
             for (int dt = 0; dt < HDT; ++dt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) rec[dt * 16 + 4 * G + r] = acc[nt][dt][r];
             if (G == 0) {
-                rec[HD] = m_run[nt] * kLn2;  // back to natural units for the merge
-                rec[HD + 1] = l_tot;
+                rec[HD] = m_fin[nt] * kLn2;
+                rec[HD + 1] = l_tot[nt];
             }
         }
     }

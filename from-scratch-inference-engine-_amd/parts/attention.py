@@ -24,8 +24,9 @@ class AttentionPlanner:
     the keys from the start of its window to its last token.  A portion of at most
     ``small_tokens`` tokens is one *small* item.  For the float32-arithmetic kernel a small item
     that reads more than ``split_keys`` keys (decoding against a long context) is split over the
-    keys into several items and merged afterwards in the order of the splits; the matrix-core
-    kernel splits the keys among the waves of a workgroup instead (one wave per 128 keys).  Longer portions are cut into *large*
+    keys into several items and merged afterwards in the order of the splits (256 keys an item
+    for the float32-arithmetic kernel; 1,024 for the matrix-core kernel, which gives every 128 of
+    them to a wave of the item's workgroup and combines those inside).  Longer portions are cut into *large*
     tiles of ``large_tokens``.  Whether and how a portion is cut depends on the portion alone,
     never on what else is in the batch.  The item table lists the small items first.
 
@@ -51,7 +52,9 @@ class AttentionPlanner:
                 small = max(1, ops.attention_mfma_rows(self.head_dim, False) // min(group, 16))
                 rows = ops.attention_mfma_rows(self.head_dim, True)
                 large = max(1, rows // min(group, rows))
-                self._geometry[mfma] = (small, large, None)  # keys are split inside the workgroup
+                # one compute unit draws only some 50 GB/s from memory: beyond 1,024 keys (eight
+                # waves of 128) a query's keys go to several workgroups
+                self._geometry[mfma] = (small, large, 128 * min(8, ops.attention_mfma_max_waves(self.head_dim)))
             else:
                 t = ops.attention_tile_tokens(self.n_heads, self.n_kv)
                 self._geometry[mfma] = (t, t, 256)
@@ -81,10 +84,12 @@ class AttentionPlanner:
                 return None
             first_key = max(0, host.past_lens[s] - self.window + 1) if self.window else 0
             keys = host.past_lens[s] + host.q_lens[s] - first_key
-            longest = max(longest, keys)
-            n += 1 if split_keys is None else max(1, -(-keys // split_keys))
-        if split_keys is None:
-            return (host.n_seqs, self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)))
+            longest = max(longest, min(keys, split_keys))
+            n += max(1, -(-keys // split_keys))
+        if mfma:
+            # items: a multiple of the number of requests (the captured graph pads with empty ones)
+            return (-(-n // host.n_seqs) * host.n_seqs,
+                    self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)))
         step = 4 * host.n_seqs
         return (-(-n // step) * step, 1)
 
