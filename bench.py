@@ -90,9 +90,13 @@ def main() -> int:
     page = 16
     context = raw["max_position_embeddings"]
     biggest = max(args.batch, 1 if args.no_points else 64)
-    per_req = args.prompt_len + args.steps + args.warmup + 2 * page
+    budget = 2048  # tokens a step may hold: the prompts of a large batch enter over several steps
+    # requests whose prompt went in first decode while the others' prompts still enter: they get
+    # that many more tokens, so that nobody ends inside the timed steps
+    head_start = -(-biggest * args.prompt_len // budget) + 1
+    per_req = args.prompt_len + args.steps + args.warmup + head_start + 2 * page
     num_blocks = max(biggest * -(-per_req // page), -(-2048 // page) * 2) + 64
-    engine = Engine(model, block_size=page, num_blocks=num_blocks, max_batch=biggest, max_tokens_per_step=2048)
+    engine = Engine(model, block_size=page, num_blocks=num_blocks, max_batch=biggest, max_tokens_per_step=budget)
     gen = torch.Generator().manual_seed(0)
 
     def prompts(n, length):
@@ -118,7 +122,7 @@ def main() -> int:
 
     # ---- decode
     def decode(batch, steps, warmup):
-        ids = [engine.add_request(p, SamplingParams(temperature=0.0), max_tokens=steps + warmup + 1)
+        ids = [engine.add_request(p, SamplingParams(temperature=0.0), max_tokens=steps + warmup + head_start + 1)
                for p in prompts(batch, args.prompt_len)]
         while any(len(engine.output(i)) == 0 for i in ids):  # prompts in portions of the token budget
             engine.step()

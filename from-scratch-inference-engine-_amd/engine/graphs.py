@@ -24,7 +24,7 @@ class DecodeGraphs:
     def __init__(self, runner, max_graphs: int = 64):
         self.runner = runner
         self.max_graphs = max_graphs
-        self._graphs: Dict[Tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor]] = {}
+        self._graphs: Dict[Tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
         model = runner.model
         self.enabled = all(getattr(block.mixer, "graph_safe", False) for block in model.spec.layers) and all(
             hasattr(p, "graph_bucket") for p in model.planners)
@@ -46,9 +46,10 @@ class DecodeGraphs:
             pad[planner.key] = bucket
         return pad
 
-    def step(self, entries: Sequence[StepEntry], pad: dict) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], pad: dict, feed: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run the (already reserved) decode step through its graph; returns the logits, which
-        stay valid until the next step of the same shape."""
+        stay valid until the next step of the same shape.  ``feed`` (int32, on the device)
+        replaces the token ids after the tables have been sent."""
         runner = self.runner
         key = (len(entries),) + tuple(sorted((str(k), v) for k, v in pad.items()))
         hit = self._graphs.get(key)
@@ -59,20 +60,24 @@ class DecodeGraphs:
             # the library's kernel selection
             ctx, tables = build_context(entries, runner.manager, runner.model.planners, runner._staging,
                                         runner.model.dtype, runner.model.device, pad=pad)
+            if feed is not None:
+                ctx.token_ids.copy_(feed)
             runner.model.forward(ctx, runner.storage)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = runner.model.forward(ctx, runner.storage)
-            self._graphs[key] = (graph, tables, logits)
+            self._graphs[key] = (graph, tables, logits, ctx.token_ids)
             self.captures += 1
             # the eager run above already wrote this step's keys and values; replaying writes the
             # same values again
             graph.replay()
             return logits
-        graph, tables, logits = hit
+        graph, tables, logits, token_ids = hit
         build_context(entries, runner.manager, runner.model.planners, runner._staging, runner.model.dtype,
                       runner.model.device, pad=pad, into=tables)
+        if feed is not None:
+            token_ids.copy_(feed)
         graph.replay()
         self.replays += 1
         return logits

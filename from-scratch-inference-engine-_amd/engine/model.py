@@ -192,11 +192,17 @@ class Runner:
                 raise ValueError(f"step: request {e.cache.request_id!r} would reach {e.cache.length + n} "
                                  f"positions, more than max_position_embeddings {self.max_position}")
 
-    def step(self, entries: Sequence[StepEntry], keep: bool = True) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], keep: bool = True,
+             feed: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run one batch.  Nothing is changed when the batch is refused (bad ids, no pages).
         ``keep=False`` allows the returned logits to live in a buffer that the next step
-        overwrites (a caller that consumes them at once saves a copy)."""
+        overwrites (a caller that consumes them at once saves a copy).  ``feed``: an int32 device
+        tensor with one token id per token of the batch, used instead of the entries' ids (which
+        only stand in): ids that an earlier step has sampled and the host has not read yet."""
         self.check(entries)
+        if feed is not None and (feed.dtype != torch.int32 or feed.ndim != 1 or
+                                 feed.shape[0] != sum(len(e.tokens) for e in entries)):
+            raise ValueError("step: feed must hold one int32 token id per token of the batch")
         if not self.manager.can_reserve((e.cache, len(e.tokens)) for e in entries):
             raise OutOfPages("step: the batch needs more pages than the pool has free")
         for e in entries:
@@ -204,12 +210,14 @@ class Runner:
         self.storage.reset_states([e.cache.slot for e in entries if e.cache.length == 0])
         pad = self.graphs.shape_of(entries) if self.graphs is not None else None
         if pad is not None:
-            logits = self.graphs.step(entries, pad)
+            logits = self.graphs.step(entries, pad, feed)
             if keep:
                 logits = logits.clone()
         else:
             ctx, _ = build_context(entries, self.manager, self.model.planners, self._staging, self.model.dtype,
                                    self.model.device)
+            if feed is not None:
+                ctx.token_ids.copy_(feed)
             logits = self.model.forward(ctx, self.storage)
         for e in entries:
             self.manager.commit(e.cache, len(e.tokens))

@@ -17,6 +17,14 @@ Policy (the reference's, src/engine/engine.cpp:53-178, plus a token budget and p
   * a request that could never fit the pool (or max_position_embeddings) is refused when added;
   * after sampling, a request ends on its end-of-sequence token (which is kept in the output)
     or at ``max_tokens``; its pages and slot go back at once.
+
+Running ahead: while the samples of a launched step are still on their way to the host,
+``lookahead`` names the step that follows it, if that does not depend on them: every running
+request decodes, none can reach ``max_tokens`` with the pending sample, nobody waits to be
+admitted and every request finds a page for one more token.  The engine launches that step with
+the token ids taken from the device.  A request that turns out to have ended on its
+end-of-sequence token has then run one token too far; that token is dropped, and what it wrote
+lies beyond the request's end in pages that go back with the rest.
 """
 
 from __future__ import annotations
@@ -74,6 +82,7 @@ class ScheduledItem:
     seq: Sequence
     tokens: List[int]
     wants_logits: bool
+    ahead: bool = False  # launched before the sample that gives its token was read (ids from the device)
 
 
 class Scheduler:
@@ -197,12 +206,33 @@ class Scheduler:
             if items or len(self.running) <= 1 or not self._preempt_youngest():
                 return items
 
+    def lookahead(self, items: List[ScheduledItem]) -> Optional[List[ScheduledItem]]:
+        """The step after ``items`` (launched, samples not read yet), or None if it cannot be
+        told without them.  Its tokens are stand-ins: the ids come from the device."""
+        if self.waiting or not items or len(items) != len(self.running) or len(items) > self.max_tokens_per_step:
+            return None
+        taken = [0] * len(self.manager.groups)
+        for item, sid in zip(items, self.running):
+            seq = item.seq
+            if seq.id != sid or not item.wants_logits or seq.status != SeqStatus.Running or seq.cache is None:
+                return None
+            if seq.remaining != 0:
+                return None  # not everything it has is computed: it is still in its prompt
+            if len(seq.output) + 1 >= seq.request.max_tokens:
+                return None  # the pending sample is its last token
+            for g, k in enumerate(self.manager.new_pages_needed(seq.cache, 1)):
+                taken[g] += k
+        if any(taken[g] > self.manager.free_pages(g) for g in range(len(taken))):
+            return None
+        return [ScheduledItem(item.seq, [0], True, ahead=True) for item in items]
+
     def finish_step(self, items: List[ScheduledItem], sampled: List[Optional[int]]) -> List[int]:
         """Record the tokens sampled for the items that wanted logits (``None`` for the others);
-        returns the ids of the requests that finished."""
+        returns the ids of the requests that finished.  The sample of a request that has ended
+        meanwhile (it had run ahead) is dropped."""
         done = []
         for item, token in zip(items, sampled):
-            if not item.wants_logits:
+            if not item.wants_logits or item.seq.status != SeqStatus.Running:
                 continue
             seq = item.seq
             seq.output.append(int(token))

@@ -42,17 +42,23 @@ class Sampler:
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], request_ids: Sequence[int],
                indices: Sequence[int]) -> List[int]:
         """One token per row of ``logits`` [n, vocab] (float32, on the device)."""
+        if logits.shape[0] == 0:
+            return []
+        return self.sample_on_device(logits, params, request_ids, indices).tolist()
+
+    def sample_on_device(self, logits: torch.Tensor, params: Sequence[SamplingParams], request_ids: Sequence[int],
+                         indices: Sequence[int]) -> torch.Tensor:
+        """The same, left on the device (int32 [n]) and not waited for: the caller reads it when
+        it needs the ids, and the next step may take them from there meanwhile."""
         n = logits.shape[0]
         if not (len(params) == len(request_ids) == len(indices) == n):
             raise ValueError("sample: one set of parameters, request id and index per row")
-        if n == 0:
-            return []
         if all(p.greedy for p in params):
-            return ops.sample(logits).tolist()
+            return ops.sample(logits)
         dev = logits.device
         temperature = torch.tensor([max(float(p.temperature), 0.0) for p in params], dtype=torch.float32, device=dev)
         top_k = torch.tensor([int(p.top_k) for p in params], dtype=torch.int32, device=dev)
         top_p = torch.tensor([float(p.top_p) for p in params], dtype=torch.float32, device=dev)
         uniform = torch.tensor([uniform_for(self.seed, r, i) for r, i in zip(request_ids, indices)],
                                dtype=torch.float64, device=dev)
-        return ops.sample(logits, temperature, top_k, top_p, uniform).tolist()
+        return ops.sample(logits, temperature, top_k, top_p, uniform)

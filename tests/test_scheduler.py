@@ -178,3 +178,119 @@ def test_many_requests_small_pool_all_finish():
     for sid, n in want.items():
         assert s.sequences[sid].output == [100 + k for k in range(n)]
     assert m.free_pages() == 6 and m.free_slots == 4
+
+
+# ------------------------------------------------------------------ running one step ahead
+def launch(m, items):
+    """Queue a step as the engine does: pages reserved and lengths advanced at once."""
+    assert m.can_reserve([(it.seq.cache, len(it.tokens)) for it in items])
+    for it in items:
+        m.reserve(it.seq.cache, len(it.tokens))
+        m.commit(it.seq.cache, len(it.tokens))
+    return items
+
+
+def run_pipelined(m, s, token_of, ahead_log=None):
+    """The engine's loop with one step queued ahead; the token of a sample depends only on the
+    request and on how many it has, as in ``run_step``."""
+    pending, steps = None, 0
+    while s.has_work() or pending is not None:
+        if pending is not None and not any(it.wants_logits and it.seq.status == SeqStatus.Running for it in pending):
+            pending = None
+        if pending is None:
+            items = s.schedule()
+            if not items:
+                break
+            pending = launch(m, items)
+        items = pending
+        # the samples "on the device": fixed before the next step is queued (the step before this
+        # one has been read by now, so a sample's index is the length of the output)
+        samples = [token_of(it.seq, len(it.seq.output)) if it.wants_logits else None for it in items]
+        nxt = s.lookahead(items)
+        pending = launch(m, nxt) if nxt is not None else None
+        if ahead_log is not None:
+            ahead_log.append(nxt is not None)
+        s.finish_step(items, samples)
+        m.check_invariants()
+        steps += 1
+        assert steps < 1000
+    return steps
+
+
+def test_lookahead_only_when_the_next_step_is_certain():
+    m, s = make(num_pages=32, budget=6)
+    a = s.add_request(Request([1, 2, 3, 4, 5, 6, 7, 8], max_tokens=4))
+    items = launch(m, s.schedule())
+    assert not items[0].wants_logits and s.lookahead(items) is None      # still in its prompt
+    s.finish_step(items, [None])
+    items = launch(m, s.schedule())
+    assert items[0].wants_logits
+    b = s.add_request(Request([9], max_tokens=1))
+    assert s.lookahead(items) is None                                    # somebody waits to be admitted
+    s.finish_step(items, [100])
+    items = launch(m, s.schedule())                                      # a decodes, b's prompt
+    assert [it.seq.id for it in items] == [a, b]
+    assert s.lookahead(items) is None                                    # b's pending sample is its last
+    s.finish_step(items, [101, 200])
+    assert s.sequences[b].status == SeqStatus.Finished
+    items = launch(m, s.schedule())
+    assert s.lookahead(items) is not None                                # a alone: third of four
+
+
+def test_lookahead_steps_and_limits():
+    m, s = make(num_pages=32)
+    a = s.add_request(Request([1, 2, 3], max_tokens=4))
+    b = s.add_request(Request([4], max_tokens=6))
+    items = launch(m, s.schedule())
+    nxt = s.lookahead(items)
+    assert nxt is not None and [(it.seq.id, it.tokens, it.wants_logits, it.ahead) for it in nxt] == \
+        [(a, [0], True, True), (b, [0], True, True)]
+    launch(m, nxt)
+    assert s.sequences[a].remaining == -1                                # one token ahead of its output
+    s.finish_step(items, [100, 200])
+    assert s.sequences[a].remaining == 0
+    nxt2 = s.lookahead(nxt)
+    assert nxt2 is not None
+    launch(m, nxt2)
+    s.finish_step(nxt, [101, 201])
+    nxt3 = s.lookahead(nxt2)                                             # a's pending sample is its third of four
+    assert nxt3 is not None
+    launch(m, nxt3)
+    s.finish_step(nxt2, [102, 202])
+    assert s.lookahead(nxt3) is None                                     # a's pending sample is its last
+    s.finish_step(nxt3, [103, 203])
+    assert s.sequences[a].status == SeqStatus.Finished and s.sequences[b].output == [200, 201, 202, 203]
+    m.check_invariants()
+
+
+def test_lookahead_needs_a_page_for_every_request():
+    m, s = make(num_pages=3, page_size=2)
+    s.add_request(Request([1, 2], max_tokens=3))
+    s.add_request(Request([3, 4], max_tokens=3))
+    items = launch(m, s.schedule())
+    assert len(items) == 2 and m.free_pages() == 1
+    assert s.lookahead(items) is None                                    # both need a new page for one more token
+
+
+def test_pipelined_loop_gives_the_same_outputs_and_frees_everything():
+    def token_of(seq, index):
+        return 7 if (seq.id * 5 + index) % 11 == 3 else 100 + index     # some requests meet their eos
+
+    outs = []
+    for pipelined in (False, True):
+        m, s = make(num_pages=24, page_size=2, budget=9, max_batch=4)
+        for i in range(10):
+            n = 1 + (i * 3) % 6
+            s.add_request(Request(list(range(1, n + 1)), max_tokens=1 + (i * 7) % 9, eos_id=7))
+        log = []
+        if pipelined:
+            run_pipelined(m, s, token_of, log)
+            assert any(log) and not all(log)
+        else:
+            while s.has_work():
+                run_step(m, s, token_of=lambda seq: token_of(seq, len(seq.output)))
+        assert m.free_pages() == 24 and m.free_slots == 4
+        outs.append({sid: list(q.output) for sid, q in s.sequences.items()})
+        assert all(q.status == SeqStatus.Finished for q in s.sequences.values())
+    assert outs[0] == outs[1]
+    assert any(o[-1] == 7 and len(o) > 1 for o in outs[0].values())     # an eos was found one step late
