@@ -27,6 +27,8 @@ def _common(p: argparse.ArgumentParser) -> None:
     p.add_argument("--top-k", type=int, default=0)
     p.add_argument("--top-p", type=float, default=1.0)
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--tune-gemms", action="store_true",
+                   help="time the library's kernels for the prefill products once per shape (seconds) and keep the best")
     p.add_argument("--json", action="store_true", help="emit results as JSON")
 
 
@@ -36,7 +38,8 @@ def _llm(args):
     if not args.model_dir:
         raise SystemExit("--model-dir (or $ENGINE_MODEL_DIR) is required")
     return LLM(args.model_dir, block_size=args.block_size, num_blocks=args.num_blocks, seed=args.seed,
-               max_batch=args.max_batch, dtype=args.dtype, max_tokens_per_step=args.max_tokens_per_step)
+               max_batch=args.max_batch, dtype=args.dtype, max_tokens_per_step=args.max_tokens_per_step,
+               tune_gemms=args.tune_gemms)
 
 
 def _prompts(args, llm):

@@ -49,9 +49,15 @@ class LLM:
     def __init__(self, model_dir, *, block_size: int = 16, num_blocks: int = 2048, seed: int = 0,
                  max_batch: int = 256, eos_id: Optional[int] = None, enable_prefix_cache: bool = True,
                  quantize: bool = False, dtype: str = "bfloat16", device: str = "cuda:0",
-                 max_tokens_per_step: int = 2048, prefill_chunk: Optional[int] = None):
+                 max_tokens_per_step: int = 2048, prefill_chunk: Optional[int] = None, tune_gemms: bool = False):
         if quantize:
             raise NotImplementedError("LLM: quantized weights are not part of this engine")
+        if tune_gemms:
+            # bfloat16 prefill: let torch time the library's kernels for each new product shape of
+            # a full token budget (seconds, once per shape) instead of trusting its heuristic
+            from ..ops import enable_library_tuning
+
+            enable_library_tuning()
         model_dir = Path(model_dir)
         self.model = Model.from_pretrained(model_dir, dtype=dtype, device=device)
         self.engine = Engine(self.model, block_size, num_blocks, seed, max_batch, enable_prefix_cache,

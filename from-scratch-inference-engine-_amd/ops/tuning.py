@@ -1,0 +1,64 @@
+"""The library matrix product of the bfloat16 path, with optional selection of the library's kernel.
+
+For many rows (prefill) the engine hands x . W^T to the vendor library through ``torch.mm`` (the
+reference's engine calls cuBLAS there).  The library picks one of its kernels by a heuristic; its
+other kernels are sometimes a good deal faster (measured on MI355X at 2,048 rows: 462 against
+568 us for N = 37888, K = 3584, and 261 against 357 us for N = 3584, K = 18944).  With tuning on,
+torch's TunableOp times the library's candidates the first time a shape is seen and keeps the
+best (in the process, and in a file under the temporary folder for later ones).  Only row counts that are a multiple of 256 are tuned (a full
+token budget; each new shape costs seconds), never inside a graph capture; other shapes use what
+has been found for them, or the heuristic.
+"""
+
+from __future__ import annotations
+
+import os
+import tempfile
+
+import torch
+
+_TUNED_ROWS = 256
+_state = {"on": False}
+
+
+def enable_library_tuning(max_ms_per_candidate: int = 30, iterations: int = 10) -> None:
+    import torch.cuda.tunable as tunable
+
+    tunable.enable(True)
+    tunable.tuning_enable(False)
+    tunable.set_max_tuning_duration(int(max_ms_per_candidate))
+    tunable.set_max_tuning_iterations(int(iterations))
+    # torch also keeps the results in a file; it goes to the temporary folder, under the user's id
+    # (the working directory may be read-only), and a later process starts from it
+    name = f"fsie-tunableop-{os.getuid()}.csv"
+    tunable.set_filename(os.path.join(tempfile.gettempdir(), name))
+    _state["on"] = True
+
+
+def disable_library_tuning() -> None:
+    import torch.cuda.tunable as tunable
+
+    tunable.tuning_enable(False)
+    tunable.enable(False)
+    _state["on"] = False
+
+
+def library_tuning_enabled() -> bool:
+    return _state["on"]
+
+
+def library_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """x [M, K] . weight [N, K]^T in the operands' dtype, float32 accumulation, by the library."""
+    if not _state["on"]:
+        return torch.mm(x, weight.t())
+    import torch.cuda.tunable as tunable
+
+    rows = x.shape[0]
+    tune = rows >= _TUNED_ROWS and rows % _TUNED_ROWS == 0 and not torch.cuda.is_current_stream_capturing()
+    if not tune:
+        return torch.mm(x, weight.t())
+    tunable.tuning_enable(True)
+    try:
+        return torch.mm(x, weight.t())
+    finally:
+        tunable.tuning_enable(False)

@@ -7,6 +7,7 @@ from typing import Optional
 import torch
 
 from .. import ops
+from ..ops.tuning import library_mm
 from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M, GEMM_MFMA_SKINNY_MAX_M, GEMM_SKINNY_MAX_M
 
 
@@ -39,7 +40,7 @@ class Linear:
             # few rows with an odd inner size; float32 results from bfloat16 operands (logits of
             # many rows); and sizes whose rows are not 16-byte aligned, which the library is not given
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
-        y = torch.mm(x, w.t())
+        y = library_mm(x, w)
         if bias is not None:
             ops.bias_add(y, bias)
         return y

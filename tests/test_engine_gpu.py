@@ -242,6 +242,26 @@ def test_decoding_with_partial_sums_in_the_residual_stream(model_dirs, name, mon
     assert any(used)
 
 
+def test_prefill_with_the_library_kernel_selection(model_dirs):
+    """With tuning on, a prompt portion of a multiple of 256 rows lets torch time the library's
+    candidates for its products; whatever it picks, the logits stay those of the plain model."""
+    from from_scratch_inference_engine_amd import load_model, ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    vocab = plain.read_config(model_dirs["B"])["vocab_size"]
+    ids = helpers.token_ids(vocab, 256, 810)
+    ref = plain.forward_dir(model_dirs["B"], ids).numpy()
+    ops.enable_library_tuning(max_ms_per_candidate=5, iterations=2)
+    try:
+        assert ops.library_tuning_enabled()
+        runner = Runner(load_model(model_dirs["B"], dtype="bfloat16"), page_size=16, num_pages=32, max_requests=2)
+        out = runner.step([StepEntry(runner.manager.open("a"), ids, list(range(256)))]).float().cpu().numpy()
+    finally:
+        ops.disable_library_tuning()
+    helpers.assert_close_to_plain(out, ref, "bfloat16", "prefill of 256 rows with library tuning")
+
+
 ODD = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
     "hidden_size": 72, "num_hidden_layers": 2, "num_attention_heads": 3, "num_key_value_heads": 3, "head_dim": 24,
