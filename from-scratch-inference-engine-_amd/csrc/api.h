@@ -71,6 +71,11 @@ int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, con
                         const int32_t* block_tables, int max_pages, const int32_t* items, int n_items, void* out,
                         float* partials, int n_heads, int n_kv, int head_dim, int page_size, int window, float scale,
                         int large, int waves, hipStream_t stream);
+int fsie_attention_mfma_lds_ok(int head_dim, int page_size);
+int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                            const int32_t* block_tables, int max_pages, const int32_t* items, const int32_t* groups,
+                            int n_groups, void* out, int n_heads, int n_kv, int head_dim, int page_size, int window,
+                            float scale, hipStream_t stream);
 int fsie_attention_mfma_tiles(int head_dim, int large);
 int fsie_attention_mfma_max_waves(int head_dim);
 

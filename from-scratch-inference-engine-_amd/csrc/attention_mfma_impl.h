@@ -231,8 +231,7 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
                         m_loc = fmaxf(m_loc, sv[t * 4 + r]);
                     }
             }
-            m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 16, FSIE_WAVE));
-            m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32, FSIE_WAVE));
+            m_loc = max_xor32(max_xor16(m_loc));
             const float m_new = fmaxf(m_run[nt], m_loc);
             const float corr = (m_run[nt] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[nt] - m_new);
             float p[8];
@@ -308,14 +307,13 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         float l_w = l_run[nt];
-        l_w += __shfl_xor(l_w, 16, FSIE_WAVE);
-        l_w += __shfl_xor(l_w, 32, FSIE_WAVE);
+        l_w = sum_xor32(sum_xor16(l_w));
         l_tot[nt] = l_w;
         m_fin[nt] = m_run[nt];
     }
     if (MAXW > 1 && n_waves > 1) {
         __shared__ float s_m[NT][MAXW][16], s_l[NT][MAXW][16];
-        __shared__ floatx4 s_o[(MAXW - 1) * NT * HDT * 64];
+        __shared__ floatx4 s_o[(MAXW > 1 ? MAXW - 1 : 1) * NT * HDT * 64];
         if (G == 0) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -406,10 +404,19 @@ int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_po
     const dim3 grid(n_items, n_kv * head_chunks);
     if (waves < 1) waves = 1;
     if (waves > MAXW) waves = MAXW;
-    attention_mfma_kernel<HDT, NT, MAXW><<<grid, 64 * waves, 0, stream>>>(
-        static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
-        block_tables, max_pages, items, static_cast<bf16_t*>(out), partials, n_heads, n_kv, page_size, window, scale,
-        gh, head_chunks);
+    // a launch of one wave per workgroup takes the instantiation without the LDS of the
+    // combination, which would otherwise limit how many workgroups a compute unit holds
+    if (waves == 1) {
+        attention_mfma_kernel<HDT, NT, 1><<<grid, 64, 0, stream>>>(
+            static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool),
+            static_cast<const bf16_t*>(v_pool), block_tables, max_pages, items, static_cast<bf16_t*>(out), partials,
+            n_heads, n_kv, page_size, window, scale, gh, head_chunks);
+    } else {
+        attention_mfma_kernel<HDT, NT, MAXW><<<grid, 64 * waves, 0, stream>>>(
+            static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool),
+            static_cast<const bf16_t*>(v_pool), block_tables, max_pages, items, static_cast<bf16_t*>(out), partials,
+            n_heads, n_kv, page_size, window, scale, gh, head_chunks);
+    }
     FSIE_CHECK_LAUNCH("attention_mfma");
     return 0;
 }

@@ -64,6 +64,27 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// This lane's value combined with that of lane ^ 16 or lane ^ 32, through the lane swaps of
+// gfx950 (v_permlane16_swap, v_permlane32_swap): two register moves, no trip through LDS as
+// a general shuffle takes.
+typedef unsigned fsie_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float max_xor16(float v) {
+    const fsie_u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_xor32(float v) {
+    const fsie_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_xor16(float v) {
+    const fsie_u2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+    const fsie_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result.  `scratch` holds at
 // least 16 floats of LDS and may be reused after the call returns.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

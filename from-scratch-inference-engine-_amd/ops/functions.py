@@ -331,6 +331,40 @@ def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
     return out
 
 
+def attention_mfma_lds_ok(head_dim: int, page_size: int) -> bool:
+    """Whether the kernel that shares a block of keys among four waves takes this geometry."""
+    return bool(load().fsie_attention_mfma_lds_ok(head_dim, page_size))
+
+
+def attention_mfma_lds(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                       block_tables: torch.Tensor, items: torch.Tensor, groups: torch.Tensor, n_groups: int,
+                       out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, window: Optional[int], scale: float,
+                       n_query_rows: int) -> torch.Tensor:
+    """Attention of large work items (long portions) with the keys and values of a block staged in
+    LDS for four tiles at once.  ``groups`` int32 [n, 2]: index in ``items`` of a group's first
+    tile and its number of tiles (1..4, consecutive tiles of one request)."""
+    if not q.is_cuda or q.dtype != torch.bfloat16:
+        raise KernelError("attention_mfma_lds q: must be bfloat16 on the GPU")
+    _need(k_pool, "k_pool", dtype=q.dtype, ndim=4)
+    _need(v_pool, "v_pool", dtype=q.dtype, shape=(k_pool.shape[0], k_pool.shape[1], k_pool.shape[3], k_pool.shape[2]))
+    _need(block_tables, "block_tables", dtype=torch.int32, ndim=2)
+    _need(items, "attention items", dtype=torch.int32, ndim=2)
+    _need(groups, "attention groups", dtype=torch.int32, ndim=2)
+    if items.shape[1] != ATTN_ITEM_INTS or groups.shape[1] != 2 or groups.shape[0] < n_groups:
+        raise KernelError(f"attention: items {tuple(items.shape)} / groups {tuple(groups.shape)} do not hold {n_groups} groups")
+    _need(out, "attention out", dtype=q.dtype, shape=(n_query_rows, n_heads * head_dim))
+    pages, kvh, page_size, hd = k_pool.shape
+    if kvh != n_kv or hd != head_dim:
+        raise KernelError(f"k_pool: shape {tuple(k_pool.shape)} does not match kv heads {n_kv}, head_dim {head_dim}")
+    if q_stride < n_heads * head_dim:
+        raise KernelError("attention: q_stride is smaller than the query width")
+    check(load().fsie_attention_mfma_lds(q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+                                         block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(),
+                                         groups.data_ptr(), n_groups, out.data_ptr(), n_heads, n_kv, head_dim,
+                                         page_size, int(window or 0), float(scale), _stream()))
+    return out
+
+
 def attention_merge(partials: torch.Tensor, merges: torch.Tensor, n_merges: int, out: torch.Tensor,
                     n_heads: int, head_dim: int) -> torch.Tensor:
     _need(partials, "attention partials", dtype=torch.float32, ndim=1)

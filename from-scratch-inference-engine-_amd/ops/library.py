@@ -41,6 +41,9 @@ _SIGNATURES = {
     "fsie_attention_mfma": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
                              c_int, c_int, c_float, c_int, c_int, _P], c_int),
     "fsie_attention_mfma_max_waves": ([c_int], c_int),
+    "fsie_attention_mfma_lds_ok": ([c_int, c_int], c_int),
+    "fsie_attention_mfma_lds": ([_P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int,
+                                 c_float, _P], c_int),
     "fsie_attention_mfma_tiles": ([c_int, c_int], c_int),
     "fsie_attention_merge": ([_P, _P, c_int, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_attention_scalar_tile_tokens": ([c_int, c_int], c_int),

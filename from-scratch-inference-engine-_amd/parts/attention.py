@@ -132,6 +132,15 @@ class AttentionPlanner:
                 merged = {m[0] for m in merges}
                 merges += [(row, 0, 0, 0) for row in range(host.n_tokens) if row not in merged]
                 n_partial = n_items * small_tokens
+        # consecutive large tiles of one request, four at a time, for the kernel that shares the
+        # keys of a block among four waves
+        groups = []
+        if mfma:
+            for i, it in enumerate(large):
+                if groups and groups[-1][1] < 4 and large[i - 1][0] == it[0] and large[i - 1][3] < it[3]:
+                    groups[-1][1] += 1
+                else:
+                    groups.append([i, 1])
         n_long = 0
         if mfma and self.long_keys is not None:
             # large tiles that read more than ``long_keys`` keys go to workgroups of four waves
@@ -141,6 +150,7 @@ class AttentionPlanner:
         return {
             "items": np.asarray(small + large, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS),
             "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
+            "groups": np.asarray(groups, dtype=np.int32).reshape(-1, 2), "n_groups": len(groups),
             "n_small": len(small), "n_large": len(large) - n_long, "n_long": n_long, "n_merges": len(merges),
             "n_partial": n_partial, "mfma": mfma, "waves": waves,
         }
@@ -154,6 +164,7 @@ class GQAttention(Mixer):
     positions a query reads (None: all)."""
 
     graph_safe = True  # forward reads the step only through device tables: a captured graph may replay it
+    share_keys = True  # long portions: four tiles of a request share each block of keys through LDS
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
                  position: PositionEncoding, window: Optional[int] = None):
@@ -214,7 +225,12 @@ class GQAttention(Mixer):
             if plan.n_small:
                 ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables, plan.items,
                                    plan.n_small, out, *args, large=False, waves=plan.waves)
-            if plan.n_large:
+            if plan.n_large and not plan.n_long and self.share_keys and ops.attention_mfma_lds_ok(self.head_dim,
+                                                                                                   cache.page_size):
+                ops.attention_mfma_lds(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
+                                       plan.items[plan.n_small:], plan.groups, plan.n_groups, out, self.n_heads,
+                                       self.n_kv, self.head_dim, self.window, self.scale, t)
+            elif plan.n_large:
                 ops.attention_mfma(qkv, qkv.shape[1], cache.k_pool, cache.v_pool, cache.block_tables,
                                    plan.items[plan.n_small:], plan.n_large, out, *args, large=True)
             if plan.n_long:

@@ -300,7 +300,9 @@ def paged_case(seqs, heads, kv, hd, page, dtype, seed, window=None, shuffle=True
                 qs=qs, ks=ks, vs=vs)
 
 
-def run_attention(ops, case, heads, kv, hd, window=None):
+def run_attention(ops, case, heads, kv, hd, window=None, share_keys=True):
+    """``share_keys``: long portions go to the kernel that stages keys in LDS for four tiles,
+    where it takes the geometry."""
     q = case["q"].cuda()
     t = q.shape[0]
     plan = case["plan"]
@@ -312,7 +314,12 @@ def run_attention(ops, case, heads, kv, hd, window=None):
     if plan["mfma"]:
         if plan["n_small"]:
             ops.attention_mfma(q, heads * hd, *pools, items, plan["n_small"], *common, large=False, waves=plan["waves"])
-        if plan["n_large"]:
+        page = case["k_pool"].shape[2]
+        if plan["n_large"] and not plan["n_long"] and share_keys and ops.attention_mfma_lds_ok(hd, page):
+            ops.attention_mfma_lds(q, heads * hd, *pools, items[plan["n_small"]:],
+                                   torch.from_numpy(plan["groups"]).cuda(), plan["n_groups"], out, heads, kv, hd,
+                                   window, 1.0 / math.sqrt(hd), t)
+        elif plan["n_large"]:
             ops.attention_mfma(q, heads * hd, *pools, items[plan["n_small"]:], plan["n_large"], *common, large=True)
         if plan["n_long"]:
             ops.attention_mfma(q, heads * hd, *pools, items[plan["n_small"] + plan["n_large"]:], plan["n_long"], *common,
@@ -347,6 +354,12 @@ def test_attention_over_pages(ops, dtype, scalar, heads, kv, hd, page, window):
         err = (out[row:row + n] - ref).abs().max().item()
         assert err <= (2e-6 if dtype == torch.float32 else 2.0 ** -7 * ref.abs().max().item()), f"seq past {p} new {n}: {err}"
         row += n
+    if not scalar and ops.attention_mfma_lds_ok(hd, page) and case["plan"]["n_large"]:
+        # the long portions went through the kernel that shares keys in LDS; the one-wave kernel
+        # must give the same up to the rounding of the probabilities
+        assert 0 < case["plan"]["n_groups"] < case["plan"]["n_large"]
+        alone = run_attention(ops, case, heads, kv, hd, window, share_keys=False)
+        assert (alone - out).abs().max() <= 2.0 ** -7 * out.abs().max()
 
 
 @pytest.mark.parametrize("dtype, scalar", [(torch.float32, True), (torch.bfloat16, False)])
