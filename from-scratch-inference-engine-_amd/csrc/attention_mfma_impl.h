@@ -5,20 +5,26 @@
 //
 //   S^T[key, row] = K[key, :] . Q[row, :]      A = K rows from the cache (16 B per lane),
 //                                              B = Q rows, kept in registers for the whole item
-//   softmax over the keys of a column: 4 keys per lane, the rest by two xor shuffles (16, 32)
+//   softmax over the keys of a column: 8 keys per lane, the rest by two lane swaps (16, 32)
 //   O^T[d, row]  += V^T[d, key] . P^T[key, row] A = V^T from the cache, which stores values
-//                                              transposed ([head_dim][slot]: 4 consecutive keys of
-//                                              one dimension are one 8-byte load),
+//                                              transposed ([head_dim][slot]: 8 consecutive keys of
+//                                              one dimension are one 16-byte load),
 //                                              B = P^T, which is exactly the layout in which the
 //                                              first product left S^T
+//
+// Keys are walked in blocks of 32, scored as two tiles of 16.  Row c of tile t is key
+// 8 (c / 4) + 4 t + c % 4 of the block: lane group G then holds, over the two tiles, the scores of
+// the keys 8 G .. 8 G + 7 in order, which is the B operand of one v_mfma_f32_16x16x32_bf16 over
+// the block's 32 keys.
 //
 // The running maximum and sum of a query row and its accumulators live in the same lanes
 // (column = lane % 16), so the online-softmax rescale is lane-local.  Scores use
 // v_mfma_f32_16x16x32_bf16 over the head dimension (16x16x16 steps when head_dim is an odd
-// multiple of 16); the second product uses 16x16x16 over 16 keys.
+// multiple of 16, on an accumulator of their own).
 //
 // HDT = head_dim / 16, NT = column tiles of 16 query rows per wave (rows = tokens x heads of the
-// kv head's group).  Keys are walked in blocks of 32.  Requires page_size % 4 == 0.
+// kv head's group).  Requires page_size % 4 == 0; with a page size that is a multiple of 8 a
+// lane's 8 values of a dimension come with one load instead of two.
 //
 // A workgroup may have several waves (up to MAXW; 4 when NT > 1): they split the item's key range
 // into contiguous runs of blocks, and their partial results are combined inside the workgroup:
@@ -58,8 +64,8 @@ constexpr int max_waves() {
     return HDT <= 4 ? 16 : (HDT <= 8 ? 8 : 4);  // registers per wave grow with the head size
 }
 
-template <int HDT, int NT, int MAXW>
-__global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
+template <int HDT, int NT, int MAXW, bool V16>
+__global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW == 1 ? 2 : 1))) void attention_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, bf16_t* __restrict__ out, float* __restrict__ partials, int n_heads,
@@ -145,8 +151,10 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
     struct Block {
         F16B kf[2][S32A];
         F8B kt[2][S16A];
-        F8B vf[2][HDT];
+        F16B vf[HDT];
     };
+    // V16: the page size is a multiple of 8, so the keys 8 G .. 8 G + 7 of a block lie in one page,
+    // 16-byte aligned (a template flag: a run-time branch around the loads costs a third of the speed)
     // Where the four runs of a block's keys lie: the two tiles of 16 keys of the scores (one key
     // per lane, c) and the two runs of 4 consecutive keys per lane group of the second product
     // (never across a page: page_size % 4 == 0).  A key without a page (past the end, or behind a
@@ -158,8 +166,8 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
         int page[4], idx[4], key[4];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            key[t] = kb + t * 16 + c;
-            key[2 + t] = kb + t * 16 + 4 * G;
+            key[t] = kb + 8 * (c >> 2) + 4 * t + (c & 3);
+            key[2 + t] = kb + 8 * G + 4 * t;
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {  // the four table reads go out together
@@ -184,11 +192,18 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
 #pragma unroll
             for (int s = 0; s < S16; ++s) blk.kt[t][s].raw = ld8(kp + s * 16);
         }
+        const bf16_t* v0 = v_pool + at.v[0];
+        if (V16) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const bf16_t* vp = v_pool + at.v[t];
+            for (int dt = 0; dt < HDT; ++dt) blk.vf[dt].raw = ld16(v0 + static_cast<int64_t>(dt * 16) * page_size);
+        } else {
+            const bf16_t* v1 = v_pool + at.v[1];
 #pragma unroll
-            for (int dt = 0; dt < HDT; ++dt) blk.vf[t][dt].raw = ld8(vp + static_cast<int64_t>(dt * 16) * page_size);
+            for (int dt = 0; dt < HDT; ++dt) {
+                const uint2 lo = ld8(v0 + static_cast<int64_t>(dt * 16) * page_size);
+                const uint2 hi = ld8(v1 + static_cast<int64_t>(dt * 16) * page_size);
+                blk.vf[dt].raw = uint4{lo.x, lo.y, hi.x, hi.y};
+            }
         }
     };
     auto compute_block = [&](int kb, const Block& blk) {
@@ -224,7 +239,7 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        const int key = kb + t * 16 + 4 * G + r;
+                        const int key = kb + 8 * G + 4 * t + r;
                         const bool vis = rvalid[nt] && key >= key_begin && key < key_end && key <= rpos[nt] &&
                                          (window <= 0 || key > rpos[nt] - window);
                         sv[t * 4 + r] = vis ? st[t][r] * scale2 : -INFINITY;
@@ -243,12 +258,8 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
             }
             l_run[nt] = l_run[nt] * corr + p_sum;  // this lane's keys only; lane groups are summed at the end
             m_run[nt] = m_new;
-            F8B pb[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                pb[t].raw.x = pack2_bf16(p[t * 4 + 0], p[t * 4 + 1]);
-                pb[t].raw.y = pack2_bf16(p[t * 4 + 2], p[t * 4 + 3]);
-            }
+            F16B pb;  // P^T for the keys 8 G .. 8 G + 7 of the block
+            pb.raw = uint4{pack2_bf16(p[0], p[1]), pack2_bf16(p[2], p[3]), pack2_bf16(p[4], p[5]), pack2_bf16(p[6], p[7])};
             // the accumulators shrink only when some row's maximum moved (rare after the first blocks)
             if (__any(corr != 1.f)) {
 #pragma unroll
@@ -261,12 +272,8 @@ __global__ __launch_bounds__(64 * MAXW) void attention_mfma_kernel(
             }
             // ---- O^T += V^T P^T
 #pragma unroll
-            for (int dt = 0; dt < HDT; ++dt) {
-                floatx4 a = acc[nt][dt];
-                a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.vf[0][dt].v, pb[0].v, a, 0, 0, 0);
-                a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.vf[1][dt].v, pb[1].v, a, 0, 0, 0);
-                acc[nt][dt] = a;
-            }
+            for (int dt = 0; dt < HDT; ++dt)
+                acc[nt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[dt].v, pb.v, acc[nt][dt], 0, 0, 0);
         }
     };
     // The table reads of a block go out one block ahead, so that its data reads never wait for
@@ -406,17 +413,20 @@ int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_po
     if (waves > MAXW) waves = MAXW;
     // a launch of one wave per workgroup takes the instantiation without the LDS of the
     // combination, which would otherwise limit how many workgroups a compute unit holds
+#define FSIE_ATTN_LAUNCH(W, THREADS, V)                                                                              \
+    attention_mfma_kernel<HDT, NT, W, V><<<grid, THREADS, 0, stream>>>(                                              \
+        static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), \
+        block_tables, max_pages, items, static_cast<bf16_t*>(out), partials, n_heads, n_kv, page_size, window, scale, \
+        gh, head_chunks)
+    const bool v16 = page_size % 8 == 0;
     if (waves == 1) {
-        attention_mfma_kernel<HDT, NT, 1><<<grid, 64, 0, stream>>>(
-            static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool),
-            static_cast<const bf16_t*>(v_pool), block_tables, max_pages, items, static_cast<bf16_t*>(out), partials,
-            n_heads, n_kv, page_size, window, scale, gh, head_chunks);
+        if (v16) FSIE_ATTN_LAUNCH(1, 64, true);
+        else FSIE_ATTN_LAUNCH(1, 64, false);
     } else {
-        attention_mfma_kernel<HDT, NT, MAXW><<<grid, 64 * waves, 0, stream>>>(
-            static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool),
-            static_cast<const bf16_t*>(v_pool), block_tables, max_pages, items, static_cast<bf16_t*>(out), partials,
-            n_heads, n_kv, page_size, window, scale, gh, head_chunks);
+        if (v16) FSIE_ATTN_LAUNCH(MAXW, 64 * waves, true);
+        else FSIE_ATTN_LAUNCH(MAXW, 64 * waves, false);
     }
+#undef FSIE_ATTN_LAUNCH
     FSIE_CHECK_LAUNCH("attention_mfma");
     return 0;
 }
