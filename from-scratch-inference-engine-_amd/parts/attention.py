@@ -128,7 +128,9 @@ class AttentionPlanner:
             if large or len(small) > n_items:
                 raise RuntimeError("attention plan does not fit the captured graph")
             small += [(0, 0, 0, 0, 0, 0, -1, 0)] * (n_items - len(small))
-            if split_keys is not None:
+            if n_items > host.n_seqs:
+                # the graph has room for items that share a request's keys: it merges every row
+                # (rows that need none get an empty merge)
                 merged = {m[0] for m in merges}
                 merges += [(row, 0, 0, 0) for row in range(host.n_tokens) if row not in merged]
                 n_partial = n_items * small_tokens
