@@ -181,7 +181,8 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = N
 def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      out_dtype: Optional[torch.dtype] = None, waves: int = 0, blocks: int = 0,
                      out: Optional[torch.Tensor] = None, epilogue: str = "plain", splits: int = 1) -> torch.Tensor:
-    """The same product on the matrix cores for bfloat16 and at most 64 rows (K a multiple of 8).
+    """The same product on the matrix cores for bfloat16 operands (K a multiple of 8): at most 16
+    rows for a bfloat16 result, at most 64 for a float32 one.
     ``epilogue="swiglu"``: the rows of ``weight`` are gate and up interleaved and the result is
     silu(gate) * up, [M, N/2].  ``splits`` in (2, 4, 8): K is cut into that many slices and the
     result is their float32 partial sums [splits, M, N] (no bias), for ``rmsnorm`` to add up."""
