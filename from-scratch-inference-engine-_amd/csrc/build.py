@@ -126,7 +126,7 @@ def ensure_built() -> Path:
     lib = find_built()
     if lib is not None:
         return lib
-    _say("no kernel library for these sources yet: building once (about a minute)")
+    _say("no kernel library for these sources yet: building once (a few seconds to half a minute, by the number of cores)")
     return build()
 
 
