@@ -85,13 +85,13 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
             }
         }
         n = min(n, N - 1);  // rows past the end repeat the last one; never written
-        wp[b] = w + static_cast<int64_t>(n) * K + kg * 8;
+        wp[b] = w + static_cast<int64_t>(n) * K;
     }
     const bf16_t* xp[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         // rows of X past the end read the last row again: their columns of D are never written
-        xp[t] = x + static_cast<int64_t>(min(t * 16 + row, M - 1)) * K + kg * 8;
+        xp[t] = x + static_cast<int64_t>(min(t * 16 + row, M - 1)) * K;
     }
     floatx4 acc[NB][MT];
 #pragma unroll
@@ -113,9 +113,9 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const int k0 = k_begin + ((p0 + u * WAVES) * 2 + h) * kStep;
-                ok[u][h] = k0 + kg * 8 < k_end;  // K is a multiple of 8: a lane's 8 values are all in or all out
-                const int k0c = ok[u][h] ? k0 : 0;
+                const int k0 = k_begin + ((p0 + u * WAVES) * 2 + h) * kStep + kg * 8;
+                ok[u][h] = k0 < k_end;  // K is a multiple of 8: a lane's 8 values are all in or all out
+                const int k0c = ok[u][h] ? k0 : k_begin;  // the slice's first 8 values: always inside the row
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) a[u][h][nb].raw = *reinterpret_cast<const uint4*>(wp[nb] + k0c);
 #pragma unroll
