@@ -26,8 +26,8 @@ class DecodeGraphs:
         self.max_graphs = max_graphs
         self._graphs: Dict[Tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
         model = runner.model
-        self.enabled = all(getattr(block.mixer, "graph_safe", False) for block in model.spec.layers) and all(
-            hasattr(p, "graph_bucket") for p in model.planners)
+        parts = [p for block in model.spec.layers for p in (block, *block.sub_parts().values())]
+        self.enabled = all(p.graph_safe for p in parts) and all(hasattr(p, "graph_bucket") for p in model.planners)
         self.replays = 0
         self.captures = 0
 

@@ -165,8 +165,12 @@ class GQAttention(Mixer):
     bias (src/model/model.cpp:110-129, src/model/nn.cpp:151-226).  ``window`` = number of latest
     positions a query reads (None: all)."""
 
-    graph_safe = True  # forward reads the step only through device tables: a captured graph may replay it
     share_keys = True  # long portions: four tiles of a request share each block of keys through LDS
+
+    @property
+    def graph_safe(self) -> bool:
+        """forward reads the step only through device tables; the position encoding must too."""
+        return self.position.graph_safe
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
                  position: PositionEncoding, window: Optional[int] = None):

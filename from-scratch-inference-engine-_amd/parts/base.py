@@ -54,6 +54,11 @@ class HiddenState:
 
 class Part:
     kind: str = "part"
+    # True if the part takes everything that changes from step to step from device tensors (its
+    # input and the context's device tables, never ctx.host) and never waits for the device, so
+    # that a captured graph of a decode step can be replayed.  A model is replayed from graphs
+    # only if every part of every layer says so.
+    graph_safe = False
 
     def param_decls(self) -> Dict[str, ParamDecl]:
         return {}
@@ -76,9 +81,6 @@ class Norm(Part):
 
 class Mixer(Part):
     kind = "mixer"
-    # True if forward() takes everything that changes from step to step from device tensors of
-    # the context (never from ctx.host), so that a captured graph of a step can be replayed
-    graph_safe = False
 
     def cache_need(self):
         return None

@@ -13,6 +13,8 @@ class PreNormBlock(Block):
     left pending in the hidden state, so the next norm (this block's second, the next block's
     first, or the model's last) adds them in the same pass that normalises."""
 
+    graph_safe = True
+
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward):
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
 

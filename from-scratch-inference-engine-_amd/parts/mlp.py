@@ -19,6 +19,8 @@ class SwiGLU(FeedForward):
     and the lane that holds gate_j also holds up_j, so that for a few rows (decoding) SiLU*up
     happens in the product's epilogue and the [T, 2I] intermediate never reaches memory."""
 
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size

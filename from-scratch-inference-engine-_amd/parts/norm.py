@@ -18,6 +18,8 @@ class RMSNorm(Norm):
 
     adds_partial_sums = True
 
+    graph_safe = True
+
     def __init__(self, hidden_size: int, eps: float):
         self.hidden_size = hidden_size
         self.eps = float(eps)

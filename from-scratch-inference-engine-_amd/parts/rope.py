@@ -28,6 +28,8 @@ class RotaryEncoding(PositionEncoding):
     frequency theta^(-2i/rotary_dim), angle = position * frequency in float64
     (src/model/nn.cpp:110-149).  Fused with the q/k/v bias and the write into the cache."""
 
+    graph_safe = True
+
     def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None):
         self.head_dim = head_dim
         self.theta = float(theta)
@@ -63,6 +65,8 @@ class RotaryEncoding(PositionEncoding):
 @register_part("position", "none")
 class NoPositionEncoding(PositionEncoding):
     """No rotation: only the bias and the write into the cache."""
+
+    graph_safe = True
 
     def __init__(self, head_dim: int = 0):
         self.head_dim = head_dim

@@ -1,0 +1,221 @@
+"""A feed-forward with routing and another position encoding, both defined here, are registered and
+used in a model beside the engine's own attention, norms and block, without a change to the
+engine's files.  The toys compute with torch (they are test code, not product kernels); what the
+test shows is that the engine's interfaces carry them: parameters by name, the step's positions,
+the cache write, portions and mixed batches."""
+
+import json
+import math
+
+import pytest
+import torch
+
+import helpers
+import plain_qwen2 as plain
+
+pytestmark = pytest.mark.gpu
+
+
+def define_toys():
+    from dataclasses import dataclass
+
+    from from_scratch_inference_engine_amd import ops
+    from from_scratch_inference_engine_amd.config.base import ModelConfig, required_int
+    from from_scratch_inference_engine_amd.models import LayerCall, ModelSpec, bind, register_architecture
+    from from_scratch_inference_engine_amd.parts import (FeedForward, LMHead, ParamDecl, PositionEncoding,
+                                                         TokenEmbedding, make_part, register_part)
+    from from_scratch_inference_engine_amd.weights import TensorSpec
+
+    @register_part("feed_forward", "toy_top1_experts")
+    class Top1Experts(FeedForward):
+        """Every token goes to the expert with the largest router logit (float32 logits, first
+        maximum wins) and comes back weighted by that expert's softmax probability:
+        y = p_e * W2_e relu(W1_e x).  The choice is per token, so it cannot depend on the batch."""
+
+        def __init__(self, hidden_size: int, inter: int, n_experts: int):
+            self.h, self.i, self.e = hidden_size, inter, n_experts
+            self.router = self.w1 = self.w2 = None
+
+        def param_decls(self):
+            return {"router": ParamDecl((self.e, self.h)), "w1": ParamDecl((self.e * self.i, self.h)),
+                    "w2": ParamDecl((self.e * self.h, self.i))}
+
+        def forward(self, x, ctx):
+            logits = x.float() @ self.router.float().t()
+            probs = torch.softmax(logits, dim=-1)
+            choice = logits.argmax(dim=-1)
+            out = torch.zeros_like(x)
+            for e in range(self.e):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                w1 = self.w1[e * self.i:(e + 1) * self.i].float()
+                w2 = self.w2[e * self.h:(e + 1) * self.h].float()
+                y = torch.relu(x[rows].float() @ w1.t()) @ w2.t()
+                out[rows] = (y * probs[rows, e].unsqueeze(1)).to(x.dtype)
+            return out
+
+    @register_part("position", "toy_interleaved_rope")
+    class InterleavedRope(PositionEncoding):
+        """Rotation of the pairs (2i, 2i + 1) of every q and k head (the engine's own encoding
+        pairs i with i + head_dim / 2).  The toy adds the bias and rotates with torch, then hands
+        q, k and v to the engine's kernel for the write into the cache (no rotation there)."""
+
+        def __init__(self, head_dim: int, theta: float):
+            self.head_dim, self.theta = head_dim, theta
+
+        def apply(self, qkv, n_heads, n_kv, head_dim, ctx, store, bias=None):
+            t = qkv.shape[0]
+            full = qkv.float() + (bias if bias is not None else 0.0)
+            rot = (n_heads + n_kv) * head_dim
+            heads = full[:, :rot].reshape(t, n_heads + n_kv, head_dim // 2, 2)
+            inv = self.theta ** (-2.0 * torch.arange(head_dim // 2, dtype=torch.float64, device=qkv.device) / head_dim)
+            ang = ctx.positions.double().unsqueeze(1) * inv.unsqueeze(0)            # [t, hd/2]
+            c, s = torch.cos(ang).float().unsqueeze(1), torch.sin(ang).float().unsqueeze(1)
+            a, b = heads[..., 0], heads[..., 1]
+            full[:, :rot] = torch.stack((a * c - b * s, b * c + a * s), dim=-1).reshape(t, rot)
+            qkv.copy_(full.to(qkv.dtype))
+            if store is None:
+                return
+            ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, None, slots=store.slots, k_pool=store.k_pool,
+                              v_pool=store.v_pool, page_size=store.page_size)
+
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        hidden_size: int = 0
+        vocab_size: int = 0
+        num_layers: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        head_dim: int = 0
+        inter: int = 0
+        experts: int = 0
+        theta: float = 1e4
+        eps: float = 1e-6
+
+        @classmethod
+        def from_dict(cls, raw):
+            ints = {k: required_int(raw, k) for k in ("hidden_size", "vocab_size", "num_layers", "heads", "kv_heads",
+                                                      "head_dim", "inter", "experts")}
+            return cls(architecture=raw["architectures"][0], theta=float(raw["theta"]), eps=float(raw["eps"]), **ints)
+
+    def build(cfg: ToyConfig) -> ModelSpec:
+        h, hd = cfg.hidden_size, cfg.head_dim
+        q_dim, kv_dim = cfg.heads * hd, cfg.kv_heads * hd
+        bindings = []
+        emb = TokenEmbedding(cfg.vocab_size, h)
+        bind(bindings, emb, "weight", [TensorSpec("emb", (cfg.vocab_size, h))])
+        layers = []
+        for l in range(cfg.num_layers):
+            pos = make_part("position", "toy_interleaved_rope", head_dim=hd, theta=cfg.theta)
+            mixer = make_part("mixer", "gqa_attention", hidden_size=h, n_heads=cfg.heads, n_kv_heads=cfg.kv_heads,
+                              head_dim=hd, qkv_bias=True, position=pos, window=None)
+            ffn = make_part("feed_forward", "toy_top1_experts", hidden_size=h, inter=cfg.inter, n_experts=cfg.experts)
+            n1 = make_part("norm", "rms_norm", hidden_size=h, eps=cfg.eps)
+            n2 = make_part("norm", "rms_norm", hidden_size=h, eps=cfg.eps)
+            layers.append(make_part("block", "pre_norm", mixer_norm=n1, mixer=mixer, ffn_norm=n2, ffn=ffn))
+            bind(bindings, n1, "weight", [TensorSpec(f"l{l}.n1", (h,), "norm")])
+            bind(bindings, n2, "weight", [TensorSpec(f"l{l}.n2", (h,), "norm")])
+            bind(bindings, mixer, "qkv_weight", [TensorSpec(f"l{l}.q", (q_dim, h)), TensorSpec(f"l{l}.k", (kv_dim, h)),
+                                                 TensorSpec(f"l{l}.v", (kv_dim, h))])
+            bind(bindings, mixer, "qkv_bias", [TensorSpec(f"l{l}.qb", (q_dim,), "bias"), TensorSpec(f"l{l}.kb", (kv_dim,), "bias"),
+                                               TensorSpec(f"l{l}.vb", (kv_dim,), "bias")])
+            bind(bindings, mixer, "o_weight", [TensorSpec(f"l{l}.o", (h, q_dim))])
+            bind(bindings, ffn, "router", [TensorSpec(f"l{l}.router", (cfg.experts, h))])
+            bind(bindings, ffn, "w1", [TensorSpec(f"l{l}.e{e}.w1", (cfg.inter, h)) for e in range(cfg.experts)])
+            bind(bindings, ffn, "w2", [TensorSpec(f"l{l}.e{e}.w2", (h, cfg.inter)) for e in range(cfg.experts)])
+        norm = make_part("norm", "rms_norm", hidden_size=h, eps=cfg.eps)
+        bind(bindings, norm, "weight", [TensorSpec("norm", (h,), "norm")])
+        head = LMHead(h, cfg.vocab_size)
+        bind(bindings, head, "weight", [TensorSpec("head", (cfg.vocab_size, h))])
+        return ModelSpec(config=cfg, embedding=emb, layers=layers, schedule=[LayerCall(l) for l in range(cfg.num_layers)],
+                         final_norm=norm, lm_head=head, bindings=bindings)
+
+    register_architecture("ToyRoutedLM", ToyConfig, build)
+    return ToyConfig
+
+
+def plain_toy(raw, w, ids):
+    """The same model, whole sequence, no cache, float64 where the plain functions use it."""
+    h, hd, nh, nkv = raw["hidden_size"], raw["head_dim"], raw["heads"], raw["kv_heads"]
+    x = w["emb"][torch.tensor(ids)]
+    t = len(ids)
+    pos = torch.arange(t, dtype=torch.float64)
+    inv = raw["theta"] ** (-2.0 * torch.arange(hd // 2, dtype=torch.float64) / hd)
+    ang = pos.unsqueeze(1) * inv.unsqueeze(0)
+    c, s = torch.cos(ang).unsqueeze(1), torch.sin(ang).unsqueeze(1)
+
+    def rotate(m, n):
+        p = m.double().reshape(t, n, hd // 2, 2)
+        a, b = p[..., 0], p[..., 1]
+        return torch.stack((a * c - b * s, b * c + a * s), dim=-1).reshape(t, n * hd).float()
+
+    for l in range(raw["num_layers"]):
+        n1 = plain.rms_norm(x, w[f"l{l}.n1"], raw["eps"])
+        q = rotate(plain.linear(n1, w[f"l{l}.q"], w[f"l{l}.qb"]), nh)
+        k = rotate(plain.linear(n1, w[f"l{l}.k"], w[f"l{l}.kb"]), nkv)
+        v = plain.linear(n1, w[f"l{l}.v"], w[f"l{l}.vb"])
+        x = x + plain.linear(plain.attention(q, k, v, nh, nkv, hd), w[f"l{l}.o"])
+        n2 = plain.rms_norm(x, w[f"l{l}.n2"], raw["eps"])
+        logits = n2 @ w[f"l{l}.router"].t()
+        probs = torch.softmax(logits, dim=-1)
+        top2 = logits.topk(2, dim=-1).values
+        assert (top2[:, 0] - top2[:, 1]).min() > 1e-2, "a near tie of two experts: the comparison would test rounding"
+        rows = []
+        for i in range(t):
+            e = int(logits[i].argmax())
+            y = torch.relu(n2[i] @ w[f"l{l}.e{e}.w1"].t()) @ w[f"l{l}.e{e}.w2"].t()
+            rows.append(y * probs[i, e])
+        x = x + torch.stack(rows)
+    return plain.linear(plain.rms_norm(x, w["norm"], raw["eps"]), w["head"])
+
+
+def test_routed_feed_forward_and_another_position_encoding(tmp_path):
+    from from_scratch_inference_engine_amd import load_config, load_model
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+    from from_scratch_inference_engine_amd.weights import SafetensorsFile, write_random_model, write_safetensors
+
+    ToyConfig = define_toys()
+    raw = {"architectures": ["ToyRoutedLM"], "hidden_size": 48, "vocab_size": 89, "num_layers": 2, "heads": 4,
+           "kv_heads": 2, "head_dim": 16, "inter": 24, "experts": 3, "theta": 500.0, "eps": 1e-5}
+    (tmp_path / "m").mkdir()
+    (tmp_path / "m" / "config.json").write_text(json.dumps(raw))
+    cfg = load_config(tmp_path / "m")
+    assert isinstance(cfg, ToyConfig)
+    object.__setattr__(cfg, "to_dict", lambda: raw)
+    write_random_model(cfg, 7, tmp_path / "m", torch.float32)
+    f = SafetensorsFile(tmp_path / "m" / "model.safetensors")
+    w = {n: f.get(n).clone() for n in f.names()}
+    for l in range(2):  # spread the router so that every expert gets tokens and no choice is a near tie
+        w[f"l{l}.router"] = w[f"l{l}.router"] * 40.0
+    write_safetensors(tmp_path / "m" / "model.safetensors", w)
+    model = load_model(tmp_path / "m", dtype="float32")
+    assert len(model.cache_layout.paged_groups) == 1
+    runner = Runner(model, page_size=4, num_pages=24, max_requests=3)
+    assert runner.graphs.enabled is False  # the toys wait for the device: no graph replay for this model
+    seqs = {"a": helpers.token_ids(89, 31, 11), "b": helpers.token_ids(89, 9, 12), "c": helpers.token_ids(89, 17, 13)}
+    ref = {k: plain_toy(raw, w, ids) for k, ids in seqs.items()}
+    # the plain model used every expert (else the test would not see a wrong expert's weights)
+    n2 = plain.rms_norm(w["emb"][torch.tensor(seqs["a"])], w["l0.n1"], raw["eps"])
+    assert len(set((n2 @ w["l0.router"].t()).argmax(-1).tolist())) >= 2
+    got = {k: [] for k in seqs}
+    caches, fed = {}, {k: 0 for k in seqs}
+    plan = [[("a", 13), ("b", 2)], [("a", 1), ("b", 7)], [("a", 2), ("c", 5)], [("c", 1), ("a", 1)], [("c", 11), ("a", 14)]]
+    for step in plan:
+        entries = []
+        for k, n in step:
+            if k not in caches:
+                if k == "c":
+                    runner.manager.close(caches.pop("b"))  # c takes over b's pages and slot
+                caches[k] = runner.manager.open(k)
+            entries.append(StepEntry(caches[k], seqs[k][fed[k]:fed[k] + n], list(range(n))))
+            fed[k] += n
+        out = runner.step(entries).cpu()
+        row = 0
+        for e in entries:
+            got[e.cache.request_id].append(out[row:row + len(e.tokens)])
+            row += len(e.tokens)
+    for k in seqs:
+        assert fed[k] == len(seqs[k])
+        assert (torch.cat(got[k]) - ref[k]).abs().max() <= 1e-4, k
