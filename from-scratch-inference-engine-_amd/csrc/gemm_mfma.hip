@@ -36,17 +36,20 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
     const int mt = (M + 15) / 16;
     const int pairs = ((K + splits - 1) / splits + 2 * fsie_mm::kStep - 1) / (2 * fsie_mm::kStep);
     if (blocks == 0) {
-        // more than a few rows of X: two blocks of W share each X fragment where N still leaves
-        // enough workgroups for the chip (measured on MI355X: 5.2 against 4.4 TB/s at N = 37888)
-        blocks = (M > 4 && static_cast<int64_t>(N) * splits >= 14336) ? 2 : 1;
+        // more than two rows of X: two blocks of W share each X fragment where N still leaves
+        // enough workgroups for the chip (measured on MI355X at N = 37888: 5.2 against 4.4 TB/s
+        // with 8 rows, 49 against 58 us with 4)
+        blocks = (M > 2 && static_cast<int64_t>(N) * splits >= 14336) ? 2 : 1;
     }
     if (waves == 0) {
-        // split K inside the workgroup until about a thousand waves stream W; a single row of X
-        // gains from more loads in flight even at large N
+        // split K inside the workgroup until about a thousand waves stream W; one or two rows of
+        // X gain from more loads in flight even at large N (eight waves; four where N alone gives
+        // two thousand workgroups: 177 against 181 us at N = 152064)
         const int groups = (N + 16 * blocks - 1) / (16 * blocks) * splits;
         waves = 1;
         while (waves < 16 && groups * waves < 1024) waves *= 2;
-        if (M <= 4 && waves < 8) waves = 8;
+        const int few_rows_waves = groups >= 2048 ? 4 : 8;
+        if (M <= 2 && waves < few_rows_waves) waves = few_rows_waves;
         while (waves > 1 && pairs < 2 * waves) waves /= 2;
     }
     if (mt * blocks > 4 && waves > 8) waves = 8;  // LDS of the reduction
@@ -83,8 +86,9 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     const int pairs = (K + 2 * fsie_mm::kStep - 1) / (2 * fsie_mm::kStep);
     const int blocks = 1;
     int waves = 1;
+    // (more waves than this only add to the reduction: 12.6 us with four against 14.1 with eight
+    // at N = 4608, K = 3584 and one row)
     while (waves < 16 && (N / 16) * waves < 1024) waves *= 2;
-    if (M <= 4 && waves < 8) waves = 8;
     while (waves > 1 && pairs < 2 * waves) waves /= 2;
     if (mt * blocks > 4 && waves > 8) waves = 8;  // LDS of the reduction
     const fsie_mm::Call call{x, w, bias, y, M, N, K, 1, stream,
