@@ -42,13 +42,16 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
         blocks = (M > 2 && static_cast<int64_t>(N) * splits >= 14336) ? 2 : 1;
     }
     if (waves == 0) {
-        // split K inside the workgroup until about a thousand waves stream W; one or two rows of
-        // X gain from more loads in flight even at large N (eight waves; four where N alone gives
-        // two thousand workgroups: 177 against 181 us at N = 152064)
+        // split K inside the workgroup until about nine hundred waves stream W (N = 3584,
+        // K = 18944 in four slices, 8 rows: 27.9 us with 896 waves, 32.7 with 1792; with 64 rows
+        // 1792 are better, 6.19 against 6.42 ms for a whole decode step of a 7B model); one or two
+        // rows of X gain from more loads in flight even at large N (four waves where N alone gives
+        // two thousand workgroups: 177 against 181 us at N = 152064; two from 896 workgroups on)
         const int groups = (N + 16 * blocks - 1) / (16 * blocks) * splits;
         waves = 1;
-        while (waves < 16 && groups * waves < 1024) waves *= 2;
-        const int few_rows_waves = groups >= 2048 ? 4 : 8;
+        const int enough = M <= 16 ? 896 : 1024;  // more rows of X: more waves to share the products
+        while (waves < 16 && groups * waves < enough) waves *= 2;
+        const int few_rows_waves = groups >= 2048 ? 4 : (groups >= 896 ? 2 : 8);
         if (M <= 2 && waves < few_rows_waves) waves = few_rows_waves;
         while (waves > 1 && pairs < 2 * waves) waves /= 2;
     }

@@ -60,12 +60,14 @@ class Linear:
 
     def residual_splits(self, m: int) -> int:
         """Slices of K for ``for_residual`` (1 = do not cut): as many as bring the workgroups to
-        about four per compute unit, each slice at least 1024 long.  Above 16 rows only where K
-        is long enough for four slices; shorter products of that many rows are the library's
-        (measured on MI355X at N = 3584, K = 18944, 64 rows: 67 us against the library's 91)."""
+        about four per compute unit, each slice at least 512 long (N = K = 3584, 8 rows: 8.2 us in
+        four slices, 8.8 in two).  Above 16 rows only where K gives four slices of 1024; shorter
+        products of that many rows are the library's (measured on MI355X at N = 3584, K = 18944,
+        64 rows: 67 us against the library's 91)."""
         groups = -(-self.out_features // 16)
+        shortest = 512 if m <= GEMM_MFMA_SKINNY_BEST_M else 1024
         splits = 1
-        while splits < 8 and groups * splits < 896 and self.in_features // (2 * splits) >= 1024:
+        while splits < 8 and groups * splits < 896 and self.in_features // (2 * splits) >= shortest:
             splits *= 2
         if m > GEMM_MFMA_SKINNY_BEST_M and splits < 4:
             return 1
