@@ -59,6 +59,11 @@ int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const float* bias, 
                                void* v_pool, int n_heads, int n_kv, int head_dim, int page_size, int64_t pool_slots,
                                hipStream_t stream);
 
+// 17 to 64 rows (any number up to 64 is taken): X shared through LDS, float32 result or partial sums
+int fsie_gemm_mfma_wide_slice(int K, int splits);
+int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits, int waves,
+                        hipStream_t stream);
+
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
                           void* out, float* partials, int n_heads, int n_kv, int head_dim, int page_size,

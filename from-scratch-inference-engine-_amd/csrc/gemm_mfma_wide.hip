@@ -1,0 +1,205 @@
+// Y[M, N] = X[M, K] . W[N, K]^T for bfloat16 operands and 17 to 64 rows of X, float32 results:
+// the weight-streaming matrix-core product for batches whose X no longer comes cheaply from cache.
+//
+// As in the product for few rows, D[n, m] = sum_k W[n, k] X[m, k]: W streams from HBM straight
+// into the A registers of v_mfma_f32_16x16x32_bf16.  With up to four tiles of 16 rows of X, reading
+// the B fragments from memory would move several times the bytes of W through every compute
+// unit's memory pipeline, which is what bounds it (some 50 GB/s a unit).  So the waves of a workgroup
+// take different blocks of 16 rows of W (none splits K) and share X: a stage of KS values of K of
+// all rows of X is laid into LDS once per workgroup, in the order of the B fragments, and every
+// wave reads its fragments from there.
+//
+// Pipeline of a stage s (one barrier a stage):
+//   global loads of X for stage s+1 (to registers), then of W for stage s+1;
+//   B fragments of stage s from LDS, products with the W of stage s (loaded a stage ago);
+//   X of stage s+1 from registers to the other LDS buffer (waits for the X loads only: they were
+//   issued before the W loads and the counter is in order); barrier.
+// The last stage runs outside the loop, so that no branch lies around a batch of loads.
+//
+// blockIdx.y selects a slice of K (a multiple of KS); with more than one slice y is
+// [slices][M][N], float32 partial sums for the consumer to add in the order of the slices.
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef const __attribute__((address_space(1))) u32x4* GlobalVec;
+
+union Frag {
+    u32x4 q;
+    bf16x8 v;
+};
+
+// MT tiles of 16 rows of X; WAVES waves = WAVES blocks of 16 rows of W per workgroup;
+// STEPS 32-wide MFMA steps per stage (KS = 32 * STEPS values of K).
+template <int MT, int WAVES, int STEPS>
+__global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t* __restrict__ x,
+                                                                   const bf16_t* __restrict__ w,
+                                                                   float* __restrict__ y, int M, int N, int K,
+                                                                   int k_slice) {
+    constexpr int KS = 32 * STEPS;
+    constexpr int ROWS = 16 * MT;             // rows of X in LDS (rows past M repeat the last one)
+    constexpr int UNITS = ROWS * 4 * STEPS;   // 16-byte units of a stage of X
+    constexpr int THREADS = WAVES * 64;
+    constexpr int PER_THREAD = (UNITS + THREADS - 1) / THREADS;
+    constexpr int PITCH = ROWS + 1;           // units between consecutive (step, k group) runs: the
+                                              // odd pitch spreads a staging wave's writes over the banks
+    constexpr int SPARE = 4 * STEPS * PITCH;  // where threads without a unit of their own write
+    __shared__ u32x4 xs[2][4 * STEPS * PITCH + 1];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int row = lane & 15;  // row of the A tile (n) and column of the B tile (m)
+    const int kg = lane >> 4;   // which 8 of a step's 32 k values this lane holds
+    const int n0 = (blockIdx.x * WAVES + wave) * 16;
+    const int k_begin = blockIdx.y * k_slice;
+    const int k_end = min(K, k_begin + k_slice);
+    const int n_stages = (k_end - k_begin) / KS;  // the host makes every slice a multiple of KS
+
+    // rows of W past the end repeat the last one; their results are never written
+    const bf16_t* wp = w + static_cast<int64_t>(min(n0 + row, N - 1)) * K + k_begin + kg * 8;
+    // staging: unit u = (row of X, j = step * 4 + k group); consecutive threads take consecutive
+    // 16 bytes of a row
+    const bf16_t* xsrc[PER_THREAD];
+    int xdst[PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) {
+        const int u = threadIdx.x + i * THREADS;
+        const int uc = u < UNITS ? u : 0;  // a thread without a unit reads unit 0 and writes the spare place:
+        const int m = uc / (4 * STEPS), j = uc - m * (4 * STEPS);  // no branch around loads or stores
+        xsrc[i] = x + static_cast<int64_t>(min(m, M - 1)) * K + k_begin + j * 8;
+        xdst[i] = u < UNITS ? j * PITCH + m : SPARE;
+    }
+
+    floatx4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    if (n_stages <= 0) return;
+
+    u32x4 xr[PER_THREAD];
+    Frag wa[STEPS], wb[STEPS];  // the W fragments of even and odd stages
+    // stage 0
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) xr[i] = *(GlobalVec)(xsrc[i]);
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) wa[s].q = *(GlobalVec)(wp + s * 32);
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; ++i) xs[0][xdst[i]] = xr[i];
+    __syncthreads();
+
+    auto products = [&](int buf, const Frag (&wc)[STEPS]) {
+        const u32x4* xb = xs[buf] + kg * PITCH + row;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            Frag b[MT];
+#pragma unroll
+            for (int t = 0; t < MT; ++t) b[t].q = xb[s * 4 * PITCH + t * 16];
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[s].v, b[t].v, acc[t], 0, 0, 0);
+        }
+    };
+    // A stage that is not the last: fetch the next one (X first, then W into `wn`), work on this
+    // one (`wc`, LDS buffer `buf`), hand the next X to the other buffer.  No branch lies around
+    // the loads and no register is copied, so the wait before the products counts exactly the
+    // loads issued after this stage's W.
+    auto stage = [&](int buf, const Frag (&wc)[STEPS], Frag (&wn)[STEPS], int k1) {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) xr[i] = *(GlobalVec)(xsrc[i] + k1);
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) wn[s].q = *(GlobalVec)(wp + k1 + s * 32);
+        __builtin_amdgcn_sched_barrier(0);
+        products(buf, wc);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) xs[buf ^ 1][xdst[i]] = xr[i];
+        __syncthreads();
+    };
+    int st = 0;  // even here: stage st lies in buffer 0, its W in wa
+    for (; st + 2 < n_stages; st += 2) {
+        stage(0, wa, wb, (st + 1) * KS);
+        stage(1, wb, wa, (st + 2) * KS);
+    }
+    if (st + 1 < n_stages) {
+        stage(0, wa, wb, (st + 1) * KS);
+        products(1, wb);
+    } else {
+        products(0, wa);
+    }
+
+    // lane holds D[n0 + 4 kg + r][m = 16 t + row]
+    float* part = y + static_cast<int64_t>(blockIdx.y) * M * N;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + row;
+        if (m >= M) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int nn = n0 + kg * 4 + r;
+            if (nn < N) part[static_cast<int64_t>(m) * N + nn] = acc[t][r];
+        }
+    }
+}
+
+template <int MT, int WAVES, int STEPS>
+int launch(const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
+           hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>((N + 16 * WAVES - 1) / (16 * WAVES)), static_cast<unsigned>(splits));
+    gemm_mfma_wide_kernel<MT, WAVES, STEPS><<<grid, WAVES * 64, 0, stream>>>(x, w, y, M, N, K, k_slice);
+    FSIE_CHECK_LAUNCH("gemm_mfma_wide");
+    return 0;
+}
+
+template <int WAVES, int STEPS>
+int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
+              hipStream_t stream) {
+    switch (mt) {
+        case 1: return launch<1, WAVES, STEPS>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 2: return launch<2, WAVES, STEPS>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 3: return launch<3, WAVES, STEPS>(x, w, y, M, N, K, splits, k_slice, stream);
+        default: return launch<4, WAVES, STEPS>(x, w, y, M, N, K, splits, k_slice, stream);
+    }
+}
+
+}  // namespace
+
+// The length of a slice of K for `splits` slices, or 0 if K cannot be cut that way: K and every
+// slice must be a multiple of the stage (128 values), and no slice may be empty.
+extern "C" int fsie_gemm_mfma_wide_slice(int K, int splits) {
+    constexpr int kStage = 128;
+    if (K <= 0 || splits < 1 || splits > FSIE_GEMM_MAX_SPLITS || K % kStage) return 0;
+    const int slice = ((K + splits - 1) / splits + kStage - 1) / kStage * kStage;
+    if (static_cast<int64_t>(slice) * (splits - 1) >= K) return 0;
+    return slice;
+}
+
+// bfloat16 operands, float32 result: y is [M, N] (splits == 1) or [splits, M, N] partial sums.
+// 1 <= M <= 64; K a multiple of 128 that `splits` slices of whole stages cover (see above);
+// x and w 16-byte aligned.  waves: 4 or 8 blocks of 16 rows of W per workgroup, 0 = choose.
+extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits,
+                                   int waves, hipStream_t stream) {
+    FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide: bad sizes M=%d N=%d K=%d", M, N, K);
+    FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide: at most %d rows, got %d",
+                 FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
+    const int k_slice = fsie_gemm_mfma_wide_slice(K, splits);
+    FSIE_REQUIRE(k_slice > 0, "gemm_mfma_wide: K=%d cannot be cut into %d slices of whole stages of 128", K, splits);
+    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
+                 "gemm_mfma_wide: operands must be 16-byte aligned");
+    FSIE_REQUIRE(waves == 0 || waves == 4 || waves == 8, "gemm_mfma_wide: waves must be 0, 4 or 8");
+    if (M == 0) return 0;
+    if (waves == 0) {
+        // eight blocks a workgroup halve the reads of X, but only a large N leaves enough
+        // workgroups for them (measured on MI355X, 64 rows: N = 152064 242 against 261 us;
+        // N = 3584, K = 18944 in 8 slices 39.6 against 38.1)
+        const int64_t groups4 = static_cast<int64_t>((N + 63) / 64) * splits;
+        waves = groups4 >= 1024 ? 8 : 4;
+    }
+    const int mt = (M + 15) / 16;
+    const bf16_t* xp = static_cast<const bf16_t*>(x);
+    const bf16_t* wq = static_cast<const bf16_t*>(w);
+    if (waves == 8) return launch_mt<8, 4>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    return launch_mt<4, 4>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+}

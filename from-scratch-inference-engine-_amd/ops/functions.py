@@ -216,6 +216,36 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     return out
 
 
+def gemm_mfma_wide_splits_ok(k: int, splits: int) -> bool:
+    """Whether ``gemm_mfma_wide`` can cut an inner size ``k`` into ``splits`` slices (whole stages
+    of 128 values each)."""
+    return load().fsie_gemm_mfma_wide_slice(int(k), int(splits)) > 0
+
+
+def gemm_mfma_wide(x: torch.Tensor, weight: torch.Tensor, splits: int = 1, waves: int = 0,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [M, K] . weight [N, K]^T for bfloat16 operands and up to 64 rows, the rows of x shared by
+    a workgroup's waves through LDS (made for 17 rows and more).  The result is float32: [M, N],
+    or with ``splits`` in (2, 4, 8) the partial sums [splits, M, N] of the slices of K, for
+    ``rmsnorm`` to add up.  K must be a multiple of 128 that the slices cover in whole stages
+    (``gemm_mfma_wide_splits_ok``)."""
+    _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
+    _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"gemm: weight inner size {weight.shape[1]} does not match x's {k}")
+    if splits != 1 and splits not in GEMM_SPLITS:
+        raise KernelError(f"gemm_mfma_wide: splits must be 1 or one of {GEMM_SPLITS}, got {splits}")
+    shape = (m, n) if splits == 1 else (splits, m, n)
+    if out is None:
+        out = torch.empty(shape, dtype=torch.float32, device=x.device)
+    _need(out, "gemm out", dtype=torch.float32, shape=shape)
+    check(load().fsie_gemm_mfma_wide(x.data_ptr(), weight.data_ptr(), out.data_ptr(), m, n, k, splits, waves,
+                                     _stream()))
+    return out
+
+
 def gemm_mfma_skinny_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
                           positions: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
                           inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor] = None,

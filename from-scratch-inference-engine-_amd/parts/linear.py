@@ -16,8 +16,10 @@ class Linear:
 
     float32: the engine's own kernels only (true 32-bit products and sums).
     bfloat16: up to 16 rows (decoding) the engine's matrix-core kernel that streams the weight
-    once (up to 64 rows for float32 results, the logits); above that the library product (hipBLASLt through torch, where the reference's engine
-    calls cuBLAS) with float32 accumulation, the bias added by a kernel of the engine."""
+    once; 17 to 64 rows its sibling that shares x through LDS, for float32 results (the logits)
+    and for the residual projections (``for_residual``); everything else the library product
+    (hipBLASLt through torch, where the reference's engine calls cuBLAS) with float32
+    accumulation, the bias added by a kernel of the engine."""
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False):
         self.in_features = in_features
@@ -25,6 +27,7 @@ class Linear:
         self.has_bias = bias
         self.weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
+        self._wide_splits: Optional[int] = None
 
     def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                  skip_bias: bool = False) -> torch.Tensor:
@@ -34,6 +37,9 @@ class Linear:
         if x.dtype == torch.float32:
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
         wants_f32 = out_dtype is not None and out_dtype != x.dtype
+        if (wants_f32 and bias is None and GEMM_MFMA_SKINNY_BEST_M < m <= GEMM_MFMA_SKINNY_MAX_M
+                and ops.gemm_mfma_wide_splits_ok(self.in_features, 1)):
+            return ops.gemm_mfma_wide(x, w)  # logits of 17 to 64 rows: x shared through LDS
         if self.in_features % 8 == 0 and m <= (GEMM_MFMA_SKINNY_MAX_M if wants_f32 else GEMM_MFMA_SKINNY_BEST_M):
             return ops.gemm_mfma_skinny(x, w, bias, out_dtype=out_dtype)
         if m <= GEMM_SKINNY_MAX_M or wants_f32 or self.in_features % 8 or self.out_features % 8:
@@ -53,10 +59,27 @@ class Linear:
         m = x.shape[0]
         if (getattr(ctx, "partial_sums_ok", False) and x.dtype == torch.bfloat16 and self.bias is None
                 and self.in_features % 8 == 0 and 0 < m <= GEMM_MFMA_SKINNY_MAX_M):
+            if m > GEMM_MFMA_SKINNY_BEST_M:
+                splits = self.wide_splits()
+                if splits > 1:
+                    return ops.gemm_mfma_wide(x, self.weight, splits=splits)
             splits = self.residual_splits(m)
             if splits > 1:
                 return ops.gemm_mfma_skinny(x, self.weight, splits=splits)
         return self(x)
+
+    def wide_splits(self) -> int:
+        """Slices of K for 17 to 64 rows (the kernel that shares x through LDS): as many as it
+        takes, each at least 512 long (measured on MI355X at 64 rows: N = 3584, K = 18944 in 8
+        slices 38 us, against 68 for the few-rows kernel and 91 for the library; N = K = 3584 in
+        4 slices 11.6 against the library's 13.7).  1 = it does not take this K."""
+        if self._wide_splits is None:
+            self._wide_splits = 1
+            for splits in (8, 4, 2):
+                if self.in_features // splits >= 512 and ops.gemm_mfma_wide_splits_ok(self.in_features, splits):
+                    self._wide_splits = splits
+                    break
+        return self._wide_splits
 
     def residual_splits(self, m: int) -> int:
         """Slices of K for ``for_residual`` (1 = do not cut): as many as bring the workgroups to

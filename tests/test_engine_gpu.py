@@ -242,6 +242,62 @@ def test_decoding_with_partial_sums_in_the_residual_stream(model_dirs, name, mon
     assert any(used)
 
 
+WIDE = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "hidden_size": 1024, "num_hidden_layers": 2, "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 128,
+    "intermediate_size": 1536, "vocab_size": 331, "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "max_position_embeddings": 512,
+}
+
+
+def test_batches_of_17_to_64_rows_share_x_through_lds(tmp_path):
+    """A model wide enough (inner sizes that are multiples of 128 and at least 1,024) that steps
+    of 17 to 64 rows take the kernel that shares x through LDS: the output and down projections
+    as partial sums for the next norm, the logits whole.  20 requests decode together, eagerly
+    and through graphs, and a 40-token portion runs beside 3 decoded tokens."""
+    from from_scratch_inference_engine_amd import load_model, ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    d = helpers.make_model_dir(tmp_path / "wide", WIDE, seed=9)
+    model = load_model(d, dtype="bfloat16")
+    calls = []
+    real = ops.gemm_mfma_wide
+
+    def counted(x, w, splits=1, **kw):
+        calls.append((x.shape[0], splits))
+        return real(x, w, splits=splits, **kw)
+
+    ops.gemm_mfma_wide = counted
+    try:
+        seqs = [helpers.token_ids(331, 9 + i, 900 + i) for i in range(20)]
+        long = helpers.token_ids(331, 60, 950)
+        ref = [plain.forward_dir(d, ids).numpy() for ids in seqs[:6]]
+        ref_long = plain.forward_dir(d, long).numpy()
+        for graphs in (False, True):
+            runner = Runner(model, page_size=16, num_pages=64, max_requests=24, use_graphs=graphs)
+            caches = [runner.manager.open(i) for i in range(20)]
+            n_pre = [len(ids) - 4 for ids in seqs]
+            runner.step([StepEntry(c, ids[:n], []) for c, ids, n in zip(caches, seqs, n_pre)])
+            for t in range(4):
+                out = runner.step([StepEntry(c, [ids[n + t]], [0]) for c, ids, n in zip(caches, seqs, n_pre)]).float().cpu()
+                for i in range(6):
+                    helpers.assert_close_to_plain(out[i:i + 1].numpy(), ref[i][n_pre[i] + t:n_pre[i] + t + 1], "bfloat16",
+                                                  f"graphs={graphs} request {i} token {t}")
+            for c in caches[3:]:
+                runner.manager.close(c)
+            # a portion of 40 tokens beside three decoded tokens: 43 rows in one step
+            lc = runner.manager.open("long")
+            runner.step([StepEntry(lc, long[:20], [])])
+            out = runner.step([StepEntry(lc, long[20:], list(range(40)))]).float().cpu()
+            helpers.assert_close_to_plain(out.numpy(), ref_long[20:], "bfloat16", f"graphs={graphs} portion of 40")
+    finally:
+        ops.gemm_mfma_wide = real
+    rows = {m for m, _ in calls}
+    assert 20 in rows and 40 in rows, rows                      # decode batch and the portion
+    assert {s for _, s in calls} == {1, 2}, calls                # logits whole, projections in two slices
+
+
 def test_prefill_with_the_library_kernel_selection(model_dirs):
     """With tuning on, a prompt portion of a multiple of 256 rows lets torch time the library's
     candidates for its products; whatever it picks, the logits stay those of the plain model."""

@@ -168,6 +168,43 @@ def test_gemm_mfma_skinny_partial_sums_feed_the_norm(ops, m, n, k, splits, waves
         assert torch.equal(res.cpu(), res0) and (out - want[rows.long()]).abs().max() <= tol(dtype, want)
 
 
+@pytest.mark.parametrize("m, n, k, splits, waves", [(17, 151, 256, 1, 0), (64, 272, 1024, 4, 8), (33, 100, 384, 2, 4),
+                                                     (50, 16, 128, 1, 8), (64, 3584, 2048, 8, 0), (40, 1000, 1152, 1, 4),
+                                                     (5, 130, 640, 2, 0)])
+def test_gemm_mfma_wide(ops, m, n, k, splits, waves):
+    """The product that shares the rows of x through LDS: whole, and cut into slices whose partial
+    sums add up; a slice holds its own part of K only; sizes it does not take are refused."""
+    x, w = rnd((m, k), 44, torch.bfloat16), rnd((n, k), 45, torch.bfloat16, 0.05)
+    ref = plain.linear(x.float(), w.float())
+    out = ops.gemm_mfma_wide(x.cuda(), w.cuda(), splits=splits, waves=waves)
+    assert out.dtype == torch.float32 and out.shape == ((m, n) if splits == 1 else (splits, m, n))
+    total = out.cpu() if splits == 1 else out.cpu().double().sum(0).float()
+    assert (total - ref).abs().max() <= 2e-5 * ref.abs().max()  # float32 sums of exact bfloat16 products
+    if splits > 1:
+        k_slice = -(-(-(-k // splits)) // 128) * 128
+        first = plain.linear(x[:, :k_slice].float(), w[:, :k_slice].float())
+        assert (out[0].cpu() - first).abs().max() <= 2e-5 * ref.abs().max()
+        last = plain.linear(x[:, k_slice * (splits - 1):].float(), w[:, k_slice * (splits - 1):].float())
+        assert (out[-1].cpu() - last).abs().max() <= 2e-5 * ref.abs().max()
+    # the same rows give the same sums whatever else is in the batch
+    if m > 3:
+        fewer = ops.gemm_mfma_wide(x[2:m - 1].contiguous().cuda(), w.cuda(), splits=splits, waves=waves)
+        assert torch.equal(fewer.cpu(), out.cpu()[..., 2:m - 1, :])
+
+
+def test_gemm_mfma_wide_refuses_what_it_does_not_take(ops):
+    x, w = rnd((20, 200), 46, torch.bfloat16), rnd((32, 200), 47, torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="whole stages of 128"):
+        ops.gemm_mfma_wide(x.cuda(), w.cuda())
+    x, w = rnd((20, 384), 46, torch.bfloat16), rnd((32, 384), 47, torch.bfloat16)
+    assert not ops.gemm_mfma_wide_splits_ok(384, 4) and ops.gemm_mfma_wide_splits_ok(384, 2)
+    with pytest.raises(ops.KernelError, match="whole stages of 128"):
+        ops.gemm_mfma_wide(x.cuda(), w.cuda(), splits=4)
+    x = rnd((65, 384), 46, torch.bfloat16)
+    with pytest.raises(ops.KernelError, match="at most 64 rows"):
+        ops.gemm_mfma_wide(x.cuda(), w.cuda())
+
+
 def test_rmsnorm_adds_partial_sums_at_odd_sizes(ops):
     """Sizes the vector kernel does not take: hidden not a multiple of 4 and larger than its registers hold."""
     for hidden, n_parts in [(102, 2), (9001 * 4, 4), (4099, 8)]:
