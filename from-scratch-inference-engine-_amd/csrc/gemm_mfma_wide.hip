@@ -178,7 +178,7 @@ extern "C" int fsie_gemm_mfma_wide_slice(int K, int splits) {
 
 // bfloat16 operands, float32 result: y is [M, N] (splits == 1) or [splits, M, N] partial sums.
 // 1 <= M <= 64; K a multiple of 128 that `splits` slices of whole stages cover (see above);
-// x and w 16-byte aligned.  waves: 4 or 8 blocks of 16 rows of W per workgroup, 0 = choose.
+// x and w 16-byte aligned.  waves: 2, 4 or 8 blocks of 16 rows of W per workgroup, 0 = choose.
 extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits,
                                    int waves, hipStream_t stream) {
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -188,7 +188,7 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
     FSIE_REQUIRE(k_slice > 0, "gemm_mfma_wide: K=%d cannot be cut into %d slices of whole stages of 128", K, splits);
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
                  "gemm_mfma_wide: operands must be 16-byte aligned");
-    FSIE_REQUIRE(waves == 0 || waves == 4 || waves == 8, "gemm_mfma_wide: waves must be 0, 4 or 8");
+    FSIE_REQUIRE(waves == 0 || waves == 2 || waves == 4 || waves == 8, "gemm_mfma_wide: waves must be 0, 2, 4 or 8");
     if (M == 0) return 0;
     if (waves == 0) {
         // eight blocks a workgroup halve the reads of X, but only a large N leaves enough
@@ -201,5 +201,6 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
     if (waves == 8) return launch_mt<8, 4>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    if (waves == 2) return launch_mt<2, 4>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
     return launch_mt<4, 4>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
 }

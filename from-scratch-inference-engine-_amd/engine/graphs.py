@@ -11,6 +11,8 @@ there and replays the graph.
 
 from __future__ import annotations
 
+import gc
+import weakref
 from typing import Dict, Optional, Sequence, Tuple
 
 import torch
@@ -22,7 +24,11 @@ PAGE_BUCKET = 32  # block-table widths are rounded up to this many pages
 
 class DecodeGraphs:
     def __init__(self, runner, max_graphs: int = 64):
-        self.runner = runner
+        # no cycle with the runner: a runner that is dropped must free its graphs and pinned
+        # buffers then and there, not whenever the collector of cycles next runs (which may be
+        # in the middle of another runner's capture, where freeing device memory is an error
+        # that ends the process)
+        self._runner = weakref.ref(runner)
         self.max_graphs = max_graphs
         self._graphs: Dict[Tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
         model = runner.model
@@ -30,6 +36,13 @@ class DecodeGraphs:
         self.enabled = all(p.graph_safe for p in parts) and all(hasattr(p, "graph_bucket") for p in model.planners)
         self.replays = 0
         self.captures = 0
+
+    @property
+    def runner(self):
+        runner = self._runner()
+        if runner is None:
+            raise RuntimeError("the runner of these graphs no longer exists")
+        return runner
 
     def shape_of(self, entries: Sequence[StepEntry]) -> Optional[dict]:
         """The padded sizes of this step, or None if it is not a plain decode step."""
@@ -65,8 +78,18 @@ class DecodeGraphs:
             runner.model.forward(ctx, runner.storage)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                logits = runner.model.forward(ctx, runner.storage)
+            # Nothing may free device or pinned memory while the stream is captured.  Dead cycles
+            # of Python objects that hold such memory (or other graphs) are therefore collected
+            # now, and the collector stays off until the capture has ended.
+            gc.collect()
+            collector_was_on = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    logits = runner.model.forward(ctx, runner.storage)
+            finally:
+                if collector_was_on:
+                    gc.enable()
             self._graphs[key] = (graph, tables, logits, ctx.token_ids)
             self.captures += 1
             # the eager run above already wrote this step's keys and values; replaying writes the

@@ -59,10 +59,12 @@ class Linear:
         m = x.shape[0]
         if (getattr(ctx, "partial_sums_ok", False) and x.dtype == torch.bfloat16 and self.bias is None
                 and self.in_features % 8 == 0 and 0 < m <= GEMM_MFMA_SKINNY_MAX_M):
-            if m > GEMM_MFMA_SKINNY_BEST_M:
-                splits = self.wide_splits()
-                if splits > 1:
-                    return ops.gemm_mfma_wide(x, self.weight, splits=splits)
+            # the kernel that shares x through LDS: above 16 rows, and at any number of rows where
+            # K is long enough for eight slices (N = 3584, K = 18944: 26 against 28 us at 8 rows,
+            # 27 against 32 at 16)
+            splits = self.wide_splits()
+            if splits > 1 and (m > GEMM_MFMA_SKINNY_BEST_M or splits == 8):
+                return ops.gemm_mfma_wide(x, self.weight, splits=splits)
             splits = self.residual_splits(m)
             if splits > 1:
                 return ops.gemm_mfma_skinny(x, self.weight, splits=splits)
