@@ -62,7 +62,7 @@ int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const float* bias, 
 // 17 to 64 rows (any number up to 64 is taken): X shared through LDS, float32 result or partial sums
 int fsie_gemm_mfma_wide_slice(int K, int splits);
 int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits, int waves,
-                        hipStream_t stream);
+                        int blocks, hipStream_t stream);
 
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,

@@ -33,9 +33,10 @@ union Frag {
     bf16x8 v;
 };
 
-// MT tiles of 16 rows of X; WAVES waves = WAVES blocks of 16 rows of W per workgroup;
-// STEPS 32-wide MFMA steps per stage (KS = 32 * STEPS values of K).
-template <int MT, int WAVES, int STEPS>
+// MT tiles of 16 rows of X; WAVES waves of NB blocks of 16 rows of W each per workgroup (a wave's
+// blocks share the B fragments it reads from LDS: with four tiles of X one block a wave would be
+// bound by those reads); STEPS 32-wide MFMA steps per stage (KS = 32 * STEPS values of K).
+template <int MT, int WAVES, int STEPS, int NB>
 __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t* __restrict__ x,
                                                                    const bf16_t* __restrict__ w,
                                                                    float* __restrict__ y, int M, int N, int K,
@@ -54,13 +55,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
     const int wave = threadIdx.x >> 6;
     const int row = lane & 15;  // row of the A tile (n) and column of the B tile (m)
     const int kg = lane >> 4;   // which 8 of a step's 32 k values this lane holds
-    const int n0 = (blockIdx.x * WAVES + wave) * 16;
+    const int n0 = (blockIdx.x * WAVES + wave) * 16 * NB;
     const int k_begin = blockIdx.y * k_slice;
     const int k_end = min(K, k_begin + k_slice);
     const int n_stages = (k_end - k_begin) / KS;  // the host makes every slice a multiple of KS
 
     // rows of W past the end repeat the last one; their results are never written
-    const bf16_t* wp = w + static_cast<int64_t>(min(n0 + row, N - 1)) * K + k_begin + kg * 8;
+    const bf16_t* wp[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+        wp[nb] = w + static_cast<int64_t>(min(n0 + nb * 16 + row, N - 1)) * K + k_begin + kg * 8;
     // staging: unit u = (row of X, j = step * 4 + k group); consecutive threads take consecutive
     // 16 bytes of a row
     const bf16_t* xsrc[PER_THREAD];
@@ -74,23 +78,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
         xdst[i] = u < UNITS ? j * PITCH + m : SPARE;
     }
 
-    floatx4 acc[MT];
+    floatx4 acc[NB][MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[nb][t] = floatx4{0.f, 0.f, 0.f, 0.f};
     if (n_stages <= 0) return;
 
     u32x4 xr[PER_THREAD];
-    Frag wa[STEPS], wb[STEPS];  // the W fragments of even and odd stages
+    Frag wa[STEPS][NB], wb[STEPS][NB];  // the W fragments of even and odd stages
     // stage 0
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) xr[i] = *(GlobalVec)(xsrc[i]);
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) wa[s].q = *(GlobalVec)(wp + s * 32);
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) wa[s][nb].q = *(GlobalVec)(wp[nb] + s * 32);
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) xs[0][xdst[i]] = xr[i];
     __syncthreads();
 
-    auto products = [&](int buf, const Frag (&wc)[STEPS]) {
+    auto products = [&](int buf, const Frag (&wc)[STEPS][NB]) {
         const u32x4* xb = xs[buf] + kg * PITCH + row;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
@@ -98,19 +106,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
 #pragma unroll
             for (int t = 0; t < MT; ++t) b[t].q = xb[s * 4 * PITCH + t * 16];
 #pragma unroll
-            for (int t = 0; t < MT; ++t)
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[s].v, b[t].v, acc[t], 0, 0, 0);
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    acc[nb][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wc[s][nb].v, b[t].v, acc[nb][t], 0, 0, 0);
         }
     };
     // A stage that is not the last: fetch the next one (X first, then W into `wn`), work on this
     // one (`wc`, LDS buffer `buf`), hand the next X to the other buffer.  No branch lies around
     // the loads and no register is copied, so the wait before the products counts exactly the
     // loads issued after this stage's W.
-    auto stage = [&](int buf, const Frag (&wc)[STEPS], Frag (&wn)[STEPS], int k1) {
+    auto stage = [&](int buf, const Frag (&wc)[STEPS][NB], Frag (&wn)[STEPS][NB], int k1) {
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) xr[i] = *(GlobalVec)(xsrc[i] + k1);
 #pragma unroll
-        for (int s = 0; s < STEPS; ++s) wn[s].q = *(GlobalVec)(wp + k1 + s * 32);
+        for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) wn[s][nb].q = *(GlobalVec)(wp[nb] + k1 + s * 32);
         __builtin_amdgcn_sched_barrier(0);
         products(buf, wc);
         __builtin_amdgcn_sched_barrier(0);
@@ -130,37 +142,40 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
         products(0, wa);
     }
 
-    // lane holds D[n0 + 4 kg + r][m = 16 t + row]
+    // lane holds D[n0 + 16 nb + 4 kg + r][m = 16 t + row]
     float* part = y + static_cast<int64_t>(blockIdx.y) * M * N;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        const int m = t * 16 + row;
-        if (m >= M) continue;
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int nn = n0 + kg * 4 + r;
-            if (nn < N) part[static_cast<int64_t>(m) * N + nn] = acc[t][r];
+        for (int t = 0; t < MT; ++t) {
+            const int m = t * 16 + row;
+            if (m >= M) continue;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int nn = n0 + nb * 16 + kg * 4 + r;
+                if (nn < N) part[static_cast<int64_t>(m) * N + nn] = acc[nb][t][r];
+            }
         }
-    }
 }
 
-template <int MT, int WAVES, int STEPS>
+template <int MT, int WAVES, int STEPS, int NB>
 int launch(const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
            hipStream_t stream) {
-    const dim3 grid(static_cast<unsigned>((N + 16 * WAVES - 1) / (16 * WAVES)), static_cast<unsigned>(splits));
-    gemm_mfma_wide_kernel<MT, WAVES, STEPS><<<grid, WAVES * 64, 0, stream>>>(x, w, y, M, N, K, k_slice);
+    const int rows = 16 * NB * WAVES;
+    const dim3 grid(static_cast<unsigned>((N + rows - 1) / rows), static_cast<unsigned>(splits));
+    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB><<<grid, WAVES * 64, 0, stream>>>(x, w, y, M, N, K, k_slice);
     FSIE_CHECK_LAUNCH("gemm_mfma_wide");
     return 0;
 }
 
-template <int WAVES, int STEPS>
+template <int WAVES, int STEPS, int NB>
 int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
               hipStream_t stream) {
     switch (mt) {
-        case 1: return launch<1, WAVES, STEPS>(x, w, y, M, N, K, splits, k_slice, stream);
-        case 2: return launch<2, WAVES, STEPS>(x, w, y, M, N, K, splits, k_slice, stream);
-        case 3: return launch<3, WAVES, STEPS>(x, w, y, M, N, K, splits, k_slice, stream);
-        default: return launch<4, WAVES, STEPS>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 1: return launch<1, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 2: return launch<2, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 3: return launch<3, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
+        default: return launch<4, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
     }
 }
 
@@ -178,9 +193,10 @@ extern "C" int fsie_gemm_mfma_wide_slice(int K, int splits) {
 
 // bfloat16 operands, float32 result: y is [M, N] (splits == 1) or [splits, M, N] partial sums.
 // 1 <= M <= 64; K a multiple of 128 that `splits` slices of whole stages cover (see above);
-// x and w 16-byte aligned.  waves: 2, 4 or 8 blocks of 16 rows of W per workgroup, 0 = choose.
+// x and w 16-byte aligned.  waves: 2, 4 or 8 waves per workgroup; blocks: 1 or 2 blocks of 16 rows
+// of W per wave; 0 = choose.
 extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits,
-                                   int waves, hipStream_t stream) {
+                                   int waves, int blocks, hipStream_t stream) {
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide: bad sizes M=%d N=%d K=%d", M, N, K);
     FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide: at most %d rows, got %d",
                  FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
@@ -189,18 +205,30 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
                  "gemm_mfma_wide: operands must be 16-byte aligned");
     FSIE_REQUIRE(waves == 0 || waves == 2 || waves == 4 || waves == 8, "gemm_mfma_wide: waves must be 0, 2, 4 or 8");
+    FSIE_REQUIRE(blocks == 0 || blocks == 1 || blocks == 2, "gemm_mfma_wide: blocks must be 0, 1 or 2");
     if (M == 0) return 0;
-    if (waves == 0) {
-        // eight blocks a workgroup halve the reads of X, but only a large N leaves enough
-        // workgroups for them (measured on MI355X, 64 rows: N = 152064 242 against 261 us;
-        // N = 3584, K = 18944 in 8 slices 39.6 against 38.1)
-        const int64_t groups4 = static_cast<int64_t>((N + 63) / 64) * splits;
-        waves = groups4 >= 1024 ? 8 : 4;
-    }
     const int mt = (M + 15) / 16;
+    if (blocks == 0) {
+        // three or four tiles of X: two blocks of W a wave share the B fragments read from LDS,
+        // where that still leaves a workgroup for most compute units (measured on MI355X, 64 rows,
+        // N = 3584, K = 18944 in 8 slices: 33.6 against 37.7 us)
+        blocks = (mt >= 3 && static_cast<int64_t>((N + 127) / 128) * splits >= 128) ? 2 : 1;
+    }
+    if (waves == 0) {
+        // eight waves a workgroup halve the reads of X, but only a large N leaves enough
+        // workgroups for them (64 rows: N = 152064 242 against 261 us; N = 3584, K = 18944 in 8
+        // slices 39.6 against 38.1); with two blocks a wave, four waves (N = 152064: 236 against 260)
+        const int64_t groups4 = static_cast<int64_t>((N + 63) / 64) * splits;
+        waves = (groups4 >= 1024 && blocks == 1) ? 8 : 4;
+    }
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
-    if (waves == 8) return launch_mt<8, 4>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-    if (waves == 2) return launch_mt<2, 4>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-    return launch_mt<4, 4>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    if (blocks == 2) {
+        if (waves == 8) return launch_mt<8, 4, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+        if (waves == 2) return launch_mt<2, 4, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+        return launch_mt<4, 4, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    }
+    if (waves == 8) return launch_mt<8, 4, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    if (waves == 2) return launch_mt<2, 4, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    return launch_mt<4, 4, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
 }

@@ -223,7 +223,7 @@ def gemm_mfma_wide_splits_ok(k: int, splits: int) -> bool:
 
 
 def gemm_mfma_wide(x: torch.Tensor, weight: torch.Tensor, splits: int = 1, waves: int = 0,
-                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   out: Optional[torch.Tensor] = None, blocks: int = 0) -> torch.Tensor:
     """x [M, K] . weight [N, K]^T for bfloat16 operands and up to 64 rows, the rows of x shared by
     a workgroup's waves through LDS (made for 17 rows and more).  The result is float32: [M, N],
     or with ``splits`` in (2, 4, 8) the partial sums [splits, M, N] of the slices of K, for
@@ -242,7 +242,7 @@ def gemm_mfma_wide(x: torch.Tensor, weight: torch.Tensor, splits: int = 1, waves
         out = torch.empty(shape, dtype=torch.float32, device=x.device)
     _need(out, "gemm out", dtype=torch.float32, shape=shape)
     check(load().fsie_gemm_mfma_wide(x.data_ptr(), weight.data_ptr(), out.data_ptr(), m, n, k, splits, waves,
-                                     _stream()))
+                                     blocks, _stream()))
     return out
 
 

@@ -190,6 +190,10 @@ def test_gemm_mfma_wide(ops, m, n, k, splits, waves):
     if m > 3:
         fewer = ops.gemm_mfma_wide(x[2:m - 1].contiguous().cuda(), w.cuda(), splits=splits, waves=waves)
         assert torch.equal(fewer.cpu(), out.cpu()[..., 2:m - 1, :])
+    # and whatever the launch shape: one or two blocks of W a wave, 2, 4 or 8 waves a workgroup
+    for blocks, wv in [(1, 2), (2, 4), (2, 8), (1, 8), (2, 2)]:
+        other = ops.gemm_mfma_wide(x.cuda(), w.cuda(), splits=splits, waves=wv, blocks=blocks)
+        assert torch.equal(other.cpu(), out.cpu()), (blocks, wv)
 
 
 def test_gemm_mfma_wide_refuses_what_it_does_not_take(ops):
