@@ -5,9 +5,11 @@ reference's engine calls cuBLAS there).  The library picks one of its kernels by
 other kernels are sometimes a good deal faster (measured on MI355X at 2,048 rows: 462 against
 568 us for N = 37888, K = 3584, and 261 against 357 us for N = 3584, K = 18944).  With tuning on,
 torch's TunableOp times the library's candidates the first time a shape is seen and keeps the
-best (in the process, and in a file under the temporary folder for later ones).  Only row counts that are a multiple of 256 are tuned (a full
-token budget; each new shape costs seconds), never inside a graph capture; other shapes use what
-has been found for them, or the heuristic.
+best (in the process, and in a file under the temporary folder for later ones).  Each new shape
+costs seconds, so only two kinds of row counts are tuned: multiples of 256 (a full token budget of
+prefill) and multiples of 16 up to 64 (decode batches, timed in the eager run that precedes the
+capture of their graph); never inside a graph capture.  Other shapes use what has been found for
+them, or the heuristic.
 """
 
 from __future__ import annotations
@@ -18,6 +20,7 @@ import tempfile
 import torch
 
 _TUNED_ROWS = 256
+_TUNED_DECODE_ROWS, _TUNED_DECODE_MAX = 16, 64
 _state = {"on": False}
 
 
@@ -54,7 +57,8 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     import torch.cuda.tunable as tunable
 
     rows = x.shape[0]
-    tune = rows >= _TUNED_ROWS and rows % _TUNED_ROWS == 0 and not torch.cuda.is_current_stream_capturing()
+    tune = ((rows % _TUNED_ROWS == 0 or (rows <= _TUNED_DECODE_MAX and rows % _TUNED_DECODE_ROWS == 0)) and rows > 0
+            and not torch.cuda.is_current_stream_capturing())
     if not tune:
         return torch.mm(x, weight.t())
     tunable.tuning_enable(True)

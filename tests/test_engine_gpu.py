@@ -299,8 +299,9 @@ def test_batches_of_17_to_64_rows_share_x_through_lds(tmp_path):
 
 
 def test_prefill_with_the_library_kernel_selection(model_dirs):
-    """With tuning on, a prompt portion of a multiple of 256 rows lets torch time the library's
-    candidates for its products; whatever it picks, the logits stay those of the plain model."""
+    """With tuning on, a prompt portion of a multiple of 256 rows, and a decode batch of a multiple
+    of 16, let torch time the library's candidates for their products; whatever it picks, the
+    logits stay those of the plain model."""
     from from_scratch_inference_engine_amd import load_model, ops
     from from_scratch_inference_engine_amd.engine.context import StepEntry
     from from_scratch_inference_engine_amd.engine.model import Runner
@@ -313,9 +314,24 @@ def test_prefill_with_the_library_kernel_selection(model_dirs):
         assert ops.library_tuning_enabled()
         runner = Runner(load_model(model_dirs["B"], dtype="bfloat16"), page_size=16, num_pages=32, max_requests=2)
         out = runner.step([StepEntry(runner.manager.open("a"), ids, list(range(256)))]).float().cpu().numpy()
+        # a decode batch of 32: its library products are timed in the eager run before the capture,
+        # the captured graph then replays the chosen kernels
+        runner = Runner(load_model(model_dirs["B"], dtype="bfloat16"), page_size=16, num_pages=80, max_requests=32)
+        seqs = [helpers.token_ids(vocab, 6 + i % 5, 820 + i) for i in range(32)]
+        refs = [plain.forward_dir(model_dirs["B"], s_).numpy() for s_ in seqs[:5]]
+        caches = [runner.manager.open(i) for i in range(32)]
+        runner.step([StepEntry(c, s_[:-3], []) for c, s_ in zip(caches, seqs)])
+        decoded = []
+        for t in range(3, 0, -1):
+            decoded.append(runner.step([StepEntry(c, [s_[-t]], [0]) for c, s_ in zip(caches, seqs)]).float().cpu().numpy())
+        assert runner.graphs.captures == 1 and runner.graphs.replays == 2
     finally:
         ops.disable_library_tuning()
     helpers.assert_close_to_plain(out, ref, "bfloat16", "prefill of 256 rows with library tuning")
+    for i in range(5):
+        for j in range(3):
+            helpers.assert_close_to_plain(decoded[j][i:i + 1], refs[i][len(seqs[i]) - 3 + j:len(seqs[i]) - 2 + j], "bfloat16",
+                                          f"decode batch of 32 with library tuning, request {i} token {j}")
 
 
 def test_a_dropped_runner_frees_its_graphs_at_once(model_dirs):
