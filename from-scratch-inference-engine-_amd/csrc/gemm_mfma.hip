@@ -2,6 +2,23 @@
 // the choice of the launch shape.
 #include "gemm_mfma_impl.h"
 
+namespace {
+
+// compute units of the current device (0 if it cannot be asked), asked once per device
+int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+}  // namespace
+
 // bfloat16 only.  M <= 64, K a multiple of 8, x and w 16-byte aligned.
 // waves (K split inside a workgroup) and blocks (16-row blocks of W per workgroup): 0 = choose.
 // epilogue: 0 = y = d (+ bias); 1 = SiLU*up over interleaved gate/up rows (N even, no bias, y is [M, N/2]).
@@ -87,16 +104,28 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     const int N = (n_heads + 2 * n_kv) * head_dim;
     const int mt = (M + 15) / 16;
     const int pairs = (K + 2 * fsie_mm::kStep - 1) / (2 * fsie_mm::kStep);
-    const int blocks = 1;
+    // Rotary pairs a workgroup owns: 8 (one block of 16 rows).  A product this small is bound by
+    // what a compute unit's memory pipeline gives, so the busiest unit sets the time: where eight
+    // pairs a workgroup would leave some units two workgroups and others one (N = 4608 on 256
+    // units: 288 workgroups), the pairs are dealt evenly instead, 9 to 16 a workgroup, in two blocks
+    // of which the second is partly filled.
+    const int total_pairs = N / 2;
+    const int units = compute_units();
+    int pairs_per_wg = 8;
+    if (mt == 1 && M > 4 && units > 0 && total_pairs > 8 * units && total_pairs <= 16 * units) {  // (no gain at 1 row)
+        pairs_per_wg = (total_pairs + units - 1) / units;
+    }
+    const int blocks = pairs_per_wg > 8 ? 2 : 1;
+    const int groups = (total_pairs + pairs_per_wg - 1) / pairs_per_wg;
     int waves = 1;
     // (more waves than this only add to the reduction: 12.6 us with four against 14.1 with eight
     // at N = 4608, K = 3584 and one row)
-    while (waves < 16 && (N / 16) * waves < 1024) waves *= 2;
+    while (waves < 16 && groups * waves < 1024) waves *= 2;
     while (waves > 1 && pairs < 2 * waves) waves /= 2;
     if (mt * blocks > 4 && waves > 8) waves = 8;  // LDS of the reduction
     const fsie_mm::Call call{x, w, bias, y, M, N, K, 1, stream,
                                fsie_mm::RopeArgs{positions, slots, inv_freq, static_cast<bf16_t*>(store ? k_pool : nullptr),
                                                    static_cast<bf16_t*>(store ? v_pool : nullptr), n_heads, n_kv, head_dim,
-                                                   store ? page_size : 1, store ? pool_slots : 0}};
+                                                   store ? page_size : 1, store ? pool_slots : 0, pairs_per_wg}};
     return fsie_mm::launch_rope(mt, waves, call);
 }

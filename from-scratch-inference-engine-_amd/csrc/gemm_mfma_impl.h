@@ -40,6 +40,7 @@ struct RopeArgs {
     bf16_t* v_pool;          // [pages][n_kv][head_dim][page_size]
     int n_heads, n_kv, head_dim, page_size;
     int64_t pool_slots;
+    int pairs_per_wg;  // rotary pairs (rows i and i + head_dim / 2 of a head) a workgroup owns: 1..8 * NB
 };
 
 // angle = position * inv_freq in float64, reduced in float64 to [-pi, pi], then float32 sine and
@@ -55,9 +56,13 @@ __device__ __forceinline__ void rotation(double pos, double inv_freq, float* c, 
 // fragments), WAVES = waves of the workgroup, which split K.
 // EPI_SWIGLU: the rows of W are gate and up interleaved; the output has N/2 columns,
 // y[m, j] = silu(d[2j]) * d[2j + 1], computed in float32 from the accumulators.
-// EPI_ROPE: see RopeArgs.  A block of 16 rows of a q or k head then holds rows 8b..8b+7 of the
-// head's first half and the same of its second half, so that both members of every rotary pair
-// (i, i + head_dim/2) lie in one accumulator tile, 32 lanes apart.
+// EPI_ROPE: see RopeArgs.  The rows of W are taken in pairs (i, i + head_dim/2) of a head, numbered
+// through all heads; a workgroup owns `pairs_per_wg` consecutive pairs, eight to a block: tile rows
+// 0..7 are the first members, rows 8..15 the second, so that both members of a pair lie in one
+// accumulator tile, 32 lanes apart.  A block that is not full repeats the workgroup's last pair
+// (the same addresses again: no further memory traffic) and does not write the repeats.  The
+// number of pairs a workgroup owns is the host's choice: it spreads the rows evenly over the
+// compute units, whose memory pipelines bound a product this small.
 // blockIdx.y selects a slice of K of `k_slice` values (a multiple of 64); with more than one slice
 // the kernel writes float32 partial sums y[slice][m][n] without bias, for the consumer to add up
 // in the order of the slices.
@@ -77,12 +82,12 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
     for (int b = 0; b < NB; ++b) {
         int n = n0 + b * 16 + row;
         if (EPI == EPI_ROPE) {
-            const int per_head = rope.head_dim / 16;
-            const int block = blockIdx.x * NB + b;
-            const int head = block / per_head, sub = block - head * per_head;
-            if (head < rope.n_heads + rope.n_kv) {
-                n = head * rope.head_dim + sub * 8 + (row < 8 ? row : rope.head_dim / 2 + row - 8);
-            }
+            const int half = rope.head_dim / 2;
+            const int base = blockIdx.x * rope.pairs_per_wg;
+            const int here = min(rope.pairs_per_wg, N / 2 - base);  // at least 1: the grid covers N / 2 pairs
+            const int pair = base + min(b * 8 + (row & 7), here - 1);
+            const int head = pair / half;
+            n = head * rope.head_dim + (pair - head * half) + (row < 8 ? 0 : half);
         }
         n = min(n, N - 1);  // rows past the end repeat the last one; never written
         wp[b] = w + static_cast<int64_t>(n) * K;
@@ -98,6 +103,43 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
     for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[b][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // What the rotary epilogue reads from memory (positions, slots, bias, frequencies) is asked for
+    // here, so that it arrives while W streams: the epilogue runs after the other waves have left,
+    // and every microsecond of it is added to the kernel's time.  Every wave asks (no branch lies
+    // around the loads, so nothing waits for them here); a table that does not exist is replaced
+    // by the start of W, and what is read there is dropped.
+    float e_bias[NB][4];
+    double e_freq[NB][4];
+    int e_pos[MT], e_slot[MT];
+    if (EPI == EPI_ROPE) {
+        const int half = rope.head_dim / 2;
+        const int base = blockIdx.x * rope.pairs_per_wg;
+        const int here = min(rope.pairs_per_wg, N / 2 - base);
+        const float* bias_src = bias ? bias : reinterpret_cast<const float*>(w);
+        const double* freq_src = rope.inv_freq ? rope.inv_freq : reinterpret_cast<const double*>(w);
+        const bool stores = rope.k_pool && rope.slots;
+        const int32_t* slot_src = stores ? rope.slots : rope.positions;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int pair = base + min(nb * 8 + (kg & 1) * 4 + r, here - 1);
+                const int head = pair / half;
+                const int i = pair - head * half;
+                const float b = bias_src[bias ? head * rope.head_dim + i + (kg >= 2 ? half : 0) : 0];
+                const double f = freq_src[rope.inv_freq ? i : 0];
+                e_bias[nb][r] = bias ? b : 0.f;
+                e_freq[nb][r] = f;
+            }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int m = min(t * 16 + row, M - 1);
+            e_pos[t] = rope.positions[m];
+            const int sl = slot_src[m];
+            e_slot[t] = stores ? sl : -1;
+        }
+    }
 
     // k steps of 32; a wave takes pairs of steps (128 bytes of every row), pairs interleaved over the waves
     const int k_begin = blockIdx.y * k_slice;
@@ -172,52 +214,42 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
                 continue;
             }
             if (EPI == EPI_ROPE) {
-                const int per_head = rope.head_dim / 16;
-                const int block = blockIdx.x * NB + nb;
-                if (block * 16 >= N) continue;  // N is a multiple of 16 here
-                const int head = block / per_head, sub = block - head * per_head;
-                const int rot_heads = rope.n_heads + rope.n_kv;
+                // tile row 4 kg + r: pair (kg & 1) * 4 + r of block nb, first member for kg < 2, second else
                 const int half = rope.head_dim / 2;
-                int slot = (rope.k_pool && rope.slots) ? rope.slots[m] : -1;
+                const int rot_heads = rope.n_heads + rope.n_kv;
+                const int base = blockIdx.x * rope.pairs_per_wg;
+                const int here = min(rope.pairs_per_wg, N / 2 - base);
+                const bool second = kg >= 2;
+                int slot = e_slot[t];
                 if (slot >= rope.pool_slots) slot = -1;
                 const int64_t page = slot >= 0 ? slot / rope.page_size : 0;
                 const int off = slot >= 0 ? slot % rope.page_size : 0;
-                if (head < rot_heads) {
-                    // tile rows 0..7: dimensions i = 8 sub + (0..7); rows 8..15: i + half
-                    const bool second = kg >= 2;
-                    const int i0 = sub * 8 + (kg & 1) * 4;
-                    const int col0 = head * rope.head_dim + i0 + (second ? half : 0);
-                    const double pos = static_cast<double>(rope.positions[m]);
-                    bf16_t res[4];
+                const double pos = static_cast<double>(e_pos[t]);
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float mine = acc[nb][t][r] + (bias ? bias[col0 + r] : 0.f);
-                        const float other = __shfl_xor(mine, 32, FSIE_WAVE);
+                for (int r = 0; r < 4; ++r) {
+                    const int lp = nb * 8 + (kg & 1) * 4 + r;
+                    const bool mine_to_write = lp < here;  // a repeat of the last pair otherwise
+                    const int pair = base + min(lp, here - 1);
+                    const int head = pair / half;
+                    const int i = pair - head * half;
+                    const int d = i + (second ? half : 0);  // dimension within the head
+                    const int col = head * rope.head_dim + d;
+                    const float mine = acc[nb][t][r] + e_bias[nb][r];
+                    const float other = __shfl_xor(mine, 32, FSIE_WAVE);  // every lane takes part
+                    if (head < rot_heads) {
                         float c = 1.f, sn = 0.f;
-                        if (rope.inv_freq) rotation(pos, rope.inv_freq[i0 + r], &c, &sn);
+                        if (rope.inv_freq) rotation(pos, e_freq[nb][r], &c, &sn);
                         // first half: x1 c - x2 s; second half: x2 c + x1 s
-                        res[r] = from_float<bf16_t>(second ? mine * c + other * sn : mine * c - other * sn);
-                    }
-                    if (head < rope.n_heads) {
-                        bf16_t* dst = reinterpret_cast<bf16_t*>(y) + static_cast<int64_t>(m) * N + col0;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) dst[r] = res[r];
-                    } else if (slot >= 0) {
-                        bf16_t* dst = rope.k_pool +
-                                      ((page * rope.n_kv + (head - rope.n_heads)) * rope.page_size + off) * rope.head_dim +
-                                      (col0 - head * rope.head_dim);
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) dst[r] = res[r];
-                    }
-                } else if (slot >= 0) {
-                    const int kvh = head - rot_heads;
-                    const int d0 = sub * 16 + kg * 4;
-                    const int col0 = head * rope.head_dim + d0;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float v = acc[nb][t][r] + (bias ? bias[col0 + r] : 0.f);
-                        rope.v_pool[((page * rope.n_kv + kvh) * rope.head_dim + d0 + r) * rope.page_size + off] =
-                            from_float<bf16_t>(v);
+                        const bf16_t res = from_float<bf16_t>(second ? mine * c + other * sn : mine * c - other * sn);
+                        if (!mine_to_write) continue;
+                        if (head < rope.n_heads) {
+                            reinterpret_cast<bf16_t*>(y)[static_cast<int64_t>(m) * N + col] = res;
+                        } else if (slot >= 0) {
+                            rope.k_pool[((page * rope.n_kv + (head - rope.n_heads)) * rope.page_size + off) * rope.head_dim + d] = res;
+                        }
+                    } else if (mine_to_write && slot >= 0) {
+                        rope.v_pool[((page * rope.n_kv + (head - rot_heads)) * rope.head_dim + d) * rope.page_size + off] =
+                            from_float<bf16_t>(mine);
                     }
                 }
                 continue;
@@ -258,8 +290,9 @@ struct Call {
 template <int MT, int NB, int WAVES, typename OutT, int EPI>
 int launch(const Call& c) {
     const int k_slice = c.splits > 1 ? ((c.K + c.splits - 1) / c.splits + 63) / 64 * 64 : c.K;
-    const dim3 grid(static_cast<unsigned>((c.N + 16 * NB - 1) / (16 * NB)),
-                    static_cast<unsigned>(c.splits > 1 ? c.splits : 1));
+    const unsigned groups = EPI == EPI_ROPE ? (c.N / 2 + c.rope.pairs_per_wg - 1) / c.rope.pairs_per_wg
+                                            : (c.N + 16 * NB - 1) / (16 * NB);
+    const dim3 grid(groups, static_cast<unsigned>(c.splits > 1 ? c.splits : 1));
     gemm_mfma_skinny_kernel<MT, NB, WAVES, OutT, EPI><<<grid, WAVES * FSIE_WAVE, 0, c.stream>>>(
         static_cast<const bf16_t*>(c.x), static_cast<const bf16_t*>(c.w), c.bias, static_cast<OutT*>(c.y), c.M, c.N,
         c.K, k_slice, c.rope);
@@ -292,6 +325,7 @@ int launch_blocks(int nb, int waves, const Call& c) {
 int launch_f32(int mt, int blocks, int waves, const Call& c);      // float32 result or partial sums, up to 64 rows
 int launch_bf16(int blocks, int waves, const Call& c);             // bfloat16 result, up to 16 rows
 int launch_swiglu(int blocks, int waves, const Call& c);           // SiLU*up epilogue, up to 16 rows
-int launch_rope(int mt, int waves, const Call& c);                 // q/k/v + rotary epilogue, one block, up to 64 rows
+int launch_rope(int mt, int waves, const Call& c);                 // q/k/v + rotary epilogue, up to 64 rows; two blocks a
+                                                                   // workgroup (9 to 16 pairs) for one tile of x only
 
 }  // namespace fsie_mm
