@@ -48,6 +48,10 @@ int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int32_t* slots
                        const float* bias, void* k_pool, void* v_pool, int n_tokens, int n_heads, int n_kv, int head_dim,
                        int rotary_dim, int page_size, int64_t pool_slots, int dtype, hipStream_t stream);
 
+// table [n_tokens, half, 2] float32: cos and sin of positions[t] * inv_freq[i]
+int fsie_rope_table(const int32_t* positions, const double* inv_freq, int n_tokens, int half, float* table,
+                    hipStream_t stream);
+
 int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, int N, int K, int dtype,
               int out_f32, int kind, hipStream_t stream);
 
@@ -55,7 +59,8 @@ int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void*
                           int out_f32, int waves, int blocks, int epilogue, int splits, hipStream_t stream);
 
 int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const float* bias, void* y, int M, int K,
-                               const int32_t* positions, const int32_t* slots, const double* inv_freq, void* k_pool,
+                               const int32_t* positions, const int32_t* slots, const double* inv_freq,
+                               const float* cos_sin, void* k_pool,
                                void* v_pool, int n_heads, int n_kv, int head_dim, int page_size, int64_t pool_slots,
                                hipStream_t stream);
 

@@ -86,7 +86,8 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
 // is stored.  M <= 64, K a multiple of 8.
 extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const float* bias, void* y, int M, int K,
                                           const int32_t* positions, const int32_t* slots, const double* inv_freq,
-                                          void* k_pool, void* v_pool, int n_heads, int n_kv, int head_dim,
+                                          const float* cos_sin, void* k_pool, void* v_pool, int n_heads, int n_kv,
+                                          int head_dim,
                                           int page_size, int64_t pool_slots, hipStream_t stream) {
     FSIE_REQUIRE(M >= 0 && K > 0 && n_heads > 0 && n_kv > 0, "gemm_mfma_skinny_rope: bad sizes");
     FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_skinny_rope: at most %d rows, got %d",
@@ -97,6 +98,8 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
                  "gemm_mfma_skinny_rope: operands must be 16-byte aligned");
     FSIE_REQUIRE(positions, "gemm_mfma_skinny_rope: no positions");
+    FSIE_REQUIRE(!cos_sin || (inv_freq && reinterpret_cast<uintptr_t>(cos_sin) % 8 == 0),
+                 "gemm_mfma_skinny_rope: a table of cosines and sines goes with a frequency table and is 8-byte aligned");
     const bool store = k_pool != nullptr;
     FSIE_REQUIRE(!store || (v_pool && slots && page_size > 0 && pool_slots > 0),
                  "gemm_mfma_skinny_rope: a cache needs both pools, slots and a page geometry");
@@ -124,7 +127,7 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     while (waves > 1 && pairs < 2 * waves) waves /= 2;
     if (mt * blocks > 4 && waves > 8) waves = 8;  // LDS of the reduction
     const fsie_mm::Call call{x, w, bias, y, M, N, K, 1, stream,
-                               fsie_mm::RopeArgs{positions, slots, inv_freq, static_cast<bf16_t*>(store ? k_pool : nullptr),
+                               fsie_mm::RopeArgs{positions, slots, inv_freq, cos_sin, static_cast<bf16_t*>(store ? k_pool : nullptr),
                                                    static_cast<bf16_t*>(store ? v_pool : nullptr), n_heads, n_kv, head_dim,
                                                    store ? page_size : 1, store ? pool_slots : 0, pairs_per_wg}};
     return fsie_mm::launch_rope(mt, waves, call);

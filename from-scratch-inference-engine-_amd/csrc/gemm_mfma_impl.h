@@ -36,6 +36,8 @@ struct RopeArgs {
     const int32_t* positions;
     const int32_t* slots;
     const double* inv_freq;  // head_dim / 2 entries; null = no rotation
+    const float* cos_sin;    // [M][head_dim / 2][2]: cos and sin of positions[m] * inv_freq[i], computed once
+                             // for all layers of a step; null = the epilogue computes them
     bf16_t* k_pool;          // [pages][n_kv][page_size][head_dim]; null = nothing stored
     bf16_t* v_pool;          // [pages][n_kv][head_dim][page_size]
     int n_heads, n_kv, head_dim, page_size;
@@ -111,6 +113,7 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
     // by the start of W, and what is read there is dropped.
     float e_bias[NB][4];
     double e_freq[NB][4];
+    float2 e_cs[NB][MT][4];
     int e_pos[MT], e_slot[MT];
     if (EPI == EPI_ROPE) {
         const int half = rope.head_dim / 2;
@@ -120,6 +123,7 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         const double* freq_src = rope.inv_freq ? rope.inv_freq : reinterpret_cast<const double*>(w);
         const bool stores = rope.k_pool && rope.slots;
         const int32_t* slot_src = stores ? rope.slots : rope.positions;
+        const float2* cs_src = reinterpret_cast<const float2*>(rope.cos_sin ? rope.cos_sin : reinterpret_cast<const float*>(w));
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -131,6 +135,11 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
                 const double f = freq_src[rope.inv_freq ? i : 0];
                 e_bias[nb][r] = bias ? b : 0.f;
                 e_freq[nb][r] = f;
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const int m = min(t * 16 + row, M - 1);
+                    e_cs[nb][t][r] = cs_src[rope.cos_sin ? m * half + i : 0];
+                }
             }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
@@ -238,7 +247,12 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
                     const float other = __shfl_xor(mine, 32, FSIE_WAVE);  // every lane takes part
                     if (head < rot_heads) {
                         float c = 1.f, sn = 0.f;
-                        if (rope.inv_freq) rotation(pos, e_freq[nb][r], &c, &sn);
+                        if (rope.cos_sin) {
+                            c = e_cs[nb][t][r].x;
+                            sn = e_cs[nb][t][r].y;
+                        } else if (rope.inv_freq) {
+                            rotation(pos, e_freq[nb][r], &c, &sn);
+                        }
                         // first half: x1 c - x2 s; second half: x2 c + x1 s
                         const bf16_t res = from_float<bf16_t>(second ? mine * c + other * sn : mine * c - other * sn);
                         if (!mine_to_write) continue;

@@ -112,7 +112,32 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_kernel(
     }
 }
 
+// table[t][i] = (cos, sin) of positions[t] * inv_freq[i]: the angles of a step are the same in
+// every layer, so a step computes them once and the layers' kernels read them.
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const double* __restrict__ inv_freq,
+                                  float2* __restrict__ table, int half) {
+    const int t = blockIdx.x;
+    const double pos = static_cast<double>(positions[t]);
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float c, s;
+        rotation(pos, inv_freq[i], &c, &s);
+        table[static_cast<int64_t>(t) * half + i] = float2{c, s};
+    }
+}
+
 }  // namespace
+
+extern "C" int fsie_rope_table(const int32_t* positions, const double* inv_freq, int n_tokens, int half,
+                               float* table, hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && half > 0 && half <= kMaxHalf, "rope_table: bad sizes T=%d half=%d", n_tokens, half);
+    FSIE_REQUIRE(positions && inv_freq && table, "rope_table: missing operand");
+    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(table) % 8 == 0, "rope_table: the table must be 8-byte aligned");
+    if (n_tokens == 0) return 0;
+    rope_table_kernel<<<n_tokens, half < 64 ? 64 : (half < 256 ? half : 256), 0, stream>>>(
+        positions, inv_freq, reinterpret_cast<float2*>(table), half);
+    FSIE_CHECK_LAUNCH("rope_table");
+    return 0;
+}
 
 extern "C" int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int32_t* slots,
                                   const double* inv_freq, const float* bias, void* k_pool, void* v_pool, int n_tokens,

@@ -129,6 +129,9 @@ class StepContext:
         self.block_tables: List[torch.Tensor] = []
         self.slots: List[torch.Tensor] = []
         self._plans: Dict[Hashable, SimpleNamespace] = {}
+        # what a part computes once per forward pass and its siblings in other layers use again
+        # (keyed by whatever identifies it); emptied when a forward pass starts
+        self.memo: Dict[Hashable, object] = {}
 
     def plan(self, planner) -> SimpleNamespace:
         try:

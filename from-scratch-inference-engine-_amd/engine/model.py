@@ -140,6 +140,7 @@ class Model:
         """float32 logits [wanted, vocab] for the step described by ``ctx``."""
         spec = self.spec
         ctx.partial_sums_ok = self.partial_sums_ok
+        ctx.memo.clear()  # a captured graph must hold whatever the layers share: nothing is kept from an earlier pass
         hidden = HiddenState(spec.embedding.forward(ctx.token_ids))
         for i, call in enumerate(spec.schedule):
             cid = self.call_cache[i]

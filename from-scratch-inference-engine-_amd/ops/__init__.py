@@ -6,10 +6,10 @@ computes with torch; a missing kernel library is an error, not a reason to fall 
 """
 
 from .functions import (bias_add, attention_merge, attention_mfma, attention_mfma_max_waves, attention_mfma_rows, attention_mfma_lds, attention_mfma_lds_ok, attention_scalar, attention_tile_tokens, dtype_code,
-                        embedding, gemm, gemm_mfma_skinny, gemm_mfma_skinny_rope, gemm_mfma_wide, gemm_mfma_wide_splits_ok, residual_add, rmsnorm, rope_kv_write, sample, swiglu)
+                        embedding, gemm, gemm_mfma_skinny, gemm_mfma_skinny_rope, gemm_mfma_wide, gemm_mfma_wide_splits_ok, residual_add, rmsnorm, rope_kv_write, rope_table, sample, swiglu)
 from .library import KernelError, KernelLibraryMissing, load
 from .tuning import disable_library_tuning, enable_library_tuning, library_mm, library_tuning_enabled
 
 __all__ = ["disable_library_tuning", "enable_library_tuning", "library_mm", "library_tuning_enabled", "KernelError", "KernelLibraryMissing", "attention_merge", "attention_mfma", "attention_mfma_max_waves", "attention_mfma_rows", "attention_mfma_lds", "attention_mfma_lds_ok", "attention_scalar", "bias_add",
            "attention_tile_tokens", "dtype_code", "embedding", "gemm", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "gemm_mfma_wide", "gemm_mfma_wide_splits_ok", "load", "residual_add",
-           "rmsnorm", "rope_kv_write", "sample", "swiglu"]
+           "rmsnorm", "rope_kv_write", "rope_table", "sample", "swiglu"]

@@ -250,12 +250,14 @@ def gemm_mfma_skinny_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[
                           positions: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
                           inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor] = None,
                           k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None,
-                          page_size: int = 0) -> torch.Tensor:
+                          page_size: int = 0, cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The fused q/k/v projection x [M, K] . weight [(n_heads + 2 n_kv) head_dim, K]^T of at most 64
     rows (bfloat16) with the position encoding in its epilogue: bias, rotation of the q and k
     heads over the whole head (``inv_freq``: float64 [head_dim / 2], ``None`` = none) and the
-    write of k and v into the cache pools at ``slots``.  Returns [M, N] whose q columns are
-    filled; the k and v columns are not written."""
+    write of k and v into the cache pools at ``slots``.  ``cos_sin``: what ``rope_table`` made of
+    these positions and frequencies (the kernel then reads the cosines and sines instead of
+    computing them).  Returns [M, N] whose q columns are filled; the k and v columns are not
+    written."""
     _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
     _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
     m, k = x.shape
@@ -267,6 +269,10 @@ def gemm_mfma_skinny_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[
     _need(positions, "positions", dtype=torch.int32, shape=(m,))
     if inv_freq is not None:
         _need(inv_freq, "inv_freq", dtype=torch.float64, shape=(head_dim // 2,))
+    if cos_sin is not None:
+        if inv_freq is None:
+            raise KernelError("gemm_mfma_skinny_rope: a table of cosines and sines without frequencies")
+        _need(cos_sin, "cos_sin", dtype=torch.float32, shape=(m, head_dim // 2, 2))
     pool_slots = 0
     if k_pool is not None:
         if v_pool is None or slots is None:
@@ -279,9 +285,22 @@ def gemm_mfma_skinny_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[
         pool_slots = k_pool.shape[0] * page_size
     out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     check(load().fsie_gemm_mfma_skinny_rope(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, k,
-                                            positions.data_ptr(), _ptr(slots), _ptr(inv_freq), _ptr(k_pool),
-                                            _ptr(v_pool), n_heads, n_kv, head_dim, page_size, pool_slots, _stream()))
+                                            positions.data_ptr(), _ptr(slots), _ptr(inv_freq), _ptr(cos_sin),
+                                            _ptr(k_pool), _ptr(v_pool), n_heads, n_kv, head_dim, page_size, pool_slots,
+                                            _stream()))
     return out
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """float32 [T, half, 2]: cos and sin of positions[t] * inv_freq[i] (the angle in float64, as in
+    the kernels that rotate).  The angles of a step are the same in every layer: a step makes the
+    table once."""
+    _need(positions, "positions", dtype=torch.int32, ndim=1)
+    _need(inv_freq, "inv_freq", dtype=torch.float64, ndim=1)
+    t, half = positions.shape[0], inv_freq.shape[0]
+    table = torch.empty((t, half, 2), dtype=torch.float32, device=positions.device)
+    check(load().fsie_rope_table(positions.data_ptr(), inv_freq.data_ptr(), t, half, table.data_ptr(), _stream()))
+    return table
 
 
 def attention_tile_tokens(n_heads: int, n_kv: int) -> int:

@@ -55,11 +55,17 @@ class RotaryEncoding(PositionEncoding):
         if (x.dtype != torch.bfloat16 or not 0 < x.shape[0] <= GEMM_MFMA_SKINNY_BEST_M or x.shape[1] % 8
                 or head_dim % 16 or self.rotary_dim != head_dim):
             return None
+        # the cosines and sines of this step's positions: the same in every layer, made by the first
+        key = ("rope cos/sin", self.theta, self.rotary_dim)
+        table = ctx.memo.get(key)
+        if table is None:
+            table = ctx.memo[key] = ops.rope_table(ctx.positions, self.inv_freq)
         if store is None:
-            return ops.gemm_mfma_skinny_rope(x, weight, bias, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq)
+            return ops.gemm_mfma_skinny_rope(x, weight, bias, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq,
+                                             cos_sin=table)
         return ops.gemm_mfma_skinny_rope(x, weight, bias, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq,
                                          slots=store.slots, k_pool=store.k_pool, v_pool=store.v_pool,
-                                         page_size=store.page_size)
+                                         page_size=store.page_size, cos_sin=table)
 
 
 @register_part("position", "none")

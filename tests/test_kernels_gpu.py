@@ -257,6 +257,16 @@ def test_projection_with_rotary_epilogue(ops, m, heads, kv, hd, k, theta, use_bi
         assert (vp[s // page, :, :, s % page].reshape(-1) - v_ref[i]).abs().max() <= tol(bf, v_ref), f"v of token {i}"
     untouched = ~written.reshape(pages, 1, page, 1).expand_as(kp)
     assert kp[untouched].abs().max() == 0 and vp.transpose(2, 3)[untouched].abs().max() == 0
+    # with the cosines and sines from the step's table instead of the kernel's own: the same bits
+    table = ops.rope_table(pos.cuda(), inv.cuda())
+    ang = pos.double().unsqueeze(1) * inv.unsqueeze(0)
+    assert (table[..., 0].cpu() - torch.cos(ang).float()).abs().max() <= 5e-7
+    assert (table[..., 1].cpu() - torch.sin(ang).float()).abs().max() <= 5e-7
+    dk2, dv2 = torch.zeros_like(dk), torch.zeros_like(dv)
+    got2 = ops.gemm_mfma_skinny_rope(x.cuda(), w.cuda(), None if bias is None else bias.cuda(), pos.cuda(), heads, kv,
+                                     hd, inv.cuda(), slots=slots.cuda(), k_pool=dk2, v_pool=dv2, page_size=page,
+                                     cos_sin=table)
+    assert torch.equal(got2[:, :heads * hd], got[:, :heads * hd]) and torch.equal(dk2, dk) and torch.equal(dv2, dv)
     # the same without a cache and without rotation: q is the product plus bias
     got = ops.gemm_mfma_skinny_rope(x.cuda(), w.cuda(), None if bias is None else bias.cuda(), pos.cuda(), heads, kv,
                                     hd, None)
