@@ -5,11 +5,17 @@ kernel and its grid assume, then queues the kernel on torch's current stream.  N
 computes with torch; a missing kernel library is an error, not a reason to fall back.
 """
 
-from .functions import (bias_add, attention_merge, attention_mfma, attention_mfma_max_waves, attention_mfma_rows, attention_mfma_lds, attention_mfma_lds_ok, attention_scalar, attention_tile_tokens, dtype_code,
-                        embedding, gemm, gemm_mfma_skinny, gemm_mfma_skinny_rope, gemm_mfma_wide, gemm_mfma_wide_splits_ok, residual_add, rmsnorm, rope_kv_write, rope_table, sample, swiglu)
+from .functions import (attention_merge, attention_mfma, attention_mfma_lds, attention_mfma_lds_ok,
+                        attention_mfma_max_waves, attention_mfma_rows, attention_scalar,
+                        attention_tile_tokens, bias_add, dtype_code, embedding, gemm, gemm_mfma_skinny,
+                        gemm_mfma_skinny_rope, gemm_mfma_wide, gemm_mfma_wide_splits_ok, residual_add,
+                        rmsnorm, rope_kv_write, rope_table, sample, swiglu)
 from .library import KernelError, KernelLibraryMissing, load
 from .tuning import disable_library_tuning, enable_library_tuning, library_mm, library_tuning_enabled
 
-__all__ = ["disable_library_tuning", "enable_library_tuning", "library_mm", "library_tuning_enabled", "KernelError", "KernelLibraryMissing", "attention_merge", "attention_mfma", "attention_mfma_max_waves", "attention_mfma_rows", "attention_mfma_lds", "attention_mfma_lds_ok", "attention_scalar", "bias_add",
-           "attention_tile_tokens", "dtype_code", "embedding", "gemm", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "gemm_mfma_wide", "gemm_mfma_wide_splits_ok", "load", "residual_add",
+__all__ = ["KernelError", "KernelLibraryMissing", "attention_merge", "attention_mfma", "attention_mfma_lds",
+           "attention_mfma_lds_ok", "attention_mfma_max_waves", "attention_mfma_rows", "attention_scalar",
+           "attention_tile_tokens", "bias_add", "disable_library_tuning", "dtype_code", "embedding",
+           "enable_library_tuning", "gemm", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "gemm_mfma_wide",
+           "gemm_mfma_wide_splits_ok", "library_mm", "library_tuning_enabled", "load", "residual_add",
            "rmsnorm", "rope_kv_write", "rope_table", "sample", "swiglu"]
