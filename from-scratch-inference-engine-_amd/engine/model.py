@@ -99,8 +99,7 @@ class Model:
         device = _require_gpu(device)
         config = parse_config(read_config_json(model_dir))
         model = cls(build_model_spec(config), dtype, device)
-        path = Path(model_dir) / "model.safetensors"
-        model.weight_bytes = load_weights(path, model.spec.bindings, model.dtype, device,
+        model.weight_bytes = load_weights(Path(model_dir), model.spec.bindings, model.dtype, device,
                                           model.spec.ignore_unexpected)
         model._prepare()
         return model

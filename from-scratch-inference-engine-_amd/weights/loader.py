@@ -130,9 +130,63 @@ def fill_parts(bindings: Sequence[ParamBinding], get_tensor, compute_dtype: torc
     return total
 
 
+class CheckpointFiles:
+    """The tensors of a model folder by name: ``model.safetensors``, or, where that file does not
+    exist, the files that ``model.safetensors.index.json`` names (``weight_map``: tensor name ->
+    file name, the layout in which large checkpoints are published; the reference reads the single
+    file only, src/cuda/model.cu:774).  A tensor that the index sends to a file which does not
+    hold it, or a file that holds tensors the index does not send there, is an error."""
+
+    def __init__(self, model_dir):
+        import json
+        from pathlib import Path
+
+        root = Path(model_dir)
+        single, index = root / "model.safetensors", root / "model.safetensors.index.json"
+        self._where: Dict[str, SafetensorsFile] = {}
+        if single.is_file():
+            f = SafetensorsFile(single)
+            self._where = {n: f for n in f.names()}
+            return
+        if not index.is_file():
+            raise WeightsError(f"{root}: neither model.safetensors nor model.safetensors.index.json")
+        try:
+            weight_map = json.loads(index.read_text())["weight_map"]
+            assert isinstance(weight_map, dict) and all(isinstance(v, str) for v in weight_map.values())
+        except (ValueError, KeyError, AssertionError) as e:
+            raise WeightsError(f"{index}: not an index of safetensors files ({e!r})") from None
+        files: Dict[str, SafetensorsFile] = {}
+        for name, fname in weight_map.items():
+            if "/" in fname or "\\" in fname or fname.startswith("."):
+                raise WeightsError(f"{index}: file name '{fname}' must lie in the model folder")
+            if fname not in files:
+                if not (root / fname).is_file():
+                    raise WeightsError(f"{index}: names {fname}, which does not exist")
+                files[fname] = SafetensorsFile(root / fname)
+            if name not in files[fname].names():
+                raise WeightsError(f"{index}: sends {name} to {fname}, which does not hold it")
+            self._where[name] = files[fname]
+        for fname, f in files.items():
+            stray = sorted(n for n in f.names() if weight_map.get(n) != fname)
+            if stray:
+                raise WeightsError(f"{fname} holds tensors the index does not send there: {', '.join(stray[:8])}")
+
+    def names(self):
+        return self._where.keys()
+
+    def shape(self, name: str):
+        return self._where[name].shape(name)
+
+    def get(self, name: str) -> torch.Tensor:
+        return self._where[name].get(name)
+
+
 def load_weights(path, bindings: Sequence[ParamBinding], compute_dtype: torch.dtype, device,
                  ignore_unexpected: Sequence[str] = ()) -> int:
-    """Check ``path`` (a .safetensors file) against ``bindings`` and fill the parts."""
-    f = SafetensorsFile(path)
+    """Check ``path`` (a .safetensors file, or a model folder: see ``CheckpointFiles``) against
+    ``bindings`` and fill the parts."""
+    import os
+
+    f = CheckpointFiles(path) if os.path.isdir(path) else SafetensorsFile(path)
     check_against(bindings, {n: f.shape(n) for n in f.names()}, ignore_unexpected)
     return fill_parts(bindings, f.get, compute_dtype, device)

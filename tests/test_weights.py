@@ -104,6 +104,49 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert piece in text
 
 
+def test_a_checkpoint_in_several_files_is_read_through_its_index(tmp_path):
+    """Large checkpoints come as several safetensors files and model.safetensors.index.json; the
+    folder loads to the same parameters as the single file, and an index that does not fit its
+    files is refused."""
+    import json
+
+    from from_scratch_inference_engine_amd.weights import write_safetensors
+
+    cfg = helpers.TINY_A
+    tensors = helpers.random_tensors(cfg, 5, torch.float32)
+    single = helpers.make_model_dir(tmp_path / "single", cfg, 5, tensors=tensors)
+    sharded = tmp_path / "sharded"
+    sharded.mkdir()
+    (sharded / "config.json").write_text((single / "config.json").read_text())
+    names = sorted(tensors)
+    parts = {"model-00001-of-00002.safetensors": names[0::2], "model-00002-of-00002.safetensors": names[1::2]}
+    for fname, held in parts.items():
+        write_safetensors(sharded / fname, {n: tensors[n] for n in held})
+    index = {"metadata": {"total_size": 0}, "weight_map": {n: f for f, held in parts.items() for n in held}}
+    (sharded / "model.safetensors.index.json").write_text(json.dumps(index))
+    a, b = _spec(cfg), _spec(cfg)
+    load_weights(single, a.bindings, torch.float32, "cpu")
+    load_weights(sharded, b.bindings, torch.float32, "cpu")
+    for pa, pb in zip(a.all_parts(), b.all_parts()):
+        for attr in pa.param_decls():
+            assert torch.equal(getattr(pa, attr), getattr(pb, attr)), attr
+    # a tensor missing from the index is reported like any missing tensor
+    del index["weight_map"][names[0]]
+    (sharded / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(WeightsError, match="holds tensors the index does not send there"):
+        load_weights(sharded, _spec(cfg).bindings, torch.float32, "cpu")
+    index["weight_map"][names[0]] = "model-00002-of-00002.safetensors"
+    (sharded / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(WeightsError, match="which does not hold it"):
+        load_weights(sharded, _spec(cfg).bindings, torch.float32, "cpu")
+    index["weight_map"][names[0]] = "../elsewhere.safetensors"
+    (sharded / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(WeightsError, match="must lie in the model folder"):
+        load_weights(sharded, _spec(cfg).bindings, torch.float32, "cpu")
+    with pytest.raises(WeightsError, match="neither model.safetensors nor"):
+        load_weights(tmp_path, _spec(cfg).bindings, torch.float32, "cpu")
+
+
 def test_storage_kinds_and_fusion(tmp_path):
     """Matrices take the compute dtype, vectors stay float32 whatever the file stores, q/k/v
     are concatenated in that order, gate/up are interleaved row by row, a tied head shares the
