@@ -1,0 +1,131 @@
+"""The host side of attention: how a step is cut into work items (no GPU needed; the geometry
+comes from host functions of the kernel library).
+
+For random batches, both kernel families and with and without a window: every query sees each
+key of its range exactly once over its items, rows whose keys are split have one partial slot per
+split and one merge that names them in order, no slot is used twice, groups for the LDS kernel
+are consecutive tiles of one request, and a request is cut the same way alone and in a batch."""
+
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from from_scratch_inference_engine_amd import ops
+from from_scratch_inference_engine_amd.parts.attention import AttentionPlanner
+
+try:  # the tile sizes are host functions of the kernel library (built at first use where hipcc exists)
+    ops.load()
+except ops.KernelLibraryMissing as e:  # pragma: no cover
+    pytest.skip(f"no kernel library: {e}", allow_module_level=True)
+
+SEQ, ROW, NQ, POS, KB, KE, PARTIAL = range(7)
+
+
+class Host:
+    def __init__(self, seqs, page_size, dtype):
+        self.n_seqs = len(seqs)
+        self.past_lens = [p for p, _ in seqs]
+        self.q_lens = [n for _, n in seqs]
+        self.q_starts = [0]
+        for n in self.q_lens:
+            self.q_starts.append(self.q_starts[-1] + n)
+        self.n_tokens = self.q_starts[-1]
+        self.page_size = page_size
+        self.compute_dtype = dtype
+        self.pad = None
+
+
+def check_plan(planner, host, plan):
+    window = planner.window
+    items, merges = plan["items"], plan["merges"]
+    assert len(items) == plan["n_small"] + plan["n_large"] + plan["n_long"] and len(merges) == plan["n_merges"]
+    seen = {}       # row -> list of (key range seen, partial slot)
+    for it in items:
+        s, row0, nq = int(it[SEQ]), int(it[ROW]), int(it[NQ])
+        assert nq > 0 and host.q_starts[s] <= row0 and row0 + nq <= host.q_starts[s + 1]
+        assert int(it[POS]) == host.past_lens[s] + (row0 - host.q_starts[s])
+        for t in range(nq):
+            pos = int(it[POS]) + t
+            lo = max(int(it[KB]), pos - window + 1 if window else 0)
+            hi = min(int(it[KE]), pos + 1)
+            slot = int(it[PARTIAL]) + t if it[PARTIAL] >= 0 else -1
+            seen.setdefault(row0 + t, []).append((lo, hi, slot))
+    assert sorted(seen) == list(range(host.n_tokens))
+    merged = {int(m[0]): m for m in merges}
+    slots_used = set()
+    for s in range(host.n_seqs):
+        for row in range(host.q_starts[s], host.q_starts[s + 1]):
+            pos = host.past_lens[s] + row - host.q_starts[s]
+            first = max(0, pos - window + 1) if window else 0
+            runs = sorted((lo, hi, slot) for lo, hi, slot in seen[row] if hi > lo)
+            # the runs tile [first, pos] exactly
+            assert runs[0][0] == first and runs[-1][1] == pos + 1, (row, runs)
+            assert all(a[1] == b[0] for a, b in zip(runs, runs[1:])), (row, runs)
+            if len(seen[row]) == 1:
+                assert seen[row][0][2] == -1 and row not in merged
+            else:
+                m = merged[row]
+                assert int(m[2]) == len(seen[row])
+                want = [int(m[1]) + i * int(m[3]) for i in range(int(m[2]))]
+                # the merge names the slots in the order of the keys
+                assert [slot for _, _, slot in sorted(seen[row])] == want
+                assert not slots_used & set(want)
+                slots_used |= set(want)
+    assert not slots_used or max(slots_used) < plan["n_partial"]
+    if plan["mfma"]:
+        large = items[plan["n_small"]:]
+        covered = []
+        for first, count in plan["groups"]:
+            assert 1 <= count <= 4
+            tiles = large[first:first + count]
+            assert len({int(t[SEQ]) for t in tiles}) == 1
+            assert all(int(a[POS]) + int(a[NQ]) == int(b[POS]) for a, b in zip(tiles, tiles[1:]))
+            covered += list(range(first, first + count))
+        assert covered == list(range(len(large)))
+    else:
+        assert plan["n_groups"] == 0
+
+
+@pytest.mark.parametrize("dtype, page_size", [(torch.bfloat16, 16), (torch.float32, 16), (torch.bfloat16, 3)])
+@pytest.mark.parametrize("heads, kv, hd, window", [(28, 4, 128, None), (4, 4, 64, None), (6, 2, 32, 100), (20, 1, 256, 700),
+                                                   (16, 8, 48, None)])
+def test_plans_cover_every_key_once(dtype, page_size, heads, kv, hd, window):
+    rng = random.Random(heads * 131 + hd + (window or 0))
+    planner = AttentionPlanner(heads, kv, hd, window)
+    assert planner.uses_mfma(dtype, page_size) == (dtype == torch.bfloat16 and page_size % 4 == 0 and hd % 16 == 0)
+    for _ in range(25):
+        seqs = [(rng.choice([0, 0, 1, 15, 16, 255, 600, 1023, 1024, 2500, 5000]),
+                 rng.choice([1, 1, 1, 2, 3, 5, 16, 17, 64, 130, 700])) for _ in range(rng.randint(1, 6))]
+        host = Host(seqs, page_size, dtype)
+        plan = planner.plan(host)
+        check_plan(planner, host, plan)
+        # a request is cut the same way alone as in the batch
+        for s, (p, n) in enumerate(seqs):
+            alone = planner.plan(Host([(p, n)], page_size, dtype))
+            mine = [it for it in plan["items"] if it[SEQ] == s]
+            theirs = list(alone["items"])
+            assert len(mine) == len(theirs)
+            key = lambda it: (int(it[ROW]), int(it[KB]))
+            for a, b in zip(sorted(mine, key=key), sorted(theirs, key=key)):
+                assert int(a[ROW]) - host.q_starts[s] == int(b[ROW])
+                assert [int(a[i]) for i in (NQ, POS, KB, KE)] == [int(b[i]) for i in (NQ, POS, KB, KE)]
+                assert (a[PARTIAL] >= 0) == (b[PARTIAL] >= 0)
+
+
+def test_graph_bucket_pads_plans_of_decode_steps():
+    planner = AttentionPlanner(28, 4, 128, None)
+    for lens in ([640] * 8, [5, 900, 1500, 3000], [2047, 2048, 2049]):
+        host = Host([(p, 1) for p in lens], 16, torch.bfloat16)
+        bucket = planner.graph_bucket(host)
+        assert bucket is not None and bucket[0] % len(lens) == 0
+        host.pad = {planner.key: bucket}
+        plan = planner.plan(host)
+        assert plan["n_small"] == bucket[0] and plan["n_large"] == 0 and plan["waves"] == bucket[1]
+        real = [it for it in plan["items"] if it[NQ] > 0]
+        assert sum(int(it[KE]) - int(it[KB]) for it in real) == sum(p + 1 for p in lens)
+        if bucket[0] > len(lens):
+            assert plan["n_merges"] == len(lens)  # every row gets a merge entry, empty where none is needed
+    # a step with a portion is no decode step
+    assert planner.graph_bucket(Host([(10, 1), (0, 40)], 16, torch.bfloat16)) is None
