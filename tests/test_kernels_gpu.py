@@ -224,7 +224,9 @@ def test_rmsnorm_adds_partial_sums_at_odd_sizes(ops):
 
 @pytest.mark.parametrize("m, heads, kv, hd, k, theta, use_bias", [
     (1, 14, 2, 64, 896, 1e6, True), (9, 3, 3, 48, 72, 1e4, True), (16, 5, 1, 256, 320, 5e5, False),
-    (7, 28, 4, 128, 3584, 1e6, True), (33, 2, 1, 16, 64, 1e4, True)])
+    (7, 28, 4, 128, 3584, 1e6, True), (33, 2, 1, 16, 64, 1e4, True),
+    # on 256 compute units these deal 10 and 14 rotary pairs a workgroup; with a head size of 160 a block's pairs span two heads
+    (8, 24, 4, 160, 256, 1e4, True), (16, 40, 8, 128, 128, 1e6, False)])
 def test_projection_with_rotary_epilogue(ops, m, heads, kv, hd, k, theta, use_bias):
     """q/k/v projection, bias, rotation and cache write in one kernel, against the plain formulas
     on the float32 product (one rounding to bfloat16, after the rotation)."""
