@@ -53,6 +53,31 @@ def test_greedy_generation_matches_plain_float32(llms, model_dirs, name, lengths
     assert llm.engine.free_blocks() == 64
 
 
+def test_llm_from_a_configuration_alone(tmp_path):
+    """``LLM.from_config`` makes the weights on the device from a seed, without a folder: what it
+    generates is what the folder written by ``write_random_model`` for that seed generates
+    (float32 weights in the file, so that both hold the same values)."""
+    from from_scratch_inference_engine_amd import LLM, GenerationConfig, load_config
+    from from_scratch_inference_engine_amd.models import parse_config
+    from from_scratch_inference_engine_amd.weights import write_random_model
+
+    raw = dict(helpers.TINY["A"][0])
+    d = write_random_model(parse_config(raw), 21, tmp_path / "m", torch.float32)
+    prompts = [helpers.token_ids(raw["vocab_size"], n, 70 + n) for n in (3, 9, 20)]
+    cfg = GenerationConfig(max_tokens=12, temperature=0.0)
+    want = [plain_greedy(d, p, 12) for p in prompts]
+    for dtype in ("float32", "bfloat16"):
+        direct = LLM.from_config(raw, 21, dtype=dtype, block_size=4, num_blocks=64)
+        folder = LLM(d, dtype=dtype, block_size=4, num_blocks=64, eos_id=-1)
+        got = direct.generate_ids_batch(prompts, cfg)
+        assert got == folder.generate_ids_batch(prompts, cfg)
+        if dtype == "float32":
+            assert got == want
+    with pytest.raises(RuntimeError, match="no tokenizer"):
+        direct.generate("text")
+    assert load_config(d).to_dict()["vocab_size"] == raw["vocab_size"]
+
+
 def test_eos_from_the_folder_stops_generation(llms, model_dirs):
     from from_scratch_inference_engine_amd import GenerationConfig
 
