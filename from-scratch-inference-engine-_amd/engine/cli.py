@@ -17,6 +17,9 @@ from time import perf_counter
 def _common(p: argparse.ArgumentParser) -> None:
     p.add_argument("--model-dir", default=os.environ.get("ENGINE_MODEL_DIR"),
                    help="folder with config.json and model.safetensors (default: $ENGINE_MODEL_DIR)")
+    p.add_argument("--config", default=None, help="a config.json, with --random-weights: a model without a folder")
+    p.add_argument("--random-weights", type=int, default=None, metavar="SEED",
+                   help="with --config: random weights made on the device from this seed")
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     p.add_argument("--block-size", type=int, default=16)
     p.add_argument("--num-blocks", type=int, default=2048)
@@ -35,8 +38,20 @@ def _common(p: argparse.ArgumentParser) -> None:
 def _llm(args):
     from .llm import LLM
 
+    if args.config is not None or args.random_weights is not None:
+        if args.config is None or args.random_weights is None:
+            raise SystemExit("--config FILE and --random-weights SEED go together")
+        if args.tune_gemms:
+            from ..ops import enable_library_tuning
+
+            enable_library_tuning()
+        with open(args.config) as f:
+            raw = json.load(f)
+        return LLM.from_config(raw, args.random_weights, block_size=args.block_size, num_blocks=args.num_blocks,
+                               seed=args.seed, max_batch=args.max_batch, dtype=args.dtype,
+                               max_tokens_per_step=args.max_tokens_per_step)
     if not args.model_dir:
-        raise SystemExit("--model-dir (or $ENGINE_MODEL_DIR) is required")
+        raise SystemExit("--model-dir (or $ENGINE_MODEL_DIR), or --config with --random-weights, is required")
     return LLM(args.model_dir, block_size=args.block_size, num_blocks=args.num_blocks, seed=args.seed,
                max_batch=args.max_batch, dtype=args.dtype, max_tokens_per_step=args.max_tokens_per_step,
                tune_gemms=args.tune_gemms)

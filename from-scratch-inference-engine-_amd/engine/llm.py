@@ -70,15 +70,15 @@ class LLM:
     def from_config(cls, config, weight_seed: int = 0, *, block_size: int = 16, num_blocks: int = 2048, seed: int = 0,
                     max_batch: int = 256, eos_id: int = -1, dtype: str = "bfloat16", device: str = "cuda:0",
                     max_tokens_per_step: int = 2048, prefill_chunk: Optional[int] = None) -> "LLM":
-        """An engine over random weights made on the device from ``config`` (the dictionary of a
-        config.json, or a typed configuration) and ``weight_seed``: no folder, no tokenizer, token
-        ids in and out.  The weights are those that ``write_random_model`` writes for the same
-        seed."""
+        """An engine over random weights made from ``config`` (the dictionary of a config.json, or a
+        typed configuration) and ``weight_seed``: no folder, no tokenizer, token ids in and out.
+        The weights are those that ``write_random_model`` writes for the same seed (as float32):
+        they are drawn on the host, tensor by tensor, and sent to the device."""
         from ..models import parse_config
 
         typed = parse_config(config) if isinstance(config, dict) else config
         llm = cls.__new__(cls)
-        llm.model = Model.from_random(typed, weight_seed, dtype=dtype, device=device)
+        llm.model = Model.from_random(typed, weight_seed, dtype=dtype, device=device, as_written=True)
         llm.engine = Engine(llm.model, block_size, num_blocks, seed, max_batch,
                             max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk)
         llm.eos_id = eos_id

@@ -61,7 +61,7 @@ def test_llm_from_a_configuration_alone(tmp_path):
     from from_scratch_inference_engine_amd.models import parse_config
     from from_scratch_inference_engine_amd.weights import write_random_model
 
-    raw = dict(helpers.TINY["A"][0])
+    raw = dict(helpers.TINY["B"][0])  # (an untied head: what it generates depends on every weight)
     d = write_random_model(parse_config(raw), 21, tmp_path / "m", torch.float32)
     prompts = [helpers.token_ids(raw["vocab_size"], n, 70 + n) for n in (3, 9, 20)]
     cfg = GenerationConfig(max_tokens=12, temperature=0.0)
@@ -190,6 +190,27 @@ def test_command_line_generate(model_dirs):
     assert proc.returncode == 0, proc.stderr[-3000:]
     out = json.loads(proc.stdout.strip().splitlines()[-1])
     assert out["outputs"] == [plain_greedy(model_dirs["A"], prompt, 8)]
+
+
+def test_command_line_generate_from_a_configuration(tmp_path):
+    """--config FILE --random-weights SEED: no model folder; the same tokens as the folder that
+    random-model writes for that seed."""
+    from from_scratch_inference_engine_amd.models import parse_config
+    from from_scratch_inference_engine_amd.weights import write_random_model
+
+    raw = dict(helpers.TINY["B"][0])
+    (tmp_path / "cfg.json").write_text(json.dumps(raw))
+    d = write_random_model(parse_config(raw), 33, tmp_path / "m", torch.float32)
+    prompt = helpers.token_ids(raw["vocab_size"], 7, 19)
+    cmd = [sys.executable, "-m", "from_scratch_inference_engine_amd", "generate", "--config", str(tmp_path / "cfg.json"),
+           "--random-weights", "33", "--dtype", "float32", "--prompt-ids", " ".join(map(str, prompt)), "--max-tokens", "6",
+           "--block-size", "8", "--num-blocks", "16", "--json"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300, cwd=str(helpers.ROOT))
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    out = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert out["outputs"] == [plain_greedy(d, prompt, 6)]
+    bad = subprocess.run(cmd[:5] + cmd[7:], capture_output=True, text=True, timeout=300, cwd=str(helpers.ROOT))
+    assert bad.returncode != 0 and "go together" in bad.stderr
 
 
 def test_graft_entry_smoke():
