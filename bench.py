@@ -32,6 +32,14 @@ QWEN25_7B = {
 }
 
 
+# the other shapes that BASELINE.json lists (configs[3] and [4]); the default run is configs[2]
+QWEN25_14B = dict(QWEN25_7B, hidden_size=5120, num_hidden_layers=48, num_attention_heads=40, num_key_value_heads=8,
+                  intermediate_size=13824, rms_norm_eps=1e-5, max_position_embeddings=8192)
+QWEN25_32B = dict(QWEN25_14B, num_hidden_layers=64, intermediate_size=27648, max_position_embeddings=16384)
+SHAPES = {"7b": ("Qwen2.5-7B shape", QWEN25_7B), "14b": ("Qwen2.5-14B shape", QWEN25_14B),
+          "32b": ("Qwen2.5-32B shape", QWEN25_32B)}
+
+
 def gemm_params_per_layer(c) -> int:
     q, kv = c.num_attention_heads * c.head_dim, c.num_key_value_heads * c.head_dim
     return c.hidden_size * (q + 2 * kv) + q * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
@@ -60,6 +68,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (named in config)")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="7b", help="layer sizes (default: BASELINE.json's configs[2])")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
@@ -79,7 +88,8 @@ def main() -> int:
     if not args.no_tune and args.dtype == "bf16":
         enable_library_tuning()  # the first prefill times the library's kernels for its shapes
 
-    raw = dict(QWEN25_7B)
+    shape_name, shape = SHAPES[args.shape]
+    raw = dict(shape)
     full_layers = raw["num_hidden_layers"]
     layers = args.layers or full_layers
     raw["num_hidden_layers"] = layers
@@ -160,12 +170,12 @@ def main() -> int:
             print(f"[bench] decode batch {b}: {d / k * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
 
     line = {
-        "metric": "decode tok/s @ batch 8, Qwen2.5-7B shape (with prefill tok/s @ 2,048 tokens, decode @ batch 1/64)",
+        "metric": f"decode tok/s @ batch {args.batch}, {shape_name} (with prefill tok/s @ 2,048 tokens, decode @ batch 1/64)",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random weights N(0,0.02), uniform random token ids",
         "config": {
-            "model": "Qwen2.5-7B shape", "layers": layers, "layers_of_config": full_layers,
+            "model": shape_name, "layers": layers, "layers_of_config": full_layers,
             "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "global_batch": args.batch, "seq_len": context, "prompt_len": args.prompt_len,

@@ -118,6 +118,9 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 // that fsie_last_error() hands out (per host thread).
 void fsie_set_error(const char* fmt, ...);
 
+// compute units of the current device (0 if it cannot be asked); asked once per device
+int fsie_compute_units();
+
 #define FSIE_REQUIRE(cond, ...)          \
     do {                                 \
         if (!(cond)) {                   \

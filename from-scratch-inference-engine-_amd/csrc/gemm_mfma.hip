@@ -2,23 +2,6 @@
 // the choice of the launch shape.
 #include "gemm_mfma_impl.h"
 
-namespace {
-
-// compute units of the current device (0 if it cannot be asked), asked once per device
-int compute_units() {
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
-
-}  // namespace
-
 // bfloat16 only.  M <= 64, K a multiple of 8, x and w 16-byte aligned.
 // waves (K split inside a workgroup) and blocks (16-row blocks of W per workgroup): 0 = choose.
 // epilogue: 0 = y = d (+ bias); 1 = SiLU*up over interleaved gate/up rows (N even, no bias, y is [M, N/2]).
@@ -59,14 +42,15 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
         blocks = (M > 2 && static_cast<int64_t>(N) * splits >= 14336) ? 2 : 1;
     }
     if (waves == 0) {
-        // split K inside the workgroup until about nine hundred waves stream W (N = 3584,
-        // K = 18944 in four slices, 8 rows: 27.9 us with 896 waves, 32.7 with 1792; with 64 rows
-        // 1792 are better, 6.19 against 6.42 ms for a whole decode step of a 7B model); one or two
+        // split K inside the workgroup until some eight hundred waves stream W (N = 3584,
+        // K = 18944 in four slices, 8 rows: 27.9 us with 896 waves, 32.7 with 1792; N = 27648,
+        // K = 5120, 8 rows: 58.4 us with 864 waves, 66.5 with 1728; with 64 rows 1792 are
+        // better, 6.19 against 6.42 ms for a whole decode step of a 7B model); one or two
         // rows of X gain from more loads in flight even at large N (four waves where N alone gives
         // two thousand workgroups: 177 against 181 us at N = 152064; two from 896 workgroups on)
         const int groups = (N + 16 * blocks - 1) / (16 * blocks) * splits;
         waves = 1;
-        const int enough = M <= 16 ? 896 : 1024;  // more rows of X: more waves to share the products
+        const int enough = M <= 16 ? 832 : 1024;  // more rows of X: more waves to share the products
         while (waves < 16 && groups * waves < enough) waves *= 2;
         const int few_rows_waves = groups >= 2048 ? 4 : (groups >= 896 ? 2 : 8);
         if (M <= 2 && waves < few_rows_waves) waves = few_rows_waves;
@@ -113,7 +97,7 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     // units: 288 workgroups), the pairs are dealt evenly instead, 9 to 16 a workgroup, in two blocks
     // of which the second is partly filled.
     const int total_pairs = N / 2;
-    const int units = compute_units();
+    const int units = fsie_compute_units();
     int pairs_per_wg = 8;
     if (mt == 1 && M > 4 && units > 0 && total_pairs > 8 * units && total_pairs <= 16 * units) {  // (no gain at 1 row)
         pairs_per_wg = (total_pairs + units - 1) / units;

@@ -21,6 +21,18 @@ extern "C" const char* fsie_last_error(void) { return g_error; }
 
 extern "C" int fsie_version(void) { return 1; }
 
+int fsie_compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 extern "C" int fsie_device_info(char* arch_out, int arch_len, int* n_compute_units) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
