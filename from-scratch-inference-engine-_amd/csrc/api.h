@@ -34,6 +34,8 @@ const char* fsie_last_error(void);
 int fsie_version(void);
 // Name of the architecture the device code was built for and of the device present.
 int fsie_device_info(char* arch_out, int arch_len, int* n_compute_units);
+// Compute units of the current device; 0 if there is no device to ask.
+int fsie_device_compute_units(void);
 
 int fsie_embedding(const void* table, int dtype, const int32_t* ids, float* out, int n_tokens, int hidden,
                    int vocab, hipStream_t stream);

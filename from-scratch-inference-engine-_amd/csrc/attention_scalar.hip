@@ -191,33 +191,79 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
 
 // Combine the partial records of one query token in the fixed order of its splits.
 // merge item: {out_row, first_slot, n_splits, slot_stride}
-template <typename T>
-__global__ void attention_merge_kernel(const float* __restrict__ partials, const int32_t* __restrict__ merges,
-                                       T* __restrict__ out, int n_heads, int hd) {
+// One wave per (token, head).  The maxima and denominators of up to 64 splits are read by one
+// lane each, and the sums of a dimension are loaded several splits ahead of their use: a loop
+// that waits for each record in turn costs a memory latency per split (28 splits took longer
+// than the attention itself).
+template <typename T, int DIMS>
+__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ partials,
+                                                             const int32_t* __restrict__ merges, T* __restrict__ out,
+                                                             int n_heads, int hd) {
     const int32_t* mi = merges + static_cast<int64_t>(blockIdx.x) * FSIE_ATTN_MERGE_INTS;
     const int out_row = mi[0], first = mi[1], n_splits = mi[2], stride = mi[3];
     if (n_splits <= 0) return;
     const int hq = blockIdx.y;
+    const int lane = threadIdx.x;
     const int64_t rec_size = hd + 2;
+    const float* rec0 = partials + (static_cast<int64_t>(first) * n_heads + hq) * rec_size;
+    const int64_t rec_step = static_cast<int64_t>(stride) * n_heads * rec_size;
     float m = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) {
-        const float* rec = partials + (static_cast<int64_t>(first + s * stride) * n_heads + hq) * rec_size;
-        m = fmaxf(m, rec[hd]);
+    for (int base = 0; base < n_splits; base += 64) {
+        const int s = base + lane;
+        m = fmaxf(m, s < n_splits ? rec0[s * rec_step + hd] : -INFINITY);
     }
-    float denom = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float* rec = partials + (static_cast<int64_t>(first + s * stride) * n_heads + hq) * rec_size;
-        if (rec[hd] != -INFINITY) denom += rec[hd + 1] * expf(rec[hd] - m);
+    m = wave_max(m);
+    float denom = 0.f;  // summed in the order of the splits, as the accumulators are
+    float a[DIMS];
+#pragma unroll
+    for (int i = 0; i < DIMS; ++i) a[i] = 0.f;
+    for (int base = 0; base < n_splits; base += 64) {
+        const int s = base + lane;
+        float w = 0.f, l = 0.f;
+        if (s < n_splits) {
+            const float ms = rec0[s * rec_step + hd];
+            l = rec0[s * rec_step + hd + 1];
+            w = ms == -INFINITY ? 0.f : expf(ms - m);
+        }
+        const int here = min(64, n_splits - base);
+        const float* rec = rec0 + base * rec_step;
+        constexpr int AHEAD = 8;
+        for (int j0 = 0; j0 < here; j0 += AHEAD) {
+            float v[AHEAD][DIMS];
+#pragma unroll
+            for (int j = 0; j < AHEAD; ++j) {  // a split past the end reads the last one again, with weight 0
+                const float* r = rec + min(j0 + j, here - 1) * rec_step;
+#pragma unroll
+                for (int i = 0; i < DIMS; ++i) v[j][i] = r[min(lane + 64 * i, hd - 1)];
+            }
+#pragma unroll
+            for (int j = 0; j < AHEAD; ++j) {
+                const int src = min(j0 + j, 63);
+                const float wj = j0 + j < here ? __shfl(w, src) : 0.f;
+                const float lj = __shfl(l, src);
+                if (wj != 0.f) {  // the same for the whole wave
+                    denom += lj * wj;
+#pragma unroll
+                    for (int i = 0; i < DIMS; ++i) a[i] += v[j][i] * wj;
+                }
+            }
+        }
     }
     const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-        float a = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float* rec = partials + (static_cast<int64_t>(first + s * stride) * n_heads + hq) * rec_size;
-            if (rec[hd] != -INFINITY) a += rec[d] * expf(rec[hd] - m);
-        }
-        out[(static_cast<int64_t>(out_row) * n_heads + hq) * hd + d] = from_float<T>(a * inv);
+#pragma unroll
+    for (int i = 0; i < DIMS; ++i) {
+        const int d = lane + 64 * i;
+        if (d < hd) out[(static_cast<int64_t>(out_row) * n_heads + hq) * hd + d] = from_float<T>(a[i] * inv);
     }
+}
+
+template <typename T>
+void launch_merge(const float* partials, const int32_t* merges, int n_merges, T* out, int n_heads, int hd,
+                  hipStream_t stream) {
+    const dim3 grid(n_merges, n_heads);
+    if (hd <= 64) attention_merge_kernel<T, 1><<<grid, 64, 0, stream>>>(partials, merges, out, n_heads, hd);
+    else if (hd <= 128) attention_merge_kernel<T, 2><<<grid, 64, 0, stream>>>(partials, merges, out, n_heads, hd);
+    else attention_merge_kernel<T, 4><<<grid, 64, 0, stream>>>(partials, merges, out, n_heads, hd);
 }
 
 }  // namespace
@@ -257,14 +303,11 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
 extern "C" int fsie_attention_merge(const float* partials, const int32_t* merges, int n_merges, void* out,
                                     int n_heads, int head_dim, int dtype, hipStream_t stream) {
     FSIE_REQUIRE(n_merges >= 0 && n_heads > 0 && head_dim > 0, "attention_merge: bad sizes");
+    FSIE_REQUIRE(head_dim <= 256, "attention_merge: head_dim %d is larger than 256", head_dim);
     FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "attention_merge: unknown dtype %d", dtype);
     if (n_merges == 0) return 0;
-    const dim3 grid(n_merges, n_heads);
-    if (dtype == FSIE_F32) {
-        attention_merge_kernel<float><<<grid, 64, 0, stream>>>(partials, merges, static_cast<float*>(out), n_heads, head_dim);
-    } else {
-        attention_merge_kernel<bf16_t><<<grid, 64, 0, stream>>>(partials, merges, static_cast<bf16_t*>(out), n_heads, head_dim);
-    }
+    if (dtype == FSIE_F32) launch_merge(partials, merges, n_merges, static_cast<float*>(out), n_heads, head_dim, stream);
+    else launch_merge(partials, merges, n_merges, static_cast<bf16_t*>(out), n_heads, head_dim, stream);
     FSIE_CHECK_LAUNCH("attention_merge");
     return 0;
 }

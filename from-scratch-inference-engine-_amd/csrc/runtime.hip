@@ -33,6 +33,8 @@ int fsie_compute_units() {
     return cached[dev];
 }
 
+extern "C" int fsie_device_compute_units(void) { return fsie_compute_units(); }
+
 extern "C" int fsie_device_info(char* arch_out, int arch_len, int* n_compute_units) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);

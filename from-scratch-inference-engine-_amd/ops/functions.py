@@ -347,6 +347,11 @@ def attention_mfma_rows(head_dim: int, large: bool) -> int:
     return 16 * load().fsie_attention_mfma_tiles(head_dim, int(large))
 
 
+def compute_units() -> int:
+    """Compute units of the current device; 0 where there is none to ask."""
+    return load().fsie_device_compute_units()
+
+
 def attention_mfma_max_waves(head_dim: int) -> int:
     return load().fsie_attention_mfma_max_waves(head_dim)
 

@@ -25,6 +25,7 @@ _P = c_void_p
 _SIGNATURES = {
     "fsie_version": ([], c_int),
     "fsie_device_info": ([c_char_p, c_int, ctypes.POINTER(c_int)], c_int),
+    "fsie_device_compute_units": ([], c_int),
     "fsie_embedding": ([_P, c_int, _P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_rmsnorm": ([_P, _P, _P, _P, _P, c_int, c_int, c_float, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_swiglu": ([_P, _P, c_int, c_int, c_int, _P], c_int),

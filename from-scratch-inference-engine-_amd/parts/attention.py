@@ -22,13 +22,15 @@ class AttentionPlanner:
 
     A request's portion of n tokens at past length p becomes tiles of query tokens; a tile reads
     the keys from the start of its window to its last token.  A portion of at most
-    ``small_tokens`` tokens is one *small* item.  For the float32-arithmetic kernel a small item
-    that reads more than ``split_keys`` keys (decoding against a long context) is split over the
-    keys into several items and merged afterwards in the order of the splits (256 keys an item
-    for the float32-arithmetic kernel; 1,024 for the matrix-core kernel, which gives every 128 of
-    them to a wave of the item's workgroup and combines those inside).  Longer portions are cut into *large*
-    tiles of ``large_tokens``.  Whether and how a portion is cut depends on the portion alone,
-    never on what else is in the batch.  The item table lists the small items first.
+    ``small_tokens`` tokens is one *small* item.  A small item that reads more than ``split_keys``
+    keys (decoding against a long context) is split over the keys into several items and merged
+    afterwards in the order of the splits: 256 keys an item for the float32-arithmetic kernel; for
+    the matrix-core kernel, which gives every 128 keys to a wave of the item's workgroup and
+    combines those inside, 1,024 keys, or 512 or 256 while the step has fewer workgroups than the
+    device has compute units (every wave still sums the same 128 keys; only where their sums
+    meet changes).  Longer portions are cut into *large* tiles of ``large_tokens``; how they are
+    cut depends on the portion alone, never on what else is in the batch.  The item table lists
+    the small items first.
 
     Two geometries exist: the matrix-core kernel (bfloat16, head size a multiple of 16, page size
     a multiple of 4) and the float32-arithmetic kernel for everything else; which one a step
@@ -38,6 +40,8 @@ class AttentionPlanner:
     # 2,048-token prefill at 28/4 heads of 128 took 235 us per layer with 512 against 176 us
     # without (idle waves in the four-wave workgroups cost more than the balance gains).
     long_keys: Optional[int] = None
+    # Compute units to fill with the workgroups of small items; None: those of the device.
+    compute_units: Optional[int] = None
 
     def __init__(self, n_heads: int, n_kv: int, head_dim: int, window: Optional[int]):
         self.n_heads, self.n_kv, self.head_dim, self.window = n_heads, n_kv, head_dim, window
@@ -52,8 +56,7 @@ class AttentionPlanner:
                 small = max(1, ops.attention_mfma_rows(self.head_dim, False) // min(group, 16))
                 rows = ops.attention_mfma_rows(self.head_dim, True)
                 large = max(1, rows // min(group, rows))
-                # one compute unit draws only some 50 GB/s from memory: beyond 1,024 keys (eight
-                # waves of 128) a query's keys go to several workgroups
+                # at most 1,024 keys (eight waves of 128) an item
                 self._geometry[mfma] = (small, large, 128 * min(8, ops.attention_mfma_max_waves(self.head_dim)))
             else:
                 t = ops.attention_tile_tokens(self.n_heads, self.n_kv)
@@ -73,11 +76,41 @@ class AttentionPlanner:
             w *= 2
         return min(w, max_waves)
 
+    def _small_keys(self, host, small_tokens):
+        """Keys that each small portion of the step reads."""
+        keys = []
+        for s in range(host.n_seqs):
+            n, p = host.q_lens[s], host.past_lens[s]
+            if n <= small_tokens:
+                keys.append(p + n - (max(0, p - self.window + 1) if self.window else 0))
+        return keys
+
+    def split_keys(self, host, mfma: bool) -> int:
+        """Keys per small item in this step.  A workgroup draws only some 50 GB/s from memory, so a
+        step with few requests is faster with more, shorter items, although they cost a merge
+        (MI355X, 28/4 heads of 128, per layer: 8 requests of 640 keys 10.7 us with 256 keys an
+        item against 12.2 with 1,024; one request of 3,550 keys 11.3 against 18.2; 64 requests of
+        640 keys 24.8 against 18.3, which is why a full device keeps the long items)."""
+        small_tokens, _, longest = self.geometry(mfma)
+        if not mfma:
+            return longest
+        units = self.compute_units if self.compute_units is not None else ops.compute_units()
+        keys = self._small_keys(host, small_tokens)
+        group = self.n_heads // self.n_kv
+        rows = ops.attention_mfma_rows(self.head_dim, False)
+        per_item = self.n_kv * -(-group // min(group, rows))  # workgroups of one item
+        split = longest
+        while split > 256 and sum(-(-k // split) for k in keys) * per_item < units:
+            split //= 2
+        return split
+
     def graph_bucket(self, host):
-        """What a captured graph of this step's shape must fix: the number of (small) work items
-        and the waves per item; None if the step has portions that do not fit small items."""
+        """What a captured graph of this step's shape must fix: the number of (small) work items,
+        the waves per item and the keys per item; None if the step has portions that do not fit
+        small items."""
         mfma = self.uses_mfma(host.compute_dtype, host.page_size)
-        small_tokens, _, split_keys = self.geometry(mfma)
+        small_tokens = self.geometry(mfma)[0]
+        split_keys = self.split_keys(host, mfma)
         n, longest = 0, 1
         for s in range(host.n_seqs):
             if host.q_lens[s] > small_tokens:
@@ -89,13 +122,15 @@ class AttentionPlanner:
         if mfma:
             # items: a multiple of the number of requests (the captured graph pads with empty ones)
             return (-(-n // host.n_seqs) * host.n_seqs,
-                    self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)))
+                    self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)), split_keys)
         step = 4 * host.n_seqs
-        return (-(-n // step) * step, 1)
+        return (-(-n // step) * step, 1, split_keys)
 
     def plan(self, host) -> Dict[str, object]:
         mfma = self.uses_mfma(host.compute_dtype, host.page_size)
-        small_tokens, large_tokens, split_keys = self.geometry(mfma)
+        small_tokens, large_tokens, _ = self.geometry(mfma)
+        padded = getattr(host, "pad", None) is not None
+        split_keys = host.pad[self.key][2] if padded else self.split_keys(host, mfma)
         small, large, merges = [], [], []
         n_partial = 0
         for s in range(host.n_seqs):
@@ -122,9 +157,9 @@ class AttentionPlanner:
         waves = 1
         if mfma and small:
             waves = self._waves_for(max(it[5] - it[4] for it in small), ops.attention_mfma_max_waves(self.head_dim))
-        if getattr(host, "pad", None) is not None:
+        if padded:
             # a captured graph launches fixed grids: pad with items and merges that do nothing
-            n_items, waves = host.pad[self.key]
+            n_items, waves, _ = host.pad[self.key]
             if large or len(small) > n_items:
                 raise RuntimeError("attention plan does not fit the captured graph")
             small += [(0, 0, 0, 0, 0, 0, -1, 0)] * (n_items - len(small))

@@ -94,6 +94,7 @@ def check_plan(planner, host, plan):
 def test_plans_cover_every_key_once(dtype, page_size, heads, kv, hd, window):
     rng = random.Random(heads * 131 + hd + (window or 0))
     planner = AttentionPlanner(heads, kv, hd, window)
+    planner.compute_units = rng.choice([0, 0, 64, 256])
     assert planner.uses_mfma(dtype, page_size) == (dtype == torch.bfloat16 and page_size % 4 == 0 and hd % 16 == 0)
     for _ in range(25):
         seqs = [(rng.choice([0, 0, 1, 15, 16, 255, 600, 1023, 1024, 2500, 5000]),
@@ -101,8 +102,12 @@ def test_plans_cover_every_key_once(dtype, page_size, heads, kv, hd, window):
         host = Host(seqs, page_size, dtype)
         plan = planner.plan(host)
         check_plan(planner, host, plan)
-        # a request is cut the same way alone as in the batch
+        # with no compute units to fill, a request is cut the same way alone as in the batch;
+        # portions longer than a small item always are
+        small_tokens = planner.geometry(plan["mfma"])[0]
         for s, (p, n) in enumerate(seqs):
+            if planner.compute_units and n <= small_tokens:
+                continue
             alone = planner.plan(Host([(p, n)], page_size, dtype))
             mine = [it for it in plan["items"] if it[SEQ] == s]
             theirs = list(alone["items"])
@@ -114,8 +119,24 @@ def test_plans_cover_every_key_once(dtype, page_size, heads, kv, hd, window):
                 assert (a[PARTIAL] >= 0) == (b[PARTIAL] >= 0)
 
 
+def test_decode_items_shorten_while_compute_units_are_idle():
+    planner = AttentionPlanner(28, 4, 128, None)
+    planner.compute_units = 256
+    for n_requests, keys, split in ((8, 640, 256), (1, 3550, 256), (64, 640, 1024), (8, 16000, 1024), (20, 3000, 512)):
+        host = Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16)
+        assert planner.split_keys(host, True) == split
+        plan = planner.plan(host)
+        check_plan(planner, host, plan)
+        assert plan["n_small"] == n_requests * -(-keys // split)
+        assert plan["waves"] == {256: 2, 512: 4, 1024: 8}[split]  # one wave per 128 keys
+        assert plan["n_merges"] == (n_requests if keys > split else 0)
+    # the float32-arithmetic kernel keeps its 256 keys an item
+    assert planner.split_keys(Host([(5000, 1)], 16, torch.float32), False) == 256
+
+
 def test_graph_bucket_pads_plans_of_decode_steps():
     planner = AttentionPlanner(28, 4, 128, None)
+    planner.compute_units = 256
     for lens in ([640] * 8, [5, 900, 1500, 3000], [2047, 2048, 2049]):
         host = Host([(p, 1) for p in lens], 16, torch.bfloat16)
         bucket = planner.graph_bucket(host)
@@ -123,6 +144,7 @@ def test_graph_bucket_pads_plans_of_decode_steps():
         host.pad = {planner.key: bucket}
         plan = planner.plan(host)
         assert plan["n_small"] == bucket[0] and plan["n_large"] == 0 and plan["waves"] == bucket[1]
+        assert bucket[2] == planner.split_keys(host, True)
         real = [it for it in plan["items"] if it[NQ] > 0]
         assert sum(int(it[KE]) - int(it[KB]) for it in real) == sum(p + 1 for p in lens)
         if bucket[0] > len(lens):

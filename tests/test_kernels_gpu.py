@@ -463,6 +463,37 @@ def test_attention_finds_one_far_key_and_respects_edges(ops, dtype, scalar):
             row += n
 
 
+@pytest.mark.parametrize("heads, hd, dtype", [(3, 32, torch.float32), (5, 80, torch.bfloat16), (28, 128, torch.bfloat16),
+                                             (2, 256, torch.float32)])
+def test_attention_merge_alone(ops, heads, hd, dtype):
+    """Records of 1 to 130 splits (more than the 64 that one pass of the wave reads), some of them
+    empty (maximum -inf), one token's records a stride apart, against the sums written out."""
+    g = torch.Generator().manual_seed(hd)
+    splits = [1, 2, 3, 9, 64, 65, 130]
+    stride = 2  # two tokens of a portion lie side by side in every split
+    slots = sum(n * stride for n in splits)
+    rec = torch.randn(slots, heads, hd + 2, generator=g)
+    rec[:, :, hd] = 3.0 * torch.randn(slots, heads, generator=g)       # maxima, natural units
+    rec[:, :, hd + 1] = torch.rand(slots, heads, generator=g) + 0.1    # denominators
+    merges, want, first = [], [], 0
+    for row, n in enumerate(splits):
+        for t in range(stride):
+            idx = [first + t + i * stride for i in range(n)]
+            if n >= 3:  # an empty split in the middle: a window that has passed it
+                rec[idx[1], :, hd] = float("-inf")
+                rec[idx[1], :, hd + 1] = 0.0
+            r = rec[idx].double()
+            w = torch.exp(r[:, :, hd] - r[:, :, hd].max(0).values)
+            want.append(((r[:, :, :hd] * w[:, :, None]).sum(0) / (r[:, :, hd + 1] * w).sum(0)[:, None]).reshape(-1))
+            merges.append((row * stride + t, first + t, n, stride))
+        first += n * stride
+    out = torch.zeros(len(merges), heads * hd, dtype=dtype).cuda()
+    ops.attention_merge(rec.reshape(-1).cuda(), torch.tensor(merges, dtype=torch.int32).cuda(), len(merges), out, heads, hd)
+    want = torch.stack(want).float()
+    err = (out.float().cpu() - want).abs().max().item()
+    assert err <= (2e-5 if dtype == torch.float32 else 2.0 ** -8) * want.abs().max().item(), err
+
+
 def test_attention_long_tiles_on_four_waves(ops, monkeypatch):
     """Large tiles may be given four waves that split the keys and merge in the workgroup."""
     from from_scratch_inference_engine_amd.parts.attention import AttentionPlanner
