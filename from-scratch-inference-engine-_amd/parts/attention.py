@@ -120,8 +120,11 @@ class AttentionPlanner:
             longest = max(longest, min(keys, split_keys))
             n += max(1, -(-keys // split_keys))
         if mfma:
-            # items: a multiple of the number of requests (the captured graph pads with empty ones)
-            return (-(-n // host.n_seqs) * host.n_seqs,
+            # items: a multiple of the number of requests, and of what 1,024 keys of each need, so
+            # that a graph serves as many steps with short items as with long ones (the captured
+            # graph pads with empty items, whose workgroups leave at once)
+            step = host.n_seqs * max(1, 1024 // split_keys)
+            return (-(-n // step) * step,
                     self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)), split_keys)
         step = 4 * host.n_seqs
         return (-(-n // step) * step, 1, split_keys)
