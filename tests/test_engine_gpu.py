@@ -416,6 +416,39 @@ ODD = {
 }
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_decoding_against_contexts_that_are_split_and_merged(tmp_path, dtype):
+    """Requests of 40, 300 and 700 tokens decode together: a device with idle compute units
+    gives the long ones to several work items of 256 keys whose partial results are merged, the
+    short one needs no merge, and the graph of the step pads both tables.  Eagerly and through
+    graphs, against the plain implementation."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    cfg = dict(helpers.TINY_B, max_position_embeddings=1024)
+    d = helpers.make_model_dir(tmp_path / "long", cfg, seed=21)
+    model = load_model(d, dtype=dtype)
+    seqs = [helpers.token_ids(cfg["vocab_size"], n, 700 + n) for n in (40, 300, 700)]
+    refs = [plain.forward_dir(d, ids).numpy() for ids in seqs]
+    n_decoded = 6
+    for graphs in (False, True):
+        runner = Runner(model, page_size=8, num_pages=160, max_requests=4, use_graphs=graphs)
+        caches = [runner.manager.open(i) for i in range(len(seqs))]
+        runner.step([StepEntry(c, ids[:-n_decoded], []) for c, ids in zip(caches, seqs)])
+        for t in range(n_decoded, 0, -1):
+            out = runner.step([StepEntry(c, [ids[-t]], [0]) for c, ids in zip(caches, seqs)]).float().cpu().numpy()
+            for i, ref in enumerate(refs):
+                helpers.assert_close_to_plain(out[i:i + 1], ref[len(ref) - t:len(ref) - t + 1], dtype,
+                                              f"graphs={graphs} request of {len(seqs[i])} tokens, {t} from its end")
+        if graphs and runner.graphs.enabled:
+            assert runner.graphs.replays >= n_decoded - 2
+    if dtype == "bfloat16":  # the step that was tested is one that splits
+        from types import SimpleNamespace
+        host = SimpleNamespace(n_seqs=3, q_lens=[1, 1, 1], past_lens=[len(ids) - 1 for ids in seqs])
+        assert model.planners[0].split_keys(host, True) == 256
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("page_size", [3, 8])
 def test_sizes_the_fast_kernels_do_not_take_still_give_right_results(tmp_path, dtype, page_size):
