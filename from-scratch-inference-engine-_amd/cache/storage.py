@@ -31,12 +31,12 @@ class CacheLayout:
 class LayerCache:
     """What a mixer sees of the cache in one step.
 
-    Paged: ``k_pool`` [pages, kv_heads, page_size, head_dim] and ``v_pool`` [pages, kv_heads,
-    head_dim, page_size] of this layer,
+    Paged: ``k_pool`` [pages + 1, kv_heads, page_size, head_dim] and ``v_pool`` [pages + 1, kv_heads,
+    head_dim, page_size] of this layer (the last page is the spare one of padding rows),
     ``block_tables`` int32 [requests in the step, pages] (-1 = no page), ``slots`` int32 [tokens]
     (where each token's entry goes), ``page_size``, and ``writes`` (False when this call only
     reads a cache that another call fills).
-    State: ``state`` [max_requests, *shape]; the step's ``ctx.seq_slots`` index it."""
+    State: ``state`` [max_requests + 1, *shape]; the step's ``ctx.seq_slots`` index it."""
 
     __slots__ = ("k_pool", "v_pool", "block_tables", "slots", "page_size", "writes", "state", "group")
 
@@ -53,20 +53,25 @@ class CacheStorage:
         self.page_size = manager.page_size
         self.device = device
         self.dtype = dtype
-        # per group: keys [caches, pages, kv_heads, page_size, head_dim] and values, transposed
-        # within a page, [caches, pages, kv_heads, head_dim, page_size]
+        # per group: keys [caches, pages + 1, kv_heads, page_size, head_dim] and values, transposed
+        # within a page, [caches, pages + 1, kv_heads, head_dim, page_size].  The last page of a
+        # pool and the last state slot belong to no request (the allocators do not know them):
+        # they are where the rows that pad a batch to a captured graph's size read and write.
         self.k_pools: List[torch.Tensor] = []
         self.v_pools: List[torch.Tensor] = []
+        self.spare_pages: List[int] = []
         for g, need in enumerate(layout.paged_groups):
             n_pages = manager.allocators[g].num_pages
             n_caches = len(layout.group_caches[g])
-            self.k_pools.append(torch.zeros((n_caches, n_pages, need.n_kv_heads, self.page_size, need.head_dim),
+            self.spare_pages.append(n_pages)
+            self.k_pools.append(torch.zeros((n_caches, n_pages + 1, need.n_kv_heads, self.page_size, need.head_dim),
                                             dtype=dtype, device=device))
-            self.v_pools.append(torch.zeros((n_caches, n_pages, need.n_kv_heads, need.head_dim, self.page_size),
+            self.v_pools.append(torch.zeros((n_caches, n_pages + 1, need.n_kv_heads, need.head_dim, self.page_size),
                                             dtype=dtype, device=device))
+        self.spare_slot = manager.max_requests
         self.states: Dict[int, torch.Tensor] = {}
         for cid, need in layout.state_caches.items():
-            self.states[cid] = torch.zeros((manager.max_requests, *need.shape),
+            self.states[cid] = torch.zeros((manager.max_requests + 1, *need.shape),
                                            dtype=getattr(torch, need.dtype), device=device)
 
     def bytes(self) -> int:

@@ -7,19 +7,35 @@ the width of the block tables and the number of attention work items, on rounded
 lengths.  For each such shape the whole forward is captured once into a graph that reads all
 its index tables from one fixed device buffer; a later step of the same shape copies its tables
 there and replays the graph.
+
+The number of requests is rounded up as well (``padded_rows``): a batch that shrinks request by
+request as they finish would otherwise want a new graph, some tens of milliseconds of capture,
+at every size.  The rows that fill a batch up are requests of one token at position 0 whose
+cache is the pools' spare page and the spare state slot; they cost a decode step nothing that
+can be measured, no request reads what they write, and their logits are dropped.
 """
 
 from __future__ import annotations
 
 import gc
 import weakref
-from typing import Dict, Optional, Sequence, Tuple
+from types import SimpleNamespace
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
 from .context import HostBatch, StepEntry, build_context
 
 PAGE_BUCKET = 32  # block-table widths are rounded up to this many pages
+
+
+def padded_rows(n: int) -> int:
+    """Rows of the graph that serves a decode step of ``n`` requests: 1, 2, 4, 8, then multiples
+    of 16 (a tile of rows in the products), above 64 of 32."""
+    if n <= 8:
+        return 1 << max(0, n - 1).bit_length()
+    step = 16 if n <= 64 else 32
+    return -(-n // step) * step
 
 
 class DecodeGraphs:
@@ -44,11 +60,20 @@ class DecodeGraphs:
             raise RuntimeError("the runner of these graphs no longer exists")
         return runner
 
+    def filled_up(self, entries: Sequence[StepEntry]) -> List:
+        """The entries and, behind them, the rows that pad the batch to a graph's size."""
+        runner = self.runner
+        spare = SimpleNamespace(length=0, slot=runner.storage.spare_slot,
+                                tables=[[page] for page in runner.storage.spare_pages])
+        filler = SimpleNamespace(cache=spare, tokens=(0,), want=(0,))
+        return list(entries) + [filler] * (padded_rows(len(entries)) - len(entries))
+
     def shape_of(self, entries: Sequence[StepEntry]) -> Optional[dict]:
         """The padded sizes of this step, or None if it is not a plain decode step."""
         if not self.enabled or not all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
             return None
         runner = self.runner
+        entries = self.filled_up(entries)
         host = HostBatch(entries, runner.manager.page_size, runner.model.dtype)
         pages = max(len(t) for e in entries for t in e.cache.tables) if runner.manager.groups else 1
         pad = {"pages": -(-pages // PAGE_BUCKET) * PAGE_BUCKET}
@@ -64,6 +89,8 @@ class DecodeGraphs:
         stay valid until the next step of the same shape.  ``feed`` (int32, on the device)
         replaces the token ids after the tables have been sent."""
         runner = self.runner
+        n = len(entries)
+        entries = self.filled_up(entries)
         key = (len(entries),) + tuple(sorted((str(k), v) for k, v in pad.items()))
         hit = self._graphs.get(key)
         if hit is None:
@@ -74,7 +101,7 @@ class DecodeGraphs:
             ctx, tables = build_context(entries, runner.manager, runner.model.planners, runner._staging,
                                         runner.model.dtype, runner.model.device, pad=pad)
             if feed is not None:
-                ctx.token_ids.copy_(feed)
+                ctx.token_ids[:n].copy_(feed)
             runner.model.forward(ctx, runner.storage)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
@@ -95,12 +122,12 @@ class DecodeGraphs:
             # the eager run above already wrote this step's keys and values; replaying writes the
             # same values again
             graph.replay()
-            return logits
+            return logits[:n]
         graph, tables, logits, token_ids = hit
         build_context(entries, runner.manager, runner.model.planners, runner._staging, runner.model.dtype,
                       runner.model.device, pad=pad, into=tables)
         if feed is not None:
-            token_ids.copy_(feed)
+            token_ids[:n].copy_(feed)
         graph.replay()
         self.replays += 1
-        return logits
+        return logits[:n]

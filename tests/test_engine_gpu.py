@@ -251,6 +251,56 @@ def test_graph_replays_equal_eager_steps(model_dirs):
     assert g.captures + g.replays == before
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_batch_that_shrinks_decodes_through_graphs_of_padded_sizes(model_dirs, dtype):
+    """Seven requests decode together and end one after the other.  Graphs are captured for 8, 4,
+    2 and 1 rows only (the rows that fill a batch up read and write the spare page); what every
+    batch size returns for the real requests is what the eager runner returns (which runs the
+    unpadded batch), agrees with the plain model, and a request that comes later and is given the pages of one that ended
+    is not disturbed by what the filler rows wrote."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.graphs import padded_rows
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    assert [padded_rows(n) for n in (1, 2, 3, 4, 5, 8, 9, 16, 17, 33, 64, 65, 100)] == \
+        [1, 2, 4, 4, 8, 8, 16, 16, 32, 48, 64, 96, 128]
+    model = load_model(model_dirs["A"], dtype=dtype)
+    vocab = plain.read_config(model_dirs["A"])["vocab_size"]
+    seqs = [helpers.token_ids(vocab, 30 + 3 * i, 900 + i) for i in range(7)]
+    late = helpers.token_ids(vocab, 20, 950)
+    ref = [plain.forward_dir(model_dirs["A"], ids).numpy() for ids in seqs + [late]]
+    runners = [Runner(model, page_size=4, num_pages=96, max_requests=8, use_graphs=g) for g in (True, False)]
+    caches = [[r.manager.open(i) for i in range(7)] for r in runners]
+    n_pre = [len(ids) - (3 + 2 * i) for i, ids in enumerate(seqs)]  # request i decodes 3 + 2 i tokens, then ends
+    for r, cs in zip(runners, caches):
+        r.step([StepEntry(c, ids[:n], []) for c, ids, n in zip(cs, seqs, n_pre)])
+    live = list(range(7))
+    t = 0
+    while live:
+        outs = []
+        for r, cs in zip(runners, caches):
+            outs.append(r.step([StepEntry(cs[i], [seqs[i][n_pre[i] + t]], [0]) for i in live]).float().cpu())
+        helpers.assert_close_to_plain(outs[0].numpy(), outs[1].numpy(), dtype, f"step {t} with {len(live)} requests, graphs against eager")
+        for row, i in enumerate(live):
+            helpers.assert_close_to_plain(outs[0][row:row + 1].numpy(), ref[i][n_pre[i] + t:n_pre[i] + t + 1], dtype,
+                                          f"step {t}, request {i} in a batch of {len(live)}")
+        t += 1
+        for i in [i for i in live if n_pre[i] + t == len(seqs[i])]:
+            live.remove(i)
+            for r, cs in zip(runners, caches):
+                r.manager.close(cs[i])
+    g = runners[0].graphs
+    assert g.captures <= 5 and g.replays >= t - 5, (g.captures, g.replays)
+    # the pages of the ended requests, handed out again
+    for r in runners:
+        c = r.manager.open("late")
+        out = r.step([StepEntry(c, late[:-2], [])])
+        for j in (2, 1):
+            out = r.step([StepEntry(c, [late[-j]], [0])]).float().cpu().numpy()
+            helpers.assert_close_to_plain(out, ref[7][len(late) - j:len(late) - j + 1], dtype, f"late request, token -{j}")
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_decoding_with_partial_sums_in_the_residual_stream(model_dirs, name, monkeypatch):
     """The tiny models are too narrow for the projections to cut K by themselves, so the cut is
