@@ -34,6 +34,9 @@ extern "C" int fsie_attention_mfma(const void* q, int64_t q_stride, const void* 
                  "attention_mfma: head_dim %d must be a multiple of 16 up to 256", head_dim);
     FSIE_REQUIRE(page_size > 0 && page_size % 4 == 0, "attention_mfma: page_size %d must be a multiple of 4", page_size);
     FSIE_REQUIRE(max_pages > 0, "attention_mfma: empty block table");
+    // the kernel divides a key's position by the page size with one multiplication, exact below this
+    FSIE_REQUIRE((static_cast<int64_t>(max_pages) + 8) * page_size * page_size < (int64_t{1} << 32),
+                 "attention_mfma: %d pages of %d keys are more than the kernel can address", max_pages, page_size);
     FSIE_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0,
                  "attention_mfma: query rows must be 16-byte aligned");
     if (n_items == 0) return 0;

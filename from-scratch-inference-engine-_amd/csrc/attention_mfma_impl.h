@@ -136,6 +136,10 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
     }
 
     const int64_t head_stride = static_cast<int64_t>(page_size) * HD;  // one kv head of one page
+    // key / page_size as one multiplication (the host has checked that keys * page_size < 2^32): a
+    // division by a size known only at run time costs some thirty vector instructions, four times
+    // per block of 32 keys
+    const uint32_t page_magic = 0xFFFFFFFFu / static_cast<uint32_t>(page_size) + 1u;
     // this wave's run of key blocks
     const int kb_first = key_begin & ~31;
     const int n_blocks = (key_end - kb_first + 31) >> 5;
@@ -171,7 +175,7 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {  // the four table reads go out together
-            idx[i] = key[i] / page_size;
+            idx[i] = static_cast<int>(__umulhi(static_cast<uint32_t>(key[i]), page_magic));
             page[i] = table[min(idx[i], max_pages - 1)];
         }
 #pragma unroll

@@ -26,13 +26,31 @@ constexpr int kLdsKeys = 64;   // keys per block
 constexpr int kLdsWaves = 4;   // waves = tiles per workgroup
 constexpr int kLdsThreads = 64 * kLdsWaves;
 
-template <int HDT>
+// Whether, with a page size known at compile time, all 256 threads copy from one page in each of
+// their steps: step i of K and step i of V then both read page i of the block.
+template <int HDT, int PS>
+constexpr bool one_page_per_step() {
+    if (PS <= 0) return false;
+    for (int i = 0; i < HDT / 2; ++i)
+        for (int t = 0; t < kLdsThreads; ++t) {
+            const int p = t + kLdsThreads * i;
+            if ((p / (2 * HDT)) / PS != i || (p / (PS / 8)) / (HDT * 16) != i) return false;
+        }
+    return true;
+}
+
+// PS: the page size where it is known when the kernel is compiled (16, the engine's default), 0 = the
+// run-time argument.  With a known page size the pieces a thread copies for one step i all lie in
+// one page, the same for the whole workgroup: the table entries come through the scalar unit and
+// the loads take a scalar base and a per-thread offset that never changes.
+template <int HDT, int PS>
 __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT <= 8 ? 2 : 1, HDT <= 8 ? 2 : 1))) void attention_mfma_lds_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, const int32_t* __restrict__ groups, bf16_t* __restrict__ out, int n_heads,
-    int n_kv, int page_size, int window, float scale, int gh, int head_chunks) {
+    int n_kv, int page_size_arg, int window, float scale, int gh, int head_chunks) {
     constexpr int HD = HDT * 16;
+    const int page_size = PS > 0 ? PS : page_size_arg;
     constexpr int S32 = HDT / 2;       // 32-wide steps over the head dimension
     constexpr int NT = 2;              // query tiles of 16 rows per wave
     constexpr int KS = HD + 8;         // elements per key row in LDS (16 bytes of padding: no bank conflicts)
@@ -67,7 +85,9 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     const int n_rows = n_q * gh;
     const int c = lane & 15;
     const int G = lane >> 4;
-    const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
+    // the tiles of a group belong to one request: its table's address is the same for every wave
+    const int seq_wg = items[static_cast<int64_t>(first) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_SEQ];
+    const int32_t* table = block_tables + static_cast<int64_t>(seq_wg) * max_pages;
     const float scale2 = scale * kLog2e;
 
     // ---- this wave's queries (B operands)
@@ -101,49 +121,69 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     // K: a key's row is 2 HDT pieces of 16 bytes; piece p = t + 256 i is part p % (2 HDT) of key p / (2 HDT).
     // V: the values of a page lie as [head_dim][slot]; piece p is, in memory order, piece p % cpp of
     //    dimension (p / cpp) % HD of the block's page p / (cpp HD), cpp = page_size / 8.
-    const int64_t head_stride = static_cast<int64_t>(page_size) * HD;
+    // The page size is a power of two (8 to 64) that divides the block of 64 keys, and a block
+    // starts at a multiple of 64: a piece's place inside its page and its page's distance from the
+    // block's first page never change, so everything but the page number is computed once, here
+    // (a division by a size known only at run time costs some thirty vector instructions, and
+    // there were a dozen of them per thread and block).
+    const int page_shift = __ffs(page_size) - 1;
+    const int head_stride = page_size * HD;                 // one kv head of one page
+    const uint32_t page_stride = head_stride * n_kv;        // at most 64 * 256 * kv heads elements
     const int cpp = page_size >> 3;
     const int t = threadIdx.x;
     uint4 kreg[PER_THREAD], vreg[PER_THREAD];
     int k_dst[PER_THREAD], v_dst[PER_THREAD];
-    int k_key[PER_THREAD], k_part[PER_THREAD], v_page[PER_THREAD], v_off[PER_THREAD];
+    int k_key[PER_THREAD], k_pg[PER_THREAD], v_pg[PER_THREAD];
+    int k_in_page[PER_THREAD], v_in_page[PER_THREAD];
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) {
         const int p = t + kLdsThreads * i;
         k_key[i] = p / (2 * HDT);
-        k_part[i] = p - k_key[i] * (2 * HDT);
+        const int k_part = p - k_key[i] * (2 * HDT);
         // in LDS the keys of a group of 32 lie in the order the lanes read them: key
         // 8 a + 4 tile + b (b < 4) of the group at row 16 tile + 4 a + b, so that the 16 lanes of a
         // score tile read 16 consecutive rows (no bank conflicts with the padded row length)
         const int k5 = k_key[i] & 31;
         const int row = (k_key[i] & 32) + ((k5 >> 2) & 1) * 16 + ((k5 >> 3) << 2) + (k5 & 3);
-        k_dst[i] = row * KS + k_part[i] * 8;
+        k_dst[i] = row * KS + k_part * 8;
+        k_pg[i] = k_key[i] >> page_shift;
+        k_in_page[i] = kvh * head_stride + (k_key[i] & (page_size - 1)) * HD + k_part * 8;
         const int w = p % cpp, rest = p / cpp;
         const int d = rest % HD, pg = rest / HD;
-        v_page[i] = pg;
-        v_off[i] = d * page_size + w * 8;      // inside the page's head
+        v_pg[i] = pg;
+        v_in_page[i] = kvh * head_stride + d * page_size + w * 8;
         v_dst[i] = d * VS + (pg * cpp + w) * 8;  // key chunk pg * cpp + w of the block
     }
     auto fetch = [&](int kb) {
-        // pages: a key past the end, or behind a window, reads page 0 (finite values, probability zero)
+        // pages: a key without a page (past the end, or behind a window) reads page 0: finite values,
+        // probability zero.  Keys past the end inside an existing page are read as they are (the
+        // scores of such keys are replaced, not multiplied, and the pools hold finite values only).
+        const int kb_page = kb >> page_shift;
+        if constexpr (one_page_per_step<HDT, PS>()) {
+            int page[PER_THREAD];
+#pragma unroll
+            for (int i = 0; i < PER_THREAD; ++i) page[i] = table[min(kb_page + i, max_pages - 1)];
+#pragma unroll
+            for (int i = 0; i < PER_THREAD; ++i) {
+                const bool ok = kb_page + i < max_pages && page[i] >= 0;
+                const uint64_t at = static_cast<uint64_t>(ok ? page[i] : 0) * page_stride;
+                kreg[i] = ld16(k_pool + at + static_cast<uint32_t>(k_in_page[i]));
+                vreg[i] = ld16(v_pool + at + static_cast<uint32_t>(v_in_page[i]));
+            }
+            return;
+        }
         int kpage[PER_THREAD], vpage[PER_THREAD];
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
-            const int ki = min((kb + k_key[i]) / page_size, max_pages - 1);
-            const int vi = min(kb / page_size + v_page[i], max_pages - 1);
-            kpage[i] = table[ki];
-            vpage[i] = table[vi];
+            kpage[i] = table[min(kb_page + k_pg[i], max_pages - 1)];
+            vpage[i] = table[min(kb_page + v_pg[i], max_pages - 1)];
         }
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
-            const int key = kb + k_key[i];
-            const bool kok = key < wg_end && key / page_size < max_pages && kpage[i] >= 0;
-            const int64_t khead = (static_cast<int64_t>(kok ? kpage[i] : 0) * n_kv + kvh) * head_stride;
-            const int slot = kok ? key % page_size : 0;
-            kreg[i] = ld16(k_pool + khead + static_cast<int64_t>(slot) * HD + k_part[i] * 8);
-            const bool vok = kb / page_size + v_page[i] < max_pages && vpage[i] >= 0;
-            const int64_t vhead = (static_cast<int64_t>(vok ? vpage[i] : 0) * n_kv + kvh) * head_stride;
-            vreg[i] = ld16(v_pool + vhead + v_off[i]);
+            const bool kok = kb_page + k_pg[i] < max_pages && kpage[i] >= 0;
+            kreg[i] = ld16(k_pool + static_cast<uint64_t>(kok ? kpage[i] : 0) * page_stride + k_in_page[i]);
+            const bool vok = kb_page + v_pg[i] < max_pages && vpage[i] >= 0;
+            vreg[i] = ld16(v_pool + static_cast<uint64_t>(vok ? vpage[i] : 0) * page_stride + v_in_page[i]);
         }
     };
     auto stash = [&](int buf) {
@@ -304,7 +344,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     }
 }
 
-template <int HDT>
+template <int HDT, int PS>
 int launch_lds(const bf16_t* q, int64_t q_stride, const bf16_t* k_pool, const bf16_t* v_pool,
                const int32_t* block_tables, int max_pages, const int32_t* items, const int32_t* groups, int n_groups,
                bf16_t* out, int n_heads, int n_kv, int page_size, int window, float scale, hipStream_t stream) {
@@ -312,7 +352,7 @@ int launch_lds(const bf16_t* q, int64_t q_stride, const bf16_t* k_pool, const bf
     const int gh = group < 32 ? group : 32;
     const int head_chunks = (group + gh - 1) / gh;
     const dim3 grid(n_groups, n_kv * head_chunks);
-    attention_mfma_lds_kernel<HDT><<<grid, kLdsThreads, 0, stream>>>(q, q_stride, k_pool, v_pool, block_tables, max_pages,
+    attention_mfma_lds_kernel<HDT, PS><<<grid, kLdsThreads, 0, stream>>>(q, q_stride, k_pool, v_pool, block_tables, max_pages,
                                                                      items, groups, out, n_heads, n_kv, page_size,
                                                                      window, scale, gh, head_chunks);
     FSIE_CHECK_LAUNCH("attention_mfma_lds");
@@ -351,8 +391,11 @@ extern "C" int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const vo
     bf16_t* oo = static_cast<bf16_t*>(out);
 #define FSIE_LDS_CASE(H)                                                                                           \
     case H:                                                                                                        \
-        return fsie_attn::launch_lds<H>(qq, q_stride, kk, vv, block_tables, max_pages, items, groups, n_groups, oo, \
-                                        n_heads, n_kv, page_size, window, scale, stream)
+        return page_size == 16                                                                                     \
+                   ? fsie_attn::launch_lds<H, 16>(qq, q_stride, kk, vv, block_tables, max_pages, items, groups,    \
+                                                  n_groups, oo, n_heads, n_kv, page_size, window, scale, stream)   \
+                   : fsie_attn::launch_lds<H, 0>(qq, q_stride, kk, vv, block_tables, max_pages, items, groups,     \
+                                                 n_groups, oo, n_heads, n_kv, page_size, window, scale, stream)
     switch (head_dim / 16) {
         FSIE_LDS_CASE(2);
         FSIE_LDS_CASE(4);
