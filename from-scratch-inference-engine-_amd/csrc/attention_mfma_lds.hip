@@ -20,6 +20,8 @@
 // Requires head_dim a multiple of 32 (up to 256) and a page size of 8, 16, 32 or 64.
 #include "attention_mfma_impl.h"
 
+#include <type_traits>
+
 namespace fsie_attn {
 
 constexpr int kLdsKeys = 64;   // keys per block
@@ -67,12 +69,13 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     const int wave = threadIdx.x >> 6;
     const bool active = wave < n_tiles;
     const int32_t* item = items + static_cast<int64_t>(first + (active ? wave : 0)) * FSIE_ATTN_ITEM_INTS;
-    const int seq = item[FSIE_ATTN_ITEM_SEQ];
-    const int q_row0 = item[FSIE_ATTN_ITEM_QROW];
-    const int n_q = item[FSIE_ATTN_ITEM_NQ];
-    const int pos0 = item[FSIE_ATTN_ITEM_POS];
-    const int key_begin = item[FSIE_ATTN_ITEM_KBEGIN];
-    const int key_end = item[FSIE_ATTN_ITEM_KEND];
+    // the same for every lane of the wave: kept in scalar registers, so that what is decided by
+    // them is a scalar branch and not a masked region
+    const int q_row0 = __builtin_amdgcn_readfirstlane(item[FSIE_ATTN_ITEM_QROW]);
+    const int n_q = __builtin_amdgcn_readfirstlane(item[FSIE_ATTN_ITEM_NQ]);
+    const int pos0 = __builtin_amdgcn_readfirstlane(item[FSIE_ATTN_ITEM_POS]);
+    const int key_begin = __builtin_amdgcn_readfirstlane(item[FSIE_ATTN_ITEM_KBEGIN]);
+    const int key_end = __builtin_amdgcn_readfirstlane(item[FSIE_ATTN_ITEM_KEND]);
     // the workgroup's keys: from the first tile's first to the last tile's last
     const int wg_begin = items[static_cast<int64_t>(first) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_KBEGIN] & ~(kLdsKeys - 1);
     const int wg_end = items[static_cast<int64_t>(first + n_tiles - 1) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_KEND];
@@ -201,13 +204,18 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     // that one maximum per query row serves the whole block and its two lane swaps are not waited
     // for twice; the scores stay in the units of the products and the softmax scale goes into the
     // exponent: p = exp2((s - m) * scale2), one fused multiply-add per score.
-    auto compute_block = [&](int kb, const bf16_t* kbuf, const bf16_t* vbuf) {
+    // INNER: a block that every row of the wave sees whole (below the diagonal, inside the key range
+    // and the window; in a long portion nearly every block): no masks and no branches, one
+    // straight run of instructions in which the compiler can place the LDS reads of a product
+    // ahead of the arithmetic that precedes it.
+    auto compute_block = [&](int kb, const bf16_t* kbuf, const bf16_t* vbuf, auto inner) {
+        constexpr bool INNER = decltype(inner)::value;
         bool use[2];
         floatx4 st[2][NT][2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int kh = kb + 32 * h;
-            use[h] = kh <= my_last && kh < key_end && kh + 32 > key_begin;  // the same for the whole wave
+            use[h] = INNER || (kh <= my_last && kh < key_end && kh + 32 > key_begin);  // the same for the whole wave
             if (!use[h]) continue;
             F16B kf[2][S32];
 #pragma unroll
@@ -236,8 +244,8 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
         for (int h = 0; h < 2; ++h) {
             if (!use[h]) continue;
             const int kh = kb + 32 * h;
-            const bool full = kh >= key_begin && kh + 32 <= key_end && kh + 31 <= pos0 &&
-                              (window <= 0 || kh > pos0 + n_q - 1 - window);
+            const bool full = INNER || (kh >= key_begin && kh + 32 <= key_end && kh + 31 <= pos0 &&
+                                        (window <= 0 || kh > pos0 + n_q - 1 - window));
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 if (full) {
@@ -258,15 +266,36 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
                 for (int i = 0; i < 8; ++i) m_loc[nt] = fmaxf(m_loc[nt], sv[h][nt][i]);
             }
         }
-        // probabilities
-        F16B pb[2][NT];
+        // new maxima; the accumulators shrink only when some row's maximum moved (rare after the
+        // first blocks), for both tiles behind one branch, so that what follows it (the exponentials,
+        // the LDS reads of the values and the second product) is one run of instructions
+        float corr[NT], shift[NT];
+        bool moved = false;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             // the maximum never goes below a finite floor, so that a row that has seen no key yet
             // gives exp2(-inf) = 0 and not exp2(-inf + inf)
             const float m_new = fmaxf(fmaxf(m_run[nt], max_xor32(max_xor16(m_loc[nt]))), -1e30f);
-            const float corr = __builtin_amdgcn_exp2f((m_run[nt] - m_new) * scale2);
-            const float shift = -m_new * scale2;
+            corr[nt] = __builtin_amdgcn_exp2f((m_run[nt] - m_new) * scale2);
+            shift[nt] = -m_new * scale2;
+            m_run[nt] = m_new;
+            moved = moved || corr[nt] != 1.f;
+        }
+        if (__any(moved)) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int dt = 0; dt < HDT; ++dt) {
+                    acc[nt][dt][0] *= corr[nt];
+                    acc[nt][dt][1] *= corr[nt];
+                    acc[nt][dt][2] *= corr[nt];
+                    acc[nt][dt][3] *= corr[nt];
+                }
+        }
+        // probabilities
+        F16B pb[2][NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
             float p_sum = 0.f;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
@@ -274,24 +303,13 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
                 float p[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    p[i] = __builtin_amdgcn_exp2f(fmaf(sv[h][nt][i], scale2, shift));
+                    p[i] = __builtin_amdgcn_exp2f(fmaf(sv[h][nt][i], scale2, shift[nt]));
                     p_sum += p[i];
                 }
                 pb[h][nt].raw = uint4{pack2_bf16(p[0], p[1]), pack2_bf16(p[2], p[3]), pack2_bf16(p[4], p[5]),
                                       pack2_bf16(p[6], p[7])};
             }
-            l_run[nt] = l_run[nt] * corr + p_sum;  // this lane's keys only; the lane groups are summed at the end
-            m_run[nt] = m_new;
-            // the accumulators shrink only when some row's maximum moved (rare after the first blocks)
-            if (__any(corr != 1.f)) {
-#pragma unroll
-                for (int dt = 0; dt < HDT; ++dt) {
-                    acc[nt][dt][0] *= corr;
-                    acc[nt][dt][1] *= corr;
-                    acc[nt][dt][2] *= corr;
-                    acc[nt][dt][3] *= corr;
-                }
-            }
+            l_run[nt] = l_run[nt] * corr[nt] + p_sum;  // this lane's keys only; the lane groups are summed at the end
         }
         // O^T += V^T P^T
 #pragma unroll
@@ -318,7 +336,10 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
         for (int kb = wg_begin; kb < wg_end; kb += kLdsKeys) {
             const bool more = kb + kLdsKeys < wg_end;
             if (more) fetch(kb + kLdsKeys);
-            if (active) compute_block(kb, k_lds[buf], v_lds[buf]);
+            const bool inner = active && kb >= key_begin && kb + kLdsKeys <= key_end && kb + kLdsKeys - 1 <= pos0 &&
+                               (window <= 0 || kb > my_last - window);
+            if (inner) compute_block(kb, k_lds[buf], v_lds[buf], std::true_type{});
+            else if (active) compute_block(kb, k_lds[buf], v_lds[buf], std::false_type{});
             if (more) stash(buf ^ 1);
             __syncthreads();
             buf ^= 1;
