@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, const int32_t* __restrict__ groups, bf16_t* __restrict__ out, int n_heads,
-    int n_kv, int page_size_arg, int window, float scale, int gh, int head_chunks) {
+    int n_kv, int page_size_arg, int window, float scale, int gh, int head_chunks, int n_groups, int n_y) {
     constexpr int HD = HDT * 16;
     const int page_size = PS > 0 ? PS : page_size_arg;
     constexpr int S32 = HDT / 2;       // 32-wide steps over the head dimension
@@ -63,7 +63,19 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
 
     // the groups are listed by ascending position, and a later group has more keys to read: the
     // grid takes them from the back, so that the longest workgroups start first
-    const int g_idx = gridDim.x - 1 - blockIdx.x;
+    // Which group and which kv head (and chunk of its heads): with a two-dimensional grid, blockIdx
+    // says so.  With a one-dimensional grid (n_y = kv heads x chunks divides the 8 dies of the
+    // device) consecutive workgroups go to consecutive dies, and die x takes y = x % n_y only:
+    // the keys and values of a kv head are then read through one die's L2 cache (two dies for 4 kv
+    // heads) and not through all eight.
+    int g_lin = blockIdx.x, by = blockIdx.y;
+    if (n_y > 0) {
+        const int die = blockIdx.x & 7;
+        by = die % n_y;
+        g_lin = (blockIdx.x >> 3) * (8 / n_y) + die / n_y;
+        if (g_lin >= n_groups) return;
+    }
+    const int g_idx = n_groups - 1 - g_lin;
     const int first = groups[2 * g_idx], n_tiles = groups[2 * g_idx + 1];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -81,8 +93,8 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     const int wg_end = items[static_cast<int64_t>(first + n_tiles - 1) * FSIE_ATTN_ITEM_INTS + FSIE_ATTN_ITEM_KEND];
 
     const int group = n_heads / n_kv;
-    const int kvh = blockIdx.y / head_chunks;
-    const int chunk = blockIdx.y - kvh * head_chunks;
+    const int kvh = by / head_chunks;
+    const int chunk = by - kvh * head_chunks;
     const int gh_here = min(gh, group - chunk * gh);
     const int h_base = kvh * group + chunk * gh;
     const int n_rows = n_q * gh;
@@ -372,10 +384,14 @@ int launch_lds(const bf16_t* q, int64_t q_stride, const bf16_t* k_pool, const bf
     const int group = n_heads / n_kv;
     const int gh = group < 32 ? group : 32;
     const int head_chunks = (group + gh - 1) / gh;
-    const dim3 grid(n_groups, n_kv * head_chunks);
+    const int ys = n_kv * head_chunks;
+    const bool by_die = ys <= 8 && 8 % ys == 0;
+    // by die: every die gets the same number of workgroups, the last ones of which may be empty
+    const dim3 grid = by_die ? dim3(static_cast<unsigned>((n_groups + 8 / ys - 1) / (8 / ys)) * 8) : dim3(n_groups, ys);
     attention_mfma_lds_kernel<HDT, PS><<<grid, kLdsThreads, 0, stream>>>(q, q_stride, k_pool, v_pool, block_tables, max_pages,
                                                                      items, groups, out, n_heads, n_kv, page_size,
-                                                                     window, scale, gh, head_chunks);
+                                                                     window, scale, gh, head_chunks, n_groups,
+                                                                     by_die ? ys : 0);
     FSIE_CHECK_LAUNCH("attention_mfma_lds");
     return 0;
 }
