@@ -24,6 +24,7 @@ extern "C" int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* 
     FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_skinny: at most %d rows, got %d",
                  FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
     FSIE_REQUIRE(K % 8 == 0, "gemm_mfma_skinny: K=%d must be a multiple of 8", K);
+    FSIE_REQUIRE(K <= (1 << 23), "gemm_mfma_skinny: K=%d is more than the kernel's 32-bit offsets into x take", K);
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
                  "gemm_mfma_skinny: operands must be 16-byte aligned");
     FSIE_REQUIRE(waves == 0 || waves == 1 || waves == 2 || waves == 4 || waves == 8 || waves == 16,
@@ -77,6 +78,7 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_skinny_rope: at most %d rows, got %d",
                  FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
     FSIE_REQUIRE(K % 8 == 0, "gemm_mfma_skinny_rope: K=%d must be a multiple of 8", K);
+    FSIE_REQUIRE(K <= (1 << 23), "gemm_mfma_skinny_rope: K=%d is more than the kernel's 32-bit offsets into x take", K);
     FSIE_REQUIRE(head_dim > 0 && head_dim % 16 == 0, "gemm_mfma_skinny_rope: head_dim %d must be a multiple of 16",
                  head_dim);
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,

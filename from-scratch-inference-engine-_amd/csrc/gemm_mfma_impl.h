@@ -18,6 +18,7 @@ namespace fsie_mm {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 union Frag {
     uint4 raw;
@@ -94,12 +95,15 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
         n = min(n, N - 1);  // rows past the end repeat the last one; never written
         wp[b] = w + static_cast<int64_t>(n) * K;
     }
-    const bf16_t* xp[MT];
+    // X is read through a buffer descriptor that ends with row M - 1: a lane whose row lies past
+    // the end gets zeros and asks the memory for nothing (its columns of D are never written).
+    // With one row (decoding a single request) 4 lanes of 64 fetch; reading the last row again
+    // instead costs as many requests to the cache as a full tile.
+    const __amdgpu_buffer_rsrc_t x_rows = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(x), 0, M * K * static_cast<int>(sizeof(bf16_t)), 0x00020000);
+    int xo[MT];  // byte offset of this lane's row
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        // rows of X past the end read the last row again: their columns of D are never written
-        xp[t] = x + static_cast<int64_t>(min(t * 16 + row, M - 1)) * K;
-    }
+    for (int t = 0; t < MT; ++t) xo[t] = (t * 16 + row) * K * static_cast<int>(sizeof(bf16_t));
     floatx4 acc[NB][MT];
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -170,7 +174,11 @@ __global__ __launch_bounds__(WAVES * FSIE_WAVE) void gemm_mfma_skinny_kernel(
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) a[u][h][nb].raw = *reinterpret_cast<const uint4*>(wp[nb] + k0c);
 #pragma unroll
-                for (int t = 0; t < MT; ++t) b[u][h][t].raw = *reinterpret_cast<const uint4*>(xp[t] + k0c);
+                for (int t = 0; t < MT; ++t) {
+                    const u32x4 got = __builtin_amdgcn_raw_buffer_load_b128(
+                        x_rows, xo[t] + k0c * static_cast<int>(sizeof(bf16_t)), 0, 0);
+                    b[u][h][t].raw = uint4{got.x, got.y, got.z, got.w};
+                }
             }
 #pragma unroll
         for (int u = 0; u < U; ++u)
