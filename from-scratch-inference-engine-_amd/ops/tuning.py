@@ -6,8 +6,8 @@ other kernels are sometimes a good deal faster (measured on MI355X at 2,048 rows
 568 us for N = 37888, K = 3584, and 261 against 357 us for N = 3584, K = 18944).  With tuning on,
 torch's TunableOp times the library's candidates the first time a shape is seen and keeps the
 best (in the process, and in a file under the temporary folder for later ones).  Each new shape
-costs seconds, so only two kinds of row counts are tuned: multiples of 256 (a full token budget of
-prefill) and multiples of 16 up to 64 (decode batches, timed in the eager run that precedes the
+costs seconds (at 16,384 rows, minutes), so only two kinds of row counts are tuned: multiples of 256
+up to 4,096 (a full token budget of prefill) and multiples of 16 up to 64 (decode batches, timed in the eager run that precedes the
 capture of their graph); never inside a graph capture.  Other shapes use what has been found for
 them, or the heuristic.
 """
@@ -19,7 +19,7 @@ import tempfile
 
 import torch
 
-_TUNED_ROWS = 256
+_TUNED_ROWS, _TUNED_MAX_ROWS = 256, 4096
 _TUNED_DECODE_ROWS, _TUNED_DECODE_MAX = 16, 64
 _state = {"on": False}
 
@@ -57,7 +57,8 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     import torch.cuda.tunable as tunable
 
     rows = x.shape[0]
-    tune = ((rows % _TUNED_ROWS == 0 or (rows <= _TUNED_DECODE_MAX and rows % _TUNED_DECODE_ROWS == 0)) and rows > 0
+    tune = (((rows % _TUNED_ROWS == 0 and rows <= _TUNED_MAX_ROWS)
+             or (rows <= _TUNED_DECODE_MAX and rows % _TUNED_DECODE_ROWS == 0)) and rows > 0
             and not torch.cuda.is_current_stream_capturing())
     if not tune:
         return torch.mm(x, weight.t())
