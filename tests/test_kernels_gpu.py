@@ -397,6 +397,9 @@ def run_attention(ops, case, heads, kv, hd, window=None, share_keys=True):
     (3, 1, 256, 64, None),
     (28, 4, 128, 16, None),  # a large model's geometry: 7 heads per kv head
     (2, 1, 80, 12, 300),     # head size an odd multiple of 16, page size no power of two
+    (6, 3, 64, 16, None),    # three kv heads: they do not divide the device's eight dies
+    (40, 8, 128, 16, None),  # the 14B and 32B geometry: 5 heads per kv head, one kv head a die
+    (5, 1, 128, 32, 200),    # head size 128 with a page size other than 16, and a window
 ])
 def test_attention_over_pages(ops, dtype, scalar, heads, kv, hd, page, window):
     # (past, new): the reference's (7, 5) and (19, 1), a long decode that is split, whole prompts,
