@@ -68,6 +68,16 @@ class Sequence:
     def context(self) -> List[int]:
         return self.request.prompt + self.output
 
+    def tokens(self, start: int, n: int) -> List[int]:
+        """``context[start:start + n]`` without putting the whole context together (a decode step
+        asks every request for one token of a context of thousands)."""
+        prompt = self.request.prompt
+        if start >= len(prompt):
+            return self.output[start - len(prompt):start - len(prompt) + n]
+        if start + n <= len(prompt):
+            return prompt[start:start + n]
+        return prompt[start:] + self.output[:start + n - len(prompt)]
+
     @property
     def computed(self) -> int:
         return self.cache.length if self.cache is not None else 0
@@ -176,9 +186,8 @@ class Scheduler:
                 n = self._fit_tokens(taken, seq, n)
                 if n <= 0:
                     continue
-                ctx = seq.context
-                tokens = ctx[seq.computed:seq.computed + n]
-                items.append(ScheduledItem(seq, tokens, seq.computed + n == len(ctx)))
+                tokens = seq.tokens(seq.computed, n)
+                items.append(ScheduledItem(seq, tokens, n == seq.remaining))
                 for g, k in enumerate(self.manager.new_pages_needed(seq.cache, n)):
                     taken[g] += k
                 budget -= n
