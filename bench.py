@@ -60,6 +60,66 @@ def decode_bytes(c, layers: int, batch: int, context: float, itemsize: int) -> f
     return weights + cache
 
 
+def other_workload(args, cfg, model, shape_name, layers, full_layers, page) -> int:
+    """The two workloads of BASELINE.json beside the default run; one JSON line each."""
+    import torch
+
+    from from_scratch_inference_engine_amd import Engine, SamplingParams
+
+    gen = torch.Generator().manual_seed(0)
+    budget = 2048
+    base = {"unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": args.dtype,
+            "data": "synthetic: random weights N(0,0.02), uniform random token ids"}
+    sizes = {"model": shape_name, "layers": layers, "layers_of_config": full_layers, "kv_block": page,
+             "tokens_per_step": budget}
+    if args.workload == "mixed":
+        longest = args.max_prompt + args.outputs
+        engine = Engine(model, block_size=page, num_blocks=args.requests * -(-longest // page) + 64,
+                        max_batch=args.requests, max_tokens_per_step=budget)
+        record = None
+        for rep in range(2):  # the first pass pays the graph captures and the library's kernel selection
+            lens = torch.randint(args.min_prompt, args.max_prompt + 1, (args.requests,), generator=gen).tolist()
+            prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for n in lens]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ids = [engine.add_request(p, SamplingParams(temperature=0.0), max_tokens=args.outputs) for p in prompts]
+            first = None
+            while engine.has_work():
+                engine.step()
+                if first is None and all(len(engine.output(i)) > 0 for i in ids):
+                    torch.cuda.synchronize()
+                    first = time.perf_counter() - t0
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            made = sum(len(engine.output(i)) for i in ids)
+            print(f"[bench] pass {rep}: {sum(lens)} prompt tokens, {made} generated in {dt * 1e3:.0f} ms "
+                  f"({first * 1e3:.0f} ms until every request had a token)", file=sys.stderr, flush=True)
+            record = {"metric": f"tokens/s (prompt + generated) of {args.requests} requests through the scheduler, {shape_name}",
+                      "value": (sum(lens) + made) / dt, "generated_per_s": made / dt, "ms": dt * 1e3,
+                      "ms_until_all_started": first * 1e3, "prompt_tokens": sum(lens), "generated_tokens": made,
+                      "config": dict(sizes, requests=args.requests, min_prompt=args.min_prompt,
+                                     max_prompt=args.max_prompt, outputs=args.outputs)}
+        print(json.dumps(dict(base, **record)))
+        return 0
+    n = args.prefill_tokens
+    engine = Engine(model, block_size=page, num_blocks=-(-(n + 1) // page) + 64, max_batch=1,
+                    max_tokens_per_step=budget)
+    times = []
+    for rep in range(3):
+        prompt = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.generate(prompt, SamplingParams(temperature=0.0), max_tokens=1)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        print(f"[bench] prefill of {n} tokens, pass {rep}: {times[-1] * 1e3:.0f} ms", file=sys.stderr, flush=True)
+    dt = min(times[1:])
+    print(json.dumps(dict(base, metric=f"prefill tokens/s, one prompt of {n} tokens in portions of {budget}, {shape_name}",
+                          value=n / dt, ms=dt * 1e3, frac=prefill_flops(cfg, layers, n) / dt / PEAK_FLOPS[args.dtype],
+                          config=dict(sizes, prefill_tokens=n))))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -72,6 +132,16 @@ def main() -> int:
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
+    ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill"], default="decode",
+                    help="decode: the default run.  mixed: --requests prompts of --min-prompt to --max-prompt tokens, "
+                         "--outputs tokens each, through the scheduler (BASELINE.json's configs[3] with --shape 14b).  "
+                         "long-prefill: one prompt of --prefill-tokens tokens in portions of the token budget "
+                         "(configs[4] with --shape 32b)")
+    ap.add_argument("--requests", type=int, default=32)
+    ap.add_argument("--min-prompt", type=int, default=128)
+    ap.add_argument("--max-prompt", type=int, default=4096)
+    ap.add_argument("--outputs", type=int, default=128)
+    ap.add_argument("--prefill-tokens", type=int, default=16384)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
@@ -104,6 +174,8 @@ def main() -> int:
 
     page = 16
     context = raw["max_position_embeddings"]
+    if args.workload != "decode":
+        return other_workload(args, cfg, model, shape_name, layers, full_layers, page)
     biggest = max(args.batch, 1 if args.no_points else 64)
     budget = 2048  # tokens a step may hold: the prompts of a large batch enter over several steps
     # requests whose prompt went in first decode while the others' prompts still enter: they get
