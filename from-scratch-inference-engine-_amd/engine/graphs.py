@@ -13,6 +13,11 @@ request as they finish would otherwise want a new graph, some tens of millisecon
 at every size.  The rows that fill a batch up are requests of one token at position 0 whose
 cache is the pools' spare page and the spare state slot; they cost a decode step nothing that
 can be measured, no request reads what they write, and their logits are dropped.
+
+A shape is captured when it comes for the third time (``capture_after``); until then its steps
+run eagerly, which costs a few milliseconds of host time each where a capture costs thirty: the
+shapes a batch passes through while its last requests end, one or two steps each, are not worth
+a graph.
 """
 
 from __future__ import annotations
@@ -27,6 +32,7 @@ import torch
 from .context import HostBatch, StepEntry, build_context
 
 PAGE_BUCKET = 32  # block-table widths are rounded up to this many pages
+CAPTURE_AFTER = 3  # a shape is captured the n-th time it is asked for (read when a runner is made)
 
 
 def padded_rows(n: int) -> int:
@@ -39,13 +45,15 @@ def padded_rows(n: int) -> int:
 
 
 class DecodeGraphs:
-    def __init__(self, runner, max_graphs: int = 64):
+    def __init__(self, runner, max_graphs: int = 64, capture_after: Optional[int] = None):
         # no cycle with the runner: a runner that is dropped must free its graphs and pinned
         # buffers then and there, not whenever the collector of cycles next runs (which may be
         # in the middle of another runner's capture, where freeing device memory is an error
         # that ends the process)
         self._runner = weakref.ref(runner)
         self.max_graphs = max_graphs
+        self.capture_after = CAPTURE_AFTER if capture_after is None else capture_after
+        self._asked: Dict[Tuple, int] = {}
         self._graphs: Dict[Tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
         model = runner.model
         parts = [p for block in model.spec.layers for p in (block, *block.sub_parts().values())]
@@ -84,16 +92,23 @@ class DecodeGraphs:
             pad[planner.key] = bucket
         return pad
 
-    def step(self, entries: Sequence[StepEntry], pad: dict, feed: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], pad: dict,
+             feed: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run the (already reserved) decode step through its graph; returns the logits, which
-        stay valid until the next step of the same shape.  ``feed`` (int32, on the device)
-        replaces the token ids after the tables have been sent."""
+        stay valid until the next step of the same shape, or None when the shape has no graph
+        and is not due for one yet (the caller then runs the step eagerly).  ``feed`` (int32, on
+        the device) replaces the token ids after the tables have been sent."""
         runner = self.runner
         n = len(entries)
         entries = self.filled_up(entries)
         key = (len(entries),) + tuple(sorted((str(k), v) for k, v in pad.items()))
         hit = self._graphs.get(key)
         if hit is None:
+            if len(self._asked) > 4096:
+                self._asked.clear()
+            asked = self._asked[key] = self._asked.get(key, 0) + 1
+            if asked < self.capture_after:
+                return None
             if len(self._graphs) >= self.max_graphs:
                 self._graphs.pop(next(iter(self._graphs)))
             # eager run on the tables of this step first: allocates nothing the graph keeps, warms

@@ -213,8 +213,8 @@ class Runner:
             self.manager.reserve(e.cache, len(e.tokens))
         self.storage.reset_states([e.cache.slot for e in entries if e.cache.length == 0])
         pad = self.graphs.shape_of(entries) if self.graphs is not None else None
-        if pad is not None:
-            logits = self.graphs.step(entries, pad, feed)
+        logits = self.graphs.step(entries, pad, feed) if pad is not None else None
+        if logits is not None:
             if keep:
                 logits = logits.clone()
         else:

@@ -301,6 +301,31 @@ def test_a_batch_that_shrinks_decodes_through_graphs_of_padded_sizes(model_dirs,
             helpers.assert_close_to_plain(out, ref[7][len(late) - j:len(late) - j + 1], dtype, f"late request, token -{j}")
 
 
+def test_a_shape_is_captured_the_third_time_it_comes(model_dirs, monkeypatch):
+    """With the engine's own threshold the first two decode steps of a shape run eagerly, the
+    third captures its graph and later ones replay it; all of them agree with the plain model."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine import graphs
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    monkeypatch.setattr(graphs, "CAPTURE_AFTER", 3)
+    model = load_model(model_dirs["B"], dtype="bfloat16")
+    runner = Runner(model, page_size=8, num_pages=32, max_requests=2)
+    assert runner.graphs.capture_after == 3
+    vocab = plain.read_config(model_dirs["B"])["vocab_size"]
+    ids = helpers.token_ids(vocab, 30, 960)
+    ref = plain.forward_dir(model_dirs["B"], ids).numpy()
+    cache = runner.manager.open("a")
+    runner.step([StepEntry(cache, ids[:24], [])])
+    seen = []
+    for t in range(24, 30):
+        out = runner.step([StepEntry(cache, [ids[t]], [0])]).float().cpu().numpy()
+        helpers.assert_close_to_plain(out, ref[t:t + 1], "bfloat16", f"token {t}")
+        seen.append((runner.graphs.captures, runner.graphs.replays))
+    assert seen == [(0, 0), (0, 0), (1, 0), (1, 1), (1, 2), (1, 3)]
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_decoding_with_partial_sums_in_the_residual_stream(model_dirs, name, monkeypatch):
     """The tiny models are too narrow for the projections to cut K by themselves, so the cut is
