@@ -36,8 +36,11 @@ QWEN25_7B = {
 QWEN25_14B = dict(QWEN25_7B, hidden_size=5120, num_hidden_layers=48, num_attention_heads=40, num_key_value_heads=8,
                   intermediate_size=13824, rms_norm_eps=1e-5, max_position_embeddings=8192)
 QWEN25_32B = dict(QWEN25_14B, num_hidden_layers=64, intermediate_size=27648, max_position_embeddings=16384)
-SHAPES = {"7b": ("Qwen2.5-7B shape", QWEN25_7B), "14b": ("Qwen2.5-14B shape", QWEN25_14B),
-          "32b": ("Qwen2.5-32B shape", QWEN25_32B)}
+# the size the reference's own benchmarks run (README.md:39-48 there): Qwen2.5-0.5B, tied embeddings
+QWEN25_05B = dict(QWEN25_7B, hidden_size=896, num_hidden_layers=24, num_attention_heads=14, num_key_value_heads=2, head_dim=64,
+                  intermediate_size=4864, vocab_size=151936, tie_word_embeddings=True, max_position_embeddings=32768)
+SHAPES = {"0.5b": ("Qwen2.5-0.5B shape", QWEN25_05B), "7b": ("Qwen2.5-7B shape", QWEN25_7B),
+          "14b": ("Qwen2.5-14B shape", QWEN25_14B), "32b": ("Qwen2.5-32B shape", QWEN25_32B)}
 
 
 def gemm_params_per_layer(c) -> int:
