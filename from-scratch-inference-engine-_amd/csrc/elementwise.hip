@@ -210,15 +210,21 @@ void launch_rmsnorm(const NormCall& c) {
                          reinterpret_cast<uintptr_t>(c.weight) % 16 == 0 && reinterpret_cast<uintptr_t>(c.delta) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(c.out) % 16 == 0 && c.part_stride % 4 == 0 &&
                          (c.n_parts == 0 || c.n_parts == 2 || c.n_parts == 4 || c.n_parts == 8);
+    // a thread holds `iters` quads of the row: as many as the row needs, so that a row of 5,120
+    // values asks for five quads a thread and not for eight of which three repeat the last one
     const int per_iter = kThreads * 4;
-    if (aligned && c.hidden >= 4 && c.hidden <= per_iter) {
-        launch_rmsnorm_vec<T, 1>(c);
-    } else if (aligned && c.hidden <= 2 * per_iter && c.hidden >= 4) {
-        launch_rmsnorm_vec<T, 2>(c);
-    } else if (aligned && c.hidden <= 4 * per_iter && c.hidden >= 4) {
-        launch_rmsnorm_vec<T, 4>(c);
-    } else if (aligned && c.hidden <= 8 * per_iter && c.hidden >= 4) {
-        launch_rmsnorm_vec<T, 8>(c);
+    const int iters = (c.hidden + per_iter - 1) / per_iter;
+    if (aligned && c.hidden >= 4 && iters <= 8) {
+        switch (iters) {
+            case 1: launch_rmsnorm_vec<T, 1>(c); break;
+            case 2: launch_rmsnorm_vec<T, 2>(c); break;
+            case 3: launch_rmsnorm_vec<T, 3>(c); break;
+            case 4: launch_rmsnorm_vec<T, 4>(c); break;
+            case 5: launch_rmsnorm_vec<T, 5>(c); break;
+            case 6: launch_rmsnorm_vec<T, 6>(c); break;
+            case 7: launch_rmsnorm_vec<T, 7>(c); break;
+            default: launch_rmsnorm_vec<T, 8>(c); break;
+        }
     } else {
         rmsnorm_kernel<T><<<c.n_rows, kThreads, 0, c.stream>>>(c.residual, static_cast<const T*>(c.delta), c.weight,
                                                              static_cast<T*>(c.out), c.rows, c.hidden, c.eps,

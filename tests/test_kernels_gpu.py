@@ -209,6 +209,21 @@ def test_gemm_mfma_wide_refuses_what_it_does_not_take(ops):
         ops.gemm_mfma_wide(x.cuda(), w.cuda())
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_at_every_row_length_class(ops, dtype):
+    """A thread of the vector kernel holds one to eight quads of the row (1,024 values a quad):
+    row lengths in every class, at its upper edge and just inside it, with eight partial sums."""
+    for hidden in (1024, 1028, 2560, 3072, 3584, 5120, 5124, 6144, 7000, 8192):
+        x, g = rnd((2, hidden), 40), rnd((hidden,), 41) + 1.0
+        parts = rnd((8, 2, hidden), 42)
+        summed = x + parts.double().sum(0).float()
+        want = plain.rms_norm(summed, g, 1e-6)
+        res = x.clone().cuda()
+        out = ops.rmsnorm(res, g.cuda(), 1e-6, dtype, delta=parts.cuda(), write_back=True).float().cpu()
+        assert (res.cpu() - summed).abs().max() <= 1e-5 * summed.abs().max(), hidden
+        assert (out - want).abs().max() <= tol(dtype, want), hidden
+
+
 def test_rmsnorm_adds_partial_sums_at_odd_sizes(ops):
     """Sizes the vector kernel does not take: hidden not a multiple of 4 and larger than its registers hold."""
     for hidden, n_parts in [(102, 2), (9001 * 4, 4), (4099, 8)]:
