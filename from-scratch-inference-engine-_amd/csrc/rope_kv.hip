@@ -112,6 +112,92 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_kernel(
     }
 }
 
+// Four values in 16 (float32) or 8 (bfloat16) bytes.
+template <typename T>
+struct Quad;
+template <>
+struct Quad<float> {
+    static __device__ __forceinline__ float4 load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+    static __device__ __forceinline__ void store(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+};
+template <>
+struct Quad<bf16_t> {
+    static __device__ __forceinline__ float4 load(const bf16_t* p) {
+        const uint2 w = *reinterpret_cast<const uint2*>(p);
+        return float4{__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                      __uint_as_float(w.y & 0xffff0000u)};
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, float4 v) {
+        *reinterpret_cast<uint2*>(p) = uint2{pack2_bf16(v.x, v.y), pack2_bf16(v.z, v.w)};
+    }
+};
+
+// The same work with the cosines and sines read from the step's table [T][head_dim / 2][2] and four
+// pairs a thread: no trigonometry, 8- and 16-byte accesses.  The whole head is rotated; head_dim is
+// a multiple of 8.  One block per token.
+template <typename T, bool HAS_BIAS>
+__global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
+    T* __restrict__ qkv, const float* __restrict__ cos_sin, const int32_t* __restrict__ slots,
+    const float* __restrict__ bias, T* __restrict__ k_pool, T* __restrict__ v_pool, int n_heads, int n_kv,
+    int head_dim, int page_size, int write_kv, int64_t pool_slots) {
+    const int t = blockIdx.x;
+    const int half = head_dim / 2;
+    const int q_dim = n_heads * head_dim;
+    const int kv_dim = n_kv * head_dim;
+    T* row = qkv + static_cast<int64_t>(t) * (q_dim + 2 * kv_dim);
+    int slot = write_kv ? slots[t] : -1;
+    if (slot >= pool_slots) slot = -1;
+    const int64_t page = slot >= 0 ? slot / page_size : 0;
+    const int off = slot >= 0 ? slot % page_size : 0;
+
+    if (slot >= 0) {
+        const T* v = row + q_dim + kv_dim;
+        for (int idx = threadIdx.x * 4; idx < kv_dim; idx += kThreads * 4) {
+            const int kvh = idx / head_dim;
+            const int d = idx - kvh * head_dim;
+            float4 x = Quad<T>::load(v + idx);
+            if (HAS_BIAS) {
+                const float4 b = *reinterpret_cast<const float4*>(bias + q_dim + kv_dim + idx);
+                x = float4{x.x + b.x, x.y + b.y, x.z + b.z, x.w + b.w};
+            }
+            T* dst = v_pool + ((page * n_kv + kvh) * head_dim + d) * page_size + off;
+            dst[0] = from_float<T>(x.x);
+            dst[page_size] = from_float<T>(x.y);
+            dst[2 * page_size] = from_float<T>(x.z);
+            dst[3 * page_size] = from_float<T>(x.w);
+        }
+    }
+
+    const float4* cs = reinterpret_cast<const float4*>(cos_sin + static_cast<int64_t>(t) * head_dim);  // two pairs each
+    const int quads = half / 4;
+    const int n_units = (n_heads + n_kv) * quads;
+#pragma unroll 2
+    for (int u = threadIdx.x; u < n_units; u += kThreads) {
+        const int h = u / quads;
+        const int i = (u - h * quads) * 4;
+        T* head = row + h * head_dim;
+        float4 a1 = Quad<T>::load(head + i), a2 = Quad<T>::load(head + i + half);
+        if (HAS_BIAS) {
+            const float4 b1 = *reinterpret_cast<const float4*>(bias + h * head_dim + i);
+            const float4 b2 = *reinterpret_cast<const float4*>(bias + h * head_dim + i + half);
+            a1 = float4{a1.x + b1.x, a1.y + b1.y, a1.z + b1.z, a1.w + b1.w};
+            a2 = float4{a2.x + b2.x, a2.y + b2.y, a2.z + b2.z, a2.w + b2.w};
+        }
+        const float4 c01 = cs[i / 2], c23 = cs[i / 2 + 1];  // (cos, sin) of pairs i, i + 1 and i + 2, i + 3
+        const float4 r1{a1.x * c01.x - a2.x * c01.y, a1.y * c01.z - a2.y * c01.w, a1.z * c23.x - a2.z * c23.y,
+                        a1.w * c23.z - a2.w * c23.w};
+        const float4 r2{a2.x * c01.x + a1.x * c01.y, a2.y * c01.z + a1.y * c01.w, a2.z * c23.x + a1.z * c23.y,
+                        a2.w * c23.z + a1.w * c23.w};
+        Quad<T>::store(head + i, r1);
+        Quad<T>::store(head + i + half, r2);
+        if (h >= n_heads && slot >= 0) {
+            T* dst = k_pool + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+            Quad<T>::store(dst + i, r1);
+            Quad<T>::store(dst + i + half, r2);
+        }
+    }
+}
+
 // table[t][i] = (cos, sin) of positions[t] * inv_freq[i]: the angles of a step are the same in
 // every layer, so a step computes them once and the layers' kernels read them.
 __global__ void rope_table_kernel(const int32_t* __restrict__ positions, const double* __restrict__ inv_freq,
@@ -164,5 +250,34 @@ extern "C" int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int
     }
 #undef FSIE_ROPE_LAUNCH
     FSIE_CHECK_LAUNCH("rope_kv_write");
+    return 0;
+}
+
+// The rotation with cosines and sines from `cos_sin` ([n_tokens, head_dim / 2, 2] float32, made by
+// fsie_rope_table): the whole head is rotated, head_dim a multiple of 8.
+extern "C" int fsie_rope_kv_write_table(void* qkv, const float* cos_sin, const int32_t* slots, const float* bias,
+                                        void* k_pool, void* v_pool, int n_tokens, int n_heads, int n_kv, int head_dim,
+                                        int page_size, int64_t pool_slots, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv > 0, "rope_kv_write_table: bad sizes");
+    FSIE_REQUIRE(head_dim > 0 && head_dim % 8 == 0, "rope_kv_write_table: head_dim %d must be a multiple of 8", head_dim);
+    FSIE_REQUIRE(cos_sin && reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0, "rope_kv_write_table: no aligned table");
+    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && (!bias || reinterpret_cast<uintptr_t>(bias) % 16 == 0) &&
+                     (!k_pool || reinterpret_cast<uintptr_t>(k_pool) % 16 == 0),
+                 "rope_kv_write_table: operands must be 16-byte aligned");
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "rope_kv_write_table: unknown dtype %d", dtype);
+    const int write_kv = (k_pool && v_pool && slots) ? 1 : 0;
+    FSIE_REQUIRE(!write_kv || (page_size > 0 && pool_slots > 0), "rope_kv_write_table: bad page geometry");
+    if (n_tokens == 0) return 0;
+#define FSIE_ROPE_LAUNCH(T, B)                                                                                  \
+    rope_kv_write_table_kernel<T, B><<<n_tokens, kThreads, 0, stream>>>(                                        \
+        static_cast<T*>(qkv), cos_sin, slots, bias, static_cast<T*>(k_pool), static_cast<T*>(v_pool), n_heads,  \
+        n_kv, head_dim, page_size, write_kv, pool_slots)
+    if (dtype == FSIE_F32) {
+        if (bias) FSIE_ROPE_LAUNCH(float, true); else FSIE_ROPE_LAUNCH(float, false);
+    } else {
+        if (bias) FSIE_ROPE_LAUNCH(bf16_t, true); else FSIE_ROPE_LAUNCH(bf16_t, false);
+    }
+#undef FSIE_ROPE_LAUNCH
+    FSIE_CHECK_LAUNCH("rope_kv_write_table");
     return 0;
 }

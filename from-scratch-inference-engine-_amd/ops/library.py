@@ -33,6 +33,8 @@ _SIGNATURES = {
     "fsie_bias_add": ([_P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_rope_kv_write": ([_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
                             c_int, _P], c_int),
+    "fsie_rope_kv_write_table": ([_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, _P],
+                                 c_int),
     "fsie_gemm": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_gemm_mfma_skinny": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_gemm_mfma_skinny_rope": ([_P, _P, _P, _P, c_int, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int,

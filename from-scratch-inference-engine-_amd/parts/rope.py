@@ -43,23 +43,30 @@ class RotaryEncoding(PositionEncoding):
         table = np.power(np.float64(self.theta), -2.0 * i / self.rotary_dim)
         self.inv_freq = torch.from_numpy(table).to(device)
 
+    def table(self, ctx) -> torch.Tensor:
+        """The cosines and sines of this step's positions: the same in every layer, made by the
+        first one that asks."""
+        key = ("rope cos/sin", self.theta, self.rotary_dim)
+        table = ctx.memo.get(key)
+        if table is None:
+            table = ctx.memo[key] = ops.rope_table(ctx.positions, self.inv_freq)
+        return table
+
     def apply(self, qkv, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore], bias=None) -> None:
+        cos_sin = self.table(ctx) if self.rotary_dim == head_dim and head_dim % 8 == 0 else None
         if store is None:
-            ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, bias=bias)
+            ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, bias=bias, cos_sin=cos_sin)
         else:
             ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, slots=store.slots,
-                              k_pool=store.k_pool, v_pool=store.v_pool, page_size=store.page_size, bias=bias)
+                              k_pool=store.k_pool, v_pool=store.v_pool, page_size=store.page_size, bias=bias,
+                              cos_sin=cos_sin)
 
     def project(self, x, weight, bias, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore]):
         """For a few rows of bfloat16 (decoding) the projection's own epilogue rotates and stores."""
         if (x.dtype != torch.bfloat16 or not 0 < x.shape[0] <= GEMM_MFMA_SKINNY_BEST_M or x.shape[1] % 8
                 or head_dim % 16 or self.rotary_dim != head_dim):
             return None
-        # the cosines and sines of this step's positions: the same in every layer, made by the first
-        key = ("rope cos/sin", self.theta, self.rotary_dim)
-        table = ctx.memo.get(key)
-        if table is None:
-            table = ctx.memo[key] = ops.rope_table(ctx.positions, self.inv_freq)
+        table = self.table(ctx)
         if store is None:
             return ops.gemm_mfma_skinny_rope(x, weight, bias, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq,
                                              cos_sin=table)

@@ -73,8 +73,9 @@ def test_swiglu_and_adds(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads, kv, hd, theta", [(14, 2, 64, 1e6), (3, 3, 48, 1e4), (5, 1, 256, 5e5)])
-def test_rope_and_cache_write(ops, dtype, heads, kv, hd, theta):
+@pytest.mark.parametrize("from_table", [False, True])  # the angles computed by the kernel, or read from the step's table
+@pytest.mark.parametrize("heads, kv, hd, theta", [(14, 2, 64, 1e6), (3, 3, 48, 1e4), (5, 1, 256, 5e5), (7, 2, 24, 3e4)])
+def test_rope_and_cache_write(ops, dtype, from_table, heads, kv, hd, theta):
     t, page, pages = 9, 4, 11
     width = (heads + 2 * kv) * hd
     qkv, bias = rnd((t, width), 9, dtype), rnd((width,), 10)
@@ -84,8 +85,15 @@ def test_rope_and_cache_write(ops, dtype, heads, kv, hd, theta):
     k_pool = torch.zeros((pages, kv, page, hd), dtype=dtype)
     v_pool = torch.zeros((pages, kv, hd, page), dtype=dtype)
     dq, dk, dv = qkv.clone().cuda(), k_pool.cuda(), v_pool.cuda()
+    table = ops.rope_table(pos.cuda(), inv.cuda()) if from_table else None
     ops.rope_kv_write(dq, pos.cuda(), heads, kv, hd, inv.cuda(), slots=slots.cuda(), k_pool=dk, v_pool=dv,
-                      page_size=page, bias=bias.cuda())
+                      page_size=page, bias=bias.cuda(), cos_sin=table)
+    if from_table:  # without a bias and without a cache as well
+        alone = qkv.clone().cuda()
+        ops.rope_kv_write(alone, pos.cuda(), heads, kv, hd, inv.cuda(), cos_sin=table)
+        want = plain.rope(qkv.float()[:, :heads * hd], heads, hd, theta, pos.tolist())
+        assert (alone.float().cpu()[:, :heads * hd] - want).abs().max() <= tol(dtype, want, f32=2e-6)
+        assert torch.equal(alone.cpu()[:, (heads + kv) * hd:], qkv[:, (heads + kv) * hd:])
     full = qkv.float() + bias
     q_ref = plain.rope(full[:, :heads * hd], heads, hd, theta, pos.tolist())
     k_ref = plain.rope(full[:, heads * hd:(heads + kv) * hd], kv, hd, theta, pos.tolist())
