@@ -134,66 +134,106 @@ struct Quad<bf16_t> {
 
 // The same work with the cosines and sines read from the step's table [T][head_dim / 2][2] and four
 // pairs a thread: no trigonometry, 8- and 16-byte accesses.  The whole head is rotated; head_dim is
-// a multiple of 8.  One block per token.
-template <typename T, bool HAS_BIAS>
+// a multiple of 8.  A block takes TOK consecutive tokens: 1, or 8 for long batches (prompt portions).
+// Values lie transposed in a page, [head_dim][slot]: a token alone writes 2 bytes per dimension, and
+// the tokens of one 32-byte run would come from blocks on different dies, each of which would hand
+// its bytes of the run to memory separately.  Eight tokens whose slots are consecutive and start at
+// a multiple of 8 (a portion of a prompt) write 16 bytes per dimension at once.
+template <typename T, bool HAS_BIAS, int TOK>
 __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
     T* __restrict__ qkv, const float* __restrict__ cos_sin, const int32_t* __restrict__ slots,
-    const float* __restrict__ bias, T* __restrict__ k_pool, T* __restrict__ v_pool, int n_heads, int n_kv,
-    int head_dim, int page_size, int write_kv, int64_t pool_slots) {
-    const int t = blockIdx.x;
+    const float* __restrict__ bias, T* __restrict__ k_pool, T* __restrict__ v_pool, int n_tokens, int n_heads,
+    int n_kv, int head_dim, int page_size, int write_kv, int64_t pool_slots) {
+    const int t0 = blockIdx.x * TOK;
+    const int n_here = min(TOK, n_tokens - t0);
     const int half = head_dim / 2;
     const int q_dim = n_heads * head_dim;
     const int kv_dim = n_kv * head_dim;
-    T* row = qkv + static_cast<int64_t>(t) * (q_dim + 2 * kv_dim);
-    int slot = write_kv ? slots[t] : -1;
-    if (slot >= pool_slots) slot = -1;
-    const int64_t page = slot >= 0 ? slot / page_size : 0;
-    const int off = slot >= 0 ? slot % page_size : 0;
+    const int width = q_dim + 2 * kv_dim;
+    int slot[TOK];
+#pragma unroll
+    for (int j = 0; j < TOK; ++j) {
+        slot[j] = (write_kv && j < n_here) ? slots[t0 + j] : -1;
+        if (slot[j] >= pool_slots) slot[j] = -1;
+    }
 
-    if (slot >= 0) {
-        const T* v = row + q_dim + kv_dim;
-        for (int idx = threadIdx.x * 4; idx < kv_dim; idx += kThreads * 4) {
+    // ---- values
+    bool run = TOK == 8 && n_here == 8 && slot[0] >= 0 && slot[0] % 8 == 0 && page_size % 8 == 0;
+#pragma unroll
+    for (int j = 1; j < TOK; ++j) run = run && slot[j] == slot[0] + j;
+    if (TOK == 8 && run) {
+        const int64_t page = slot[0] / page_size;
+        const int off = slot[0] % page_size;
+        for (int idx = threadIdx.x; idx < kv_dim; idx += kThreads) {  // lanes over the dimensions: rows read whole
             const int kvh = idx / head_dim;
             const int d = idx - kvh * head_dim;
-            float4 x = Quad<T>::load(v + idx);
-            if (HAS_BIAS) {
-                const float4 b = *reinterpret_cast<const float4*>(bias + q_dim + kv_dim + idx);
-                x = float4{x.x + b.x, x.y + b.y, x.z + b.z, x.w + b.w};
-            }
+            const float b = HAS_BIAS ? bias[q_dim + kv_dim + idx] : 0.f;
+            float x[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                x[j] = to_float(qkv[static_cast<int64_t>(t0 + j) * width + q_dim + kv_dim + idx]) + b;
             T* dst = v_pool + ((page * n_kv + kvh) * head_dim + d) * page_size + off;
-            dst[0] = from_float<T>(x.x);
-            dst[page_size] = from_float<T>(x.y);
-            dst[2 * page_size] = from_float<T>(x.z);
-            dst[3 * page_size] = from_float<T>(x.w);
+            Quad<T>::store(dst, float4{x[0], x[1], x[2], x[3]});
+            Quad<T>::store(dst + 4, float4{x[4], x[5], x[6], x[7]});
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TOK; ++j) {
+            if (slot[j] < 0) continue;
+            const int64_t page = slot[j] / page_size;
+            const int off = slot[j] % page_size;
+            const T* v = qkv + static_cast<int64_t>(t0 + j) * width + q_dim + kv_dim;
+            for (int idx = threadIdx.x * 4; idx < kv_dim; idx += kThreads * 4) {
+                const int kvh = idx / head_dim;
+                const int d = idx - kvh * head_dim;
+                float4 x = Quad<T>::load(v + idx);
+                if (HAS_BIAS) {
+                    const float4 b = *reinterpret_cast<const float4*>(bias + q_dim + kv_dim + idx);
+                    x = float4{x.x + b.x, x.y + b.y, x.z + b.z, x.w + b.w};
+                }
+                T* dst = v_pool + ((page * n_kv + kvh) * head_dim + d) * page_size + off;
+                dst[0] = from_float<T>(x.x);
+                dst[page_size] = from_float<T>(x.y);
+                dst[2 * page_size] = from_float<T>(x.z);
+                dst[3 * page_size] = from_float<T>(x.w);
+            }
         }
     }
 
-    const float4* cs = reinterpret_cast<const float4*>(cos_sin + static_cast<int64_t>(t) * head_dim);  // two pairs each
+    // ---- q and k heads: unit u of a token = four pairs of one head; the tokens of the block in turn
     const int quads = half / 4;
     const int n_units = (n_heads + n_kv) * quads;
-#pragma unroll 2
     for (int u = threadIdx.x; u < n_units; u += kThreads) {
         const int h = u / quads;
         const int i = (u - h * quads) * 4;
-        T* head = row + h * head_dim;
-        float4 a1 = Quad<T>::load(head + i), a2 = Quad<T>::load(head + i + half);
+        float4 b1{0.f, 0.f, 0.f, 0.f}, b2{0.f, 0.f, 0.f, 0.f};
         if (HAS_BIAS) {
-            const float4 b1 = *reinterpret_cast<const float4*>(bias + h * head_dim + i);
-            const float4 b2 = *reinterpret_cast<const float4*>(bias + h * head_dim + i + half);
+            b1 = *reinterpret_cast<const float4*>(bias + h * head_dim + i);
+            b2 = *reinterpret_cast<const float4*>(bias + h * head_dim + i + half);
+        }
+#pragma unroll
+        for (int j = 0; j < TOK; ++j) {
+            if (j >= n_here) break;
+            const int t = t0 + j;
+            T* head = qkv + static_cast<int64_t>(t) * width + h * head_dim;
+            float4 a1 = Quad<T>::load(head + i), a2 = Quad<T>::load(head + i + half);
             a1 = float4{a1.x + b1.x, a1.y + b1.y, a1.z + b1.z, a1.w + b1.w};
             a2 = float4{a2.x + b2.x, a2.y + b2.y, a2.z + b2.z, a2.w + b2.w};
-        }
-        const float4 c01 = cs[i / 2], c23 = cs[i / 2 + 1];  // (cos, sin) of pairs i, i + 1 and i + 2, i + 3
-        const float4 r1{a1.x * c01.x - a2.x * c01.y, a1.y * c01.z - a2.y * c01.w, a1.z * c23.x - a2.z * c23.y,
-                        a1.w * c23.z - a2.w * c23.w};
-        const float4 r2{a2.x * c01.x + a1.x * c01.y, a2.y * c01.z + a1.y * c01.w, a2.z * c23.x + a1.z * c23.y,
-                        a2.w * c23.z + a1.w * c23.w};
-        Quad<T>::store(head + i, r1);
-        Quad<T>::store(head + i + half, r2);
-        if (h >= n_heads && slot >= 0) {
-            T* dst = k_pool + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
-            Quad<T>::store(dst + i, r1);
-            Quad<T>::store(dst + i + half, r2);
+            const float4* cs = reinterpret_cast<const float4*>(cos_sin + static_cast<int64_t>(t) * head_dim);
+            const float4 c01 = cs[i / 2], c23 = cs[i / 2 + 1];  // (cos, sin) of pairs i, i + 1 and i + 2, i + 3
+            const float4 r1{a1.x * c01.x - a2.x * c01.y, a1.y * c01.z - a2.y * c01.w, a1.z * c23.x - a2.z * c23.y,
+                            a1.w * c23.z - a2.w * c23.w};
+            const float4 r2{a2.x * c01.x + a1.x * c01.y, a2.y * c01.z + a1.y * c01.w, a2.z * c23.x + a1.z * c23.y,
+                            a2.w * c23.z + a1.w * c23.w};
+            Quad<T>::store(head + i, r1);
+            Quad<T>::store(head + i + half, r2);
+            if (h >= n_heads && slot[j] >= 0) {
+                const int64_t page = slot[j] / page_size;
+                const int off = slot[j] % page_size;
+                T* dst = k_pool + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+                Quad<T>::store(dst + i, r1);
+                Quad<T>::store(dst + i + half, r2);
+            }
         }
     }
 }
@@ -268,10 +308,18 @@ extern "C" int fsie_rope_kv_write_table(void* qkv, const float* cos_sin, const i
     const int write_kv = (k_pool && v_pool && slots) ? 1 : 0;
     FSIE_REQUIRE(!write_kv || (page_size > 0 && pool_slots > 0), "rope_kv_write_table: bad page geometry");
     if (n_tokens == 0) return 0;
-#define FSIE_ROPE_LAUNCH(T, B)                                                                                  \
-    rope_kv_write_table_kernel<T, B><<<n_tokens, kThreads, 0, stream>>>(                                        \
-        static_cast<T*>(qkv), cos_sin, slots, bias, static_cast<T*>(k_pool), static_cast<T*>(v_pool), n_heads,  \
-        n_kv, head_dim, page_size, write_kv, pool_slots)
+    // eight tokens a block where there are enough blocks left to fill the device
+#define FSIE_ROPE_LAUNCH(T, B)                                                                                    \
+    do {                                                                                                          \
+        if (n_tokens >= 1024)                                                                                     \
+            rope_kv_write_table_kernel<T, B, 8><<<(n_tokens + 7) / 8, kThreads, 0, stream>>>(                     \
+                static_cast<T*>(qkv), cos_sin, slots, bias, static_cast<T*>(k_pool), static_cast<T*>(v_pool),     \
+                n_tokens, n_heads, n_kv, head_dim, page_size, write_kv, pool_slots);                              \
+        else                                                                                                      \
+            rope_kv_write_table_kernel<T, B, 1><<<n_tokens, kThreads, 0, stream>>>(                               \
+                static_cast<T*>(qkv), cos_sin, slots, bias, static_cast<T*>(k_pool), static_cast<T*>(v_pool),     \
+                n_tokens, n_heads, n_kv, head_dim, page_size, write_kv, pool_slots);                              \
+    } while (0)
     if (dtype == FSIE_F32) {
         if (bias) FSIE_ROPE_LAUNCH(float, true); else FSIE_ROPE_LAUNCH(float, false);
     } else {

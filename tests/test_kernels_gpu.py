@@ -117,6 +117,69 @@ def test_rope_and_cache_write(ops, dtype, from_table, heads, kv, hd, theta):
     assert (dq.float().cpu()[:, :(heads + kv) * hd] - full[:, :(heads + kv) * hd]).abs().max() <= tol(dtype, full)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page", [16, 8, 4])
+def test_rope_from_table_on_a_long_batch(ops, dtype, page):
+    """From 1,024 tokens on a block takes eight tokens and writes the values of eight consecutive
+    slots that start at a multiple of 8 with one store per dimension.  A batch of 1,029 tokens:
+    portions whose slots run on (aligned and not), single tokens anywhere, tokens that are not
+    stored, a tail of five; every slot of the pools is compared."""
+    heads, kv, hd, theta = 4, 2, 32, 1e4
+    t = 1029
+    pages = 2 * t // page + 8
+    g = torch.Generator().manual_seed(77 + page)
+    slots = torch.full((t,), -1, dtype=torch.int32)
+    free = torch.randperm(pages, generator=g).tolist()
+    i = 0
+    while i < t:
+        kind = int(torch.randint(0, 4, (1,), generator=g))
+        if kind == 0:                      # a portion: consecutive slots over whole pages, from a random offset
+            n = min(int(torch.randint(5, 90, (1,), generator=g)), t - i)
+            off = int(torch.randint(0, page, (1,), generator=g))
+            need = -(-(off + n) // page)
+            mine = [free.pop() for _ in range(need)]
+            for j in range(n):
+                slots[i + j] = mine[(off + j) // page] * page + (off + j) % page
+            i += n
+        elif kind == 1:                    # a decoded token
+            slots[i] = free.pop() * page + int(torch.randint(0, page, (1,), generator=g))
+            i += 1
+        elif kind == 2:                    # not stored
+            i += 1
+        else:                              # eight aligned ones
+            n = min(8, t - i)
+            p0 = free.pop() if page >= 8 else None
+            for j in range(n):
+                slots[i + j] = (p0 * page + j) if p0 is not None else free.pop() * page
+            i += n
+    width = (heads + 2 * kv) * hd
+    qkv, bias = rnd((t, width), 90, dtype), rnd((width,), 91)
+    pos = torch.randint(0, 5000, (t,), generator=g, dtype=torch.int32)
+    inv = torch.tensor([theta ** (-2.0 * k / hd) for k in range(hd // 2)], dtype=torch.float64)
+    dq = qkv.clone().cuda()
+    dk = torch.zeros((pages, kv, page, hd), dtype=dtype).cuda()
+    dv = torch.zeros((pages, kv, hd, page), dtype=dtype).cuda()
+    table = ops.rope_table(pos.cuda(), inv.cuda())
+    ops.rope_kv_write(dq, pos.cuda(), heads, kv, hd, inv.cuda(), slots=slots.cuda(), k_pool=dk, v_pool=dv,
+                      page_size=page, bias=bias.cuda(), cos_sin=table)
+    full = qkv.float() + bias
+    q_ref = plain.rope(full[:, :heads * hd], heads, hd, theta, pos.tolist())
+    k_ref = plain.rope(full[:, heads * hd:(heads + kv) * hd], kv, hd, theta, pos.tolist())
+    v_ref = full[:, (heads + kv) * hd:]
+    got = dq.float().cpu()
+    assert (got[:, :heads * hd] - q_ref).abs().max() <= tol(dtype, q_ref, f32=2e-6)
+    assert (got[:, heads * hd:(heads + kv) * hd] - k_ref).abs().max() <= tol(dtype, k_ref, f32=2e-6)
+    want_k = torch.zeros(pages * page, kv * hd)
+    want_v = torch.zeros(pages * page, kv * hd)
+    stored = slots >= 0
+    want_k[slots[stored].long()] = k_ref[stored]
+    want_v[slots[stored].long()] = v_ref[stored]
+    kp = dk.float().cpu().permute(0, 2, 1, 3).reshape(pages * page, kv * hd)   # [slot][kv head][dim]
+    vp = dv.float().cpu().permute(0, 3, 1, 2).reshape(pages * page, kv * hd)
+    assert (kp - want_k).abs().max() <= tol(dtype, k_ref, f32=2e-6)
+    assert (vp - want_v).abs().max() <= tol(dtype, v_ref, f32=2e-6)
+
+
 @pytest.mark.parametrize("m, n, k", [(1, 4864, 896), (5, 151, 100), (8, 1000, 4864), (37, 300, 129), (130, 896, 1000)])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm(ops, dtype, m, n, k):
