@@ -16,7 +16,7 @@ class Linear:
 
     float32: the engine's own kernels only (true 32-bit products and sums).
     bfloat16: up to 16 rows (decoding) the engine's matrix-core kernel that streams the weight
-    once; its sibling that shares x through LDS for float32 results of 8 to 64 rows (the logits)
+    once; its sibling that shares x through LDS for float32 results of 8 to 64 rows (the logits; beyond 64 rows the library with a float32 result)
     and for the residual projections (``for_residual``: 17 to 64 rows, and any number where K is
     long); everything else the library product
     (hipBLASLt through torch, where the reference's engine calls cuBLAS) with float32
@@ -43,6 +43,13 @@ class Linear:
             # logits of 8 to 64 rows: x shared through LDS (N = 152064, K = 3584 on MI355X: 200
             # against 215 us at 8 rows, 242 against 486 at 64)
             return ops.gemm_mfma_wide(x, w)
+        if (wants_f32 and bias is None and m > GEMM_MFMA_SKINNY_MAX_M and out_dtype == torch.float32
+                and self.in_features % 8 == 0 and self.out_features % 8 == 0):
+            # logits of more rows than the engine's kernels take (a decode batch beyond 64, a replay
+            # that wants every position): the library with a float32 result (N = 152064, K = 3584
+            # on MI355X at 256 rows: 0.38 ms; the engine's 64-row kernel four times 0.96, its tiled
+            # float32 kernel 7)
+            return library_mm(x, w, float32_result=True)
         if self.in_features % 8 == 0 and m <= (GEMM_MFMA_SKINNY_MAX_M if wants_f32 else GEMM_MFMA_SKINNY_BEST_M):
             return ops.gemm_mfma_skinny(x, w, bias, out_dtype=out_dtype)
         if m <= GEMM_SKINNY_MAX_M or wants_f32 or self.in_features % 8 or self.out_features % 8:
