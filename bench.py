@@ -80,8 +80,10 @@ def other_workload(args, cfg, model, shape_name, layers, full_layers, page) -> i
         engine = Engine(model, block_size=page, num_blocks=args.requests * -(-longest // page) + 64,
                         max_batch=args.requests, max_tokens_per_step=budget)
         record = None
-        for rep in range(2):  # the first pass pays the graph captures and the library's kernel selection
-            lens = torch.randint(args.min_prompt, args.max_prompt + 1, (args.requests,), generator=gen).tolist()
+        # the same lengths in both passes: the first pays the graph captures and the library's kernel
+        # selection for every step size they lead to, the second is measured
+        lens = torch.randint(args.min_prompt, args.max_prompt + 1, (args.requests,), generator=gen).tolist()
+        for rep in range(2):
             prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist() for n in lens]
             torch.cuda.synchronize()
             t0 = time.perf_counter()

@@ -24,12 +24,11 @@ from __future__ import annotations
 
 import gc
 import weakref
-from types import SimpleNamespace
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from .context import HostBatch, StepEntry, build_context
+from .context import HostBatch, StepEntry, build_context, filler_entry
 
 PAGE_BUCKET = 32  # block-table widths are rounded up to this many pages
 CAPTURE_AFTER = 3  # a shape is captured the n-th time it is asked for (read when a runner is made)
@@ -71,9 +70,8 @@ class DecodeGraphs:
     def filled_up(self, entries: Sequence[StepEntry]) -> List:
         """The entries and, behind them, the rows that pad the batch to a graph's size."""
         runner = self.runner
-        spare = SimpleNamespace(length=0, slot=runner.storage.spare_slot,
-                                tables=[[page] for page in runner.storage.spare_pages])
-        filler = SimpleNamespace(cache=spare, tokens=(0,), want=(0,))
+        filler = filler_entry(runner.storage, 1, runner.manager.page_size)
+        filler.want = (0,)
         return list(entries) + [filler] * (padded_rows(len(entries)) - len(entries))
 
     def shape_of(self, entries: Sequence[StepEntry]) -> Optional[dict]:

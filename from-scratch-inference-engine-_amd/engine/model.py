@@ -23,7 +23,7 @@ from ..models.spec import ModelSpec
 from ..parts.base import HiddenState
 from ..weights.loader import fill_parts, load_weights
 from ..weights.random_init import random_tensor, expected_tensors
-from .context import PinnedStaging, StepContext, StepEntry, build_context
+from .context import PinnedStaging, StepContext, StepEntry, build_context, filler_entry, padded_tokens
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -218,10 +218,20 @@ class Runner:
             if keep:
                 logits = logits.clone()
         else:
-            ctx, _ = build_context(entries, self.manager, self.model.planners, self._staging, self.model.dtype,
+            n_tokens = sum(len(e.tokens) for e in entries)
+            batch = list(entries)
+            if (self.model.dtype == torch.bfloat16 and ops.library_tuning_enabled()
+                    and self.graphs is not None and self.graphs.enabled):
+                # with the library's kernels chosen by timing, a step is filled up to one of the few
+                # row counts that are timed, with the tokens of a request that does not exist (only
+                # for models whose parts all read the step through its device tables, as for graphs)
+                extra = padded_tokens(n_tokens) - n_tokens
+                if extra > 0:
+                    batch.append(filler_entry(self.storage, extra, self.manager.page_size))
+            ctx, _ = build_context(batch, self.manager, self.model.planners, self._staging, self.model.dtype,
                                    self.model.device)
             if feed is not None:
-                ctx.token_ids.copy_(feed)
+                ctx.token_ids[:n_tokens].copy_(feed)
             logits = self.model.forward(ctx, self.storage)
         for e in entries:
             self.manager.commit(e.cache, len(e.tokens))

@@ -446,8 +446,23 @@ def test_prefill_with_the_library_kernel_selection(model_dirs):
         for t in range(3, 0, -1):
             decoded.append(runner.step([StepEntry(c, [s_[-t]], [0]) for c, s_ in zip(caches, seqs)]).float().cpu().numpy())
         assert runner.graphs.captures == 1 and runner.graphs.replays == 2
+        # with the timing on, a step of 107 tokens is filled up to 128 with the tokens of a request
+        # that does not exist: what the real requests get does not change, nor what they decode next
+        from from_scratch_inference_engine_amd.engine.context import padded_tokens
+        assert padded_tokens(70 + 37) == 128
+        runner = Runner(load_model(model_dirs["B"], dtype="bfloat16"), page_size=8, num_pages=40, max_requests=3)
+        pair = [helpers.token_ids(vocab, 71, 870), helpers.token_ids(vocab, 38, 871)]
+        pair_ref = [plain.forward_dir(model_dirs["B"], s_).numpy() for s_ in pair]
+        pc = [runner.manager.open(i) for i in range(2)]
+        filled = runner.step([StepEntry(c, s_[:-1], [len(s_) - 2]) for c, s_ in zip(pc, pair)]).float().cpu().numpy()
+        after = runner.step([StepEntry(c, [s_[-1]], [0]) for c, s_ in zip(pc, pair)]).float().cpu().numpy()
     finally:
         ops.disable_library_tuning()
+    for i, s_ in enumerate(pair):
+        helpers.assert_close_to_plain(filled[i:i + 1], pair_ref[i][len(s_) - 2:len(s_) - 1], "bfloat16",
+                                      f"filled-up step, request {i}")
+        helpers.assert_close_to_plain(after[i:i + 1], pair_ref[i][len(s_) - 1:], "bfloat16",
+                                      f"decoding after a filled-up step, request {i}")
     helpers.assert_close_to_plain(out, ref, "bfloat16", "prefill of 256 rows with library tuning")
     for i in range(5):
         for j in range(3):
