@@ -470,6 +470,49 @@ def test_prefill_with_the_library_kernel_selection(model_dirs):
                                           f"decode batch of 32 with library tuning, request {i} token {j}")
 
 
+def test_graphs_replay_the_librarys_timed_kernels_at_large_layer_sizes():
+    """Two layers of Qwen2.5-7B size (random weights made on the device), the library's kernels
+    chosen by timing: decode batches of 32, 64 and 128 through replayed graphs against eager
+    steps, twelve steps each with other work between the replays.  A library kernel that clears
+    its workspace with a memset node, or one that is not fit for capture in another way, shows as
+    a gross difference on a later replay; the kernels' own rounding stays below a bfloat16 step."""
+    from from_scratch_inference_engine_amd import ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Model, Runner
+    from from_scratch_inference_engine_amd.models import parse_config
+
+    raw = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 3584, "num_hidden_layers": 2,
+           "num_attention_heads": 28, "num_key_value_heads": 4, "head_dim": 128, "intermediate_size": 18944,
+           "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+           "max_position_embeddings": 4096}
+    cfg = parse_config(raw)
+    model = Model.from_random(cfg, seed=5, dtype="bfloat16")
+    gen = torch.Generator().manual_seed(5)
+    ops.enable_library_tuning(max_ms_per_candidate=5, iterations=2)
+    try:
+        for batch in (32, 64, 128):
+            runners = [Runner(model, page_size=16, num_pages=batch * 4 + 8, max_requests=batch, use_graphs=g)
+                       for g in (True, False)]
+            prompts = [torch.randint(0, cfg.vocab_size, (20 + i % 7,), generator=gen).tolist() for i in range(batch)]
+            caches = [[r.manager.open(i) for i in range(batch)] for r in runners]
+            for r, cs in zip(runners, caches):
+                r.step([StepEntry(c, p, []) for c, p in zip(cs, prompts)])
+            feed = torch.randint(0, cfg.vocab_size, (12, batch), generator=gen).tolist()
+            for t in range(12):
+                outs = []
+                for r, cs in zip(runners, caches):
+                    outs.append(r.step([StepEntry(c, [feed[t][i]], [0]) for i, c in enumerate(cs)]).float())
+                    torch.cuda.synchronize()
+                    _ = (torch.randn(128, 128, device="cuda") @ torch.randn(128, 128, device="cuda")).sum().item()
+                assert torch.isfinite(outs[0]).all()
+                worst = ((outs[0] - outs[1]).abs().max() / outs[1].abs().max()).item()
+                assert worst <= 2e-2, f"batch {batch}, step {t}: graphs against eager {worst:.3e}"
+            assert runners[0].graphs.captures == 1 and runners[0].graphs.replays == 11
+            del runners, caches
+    finally:
+        ops.disable_library_tuning()
+
+
 def test_a_dropped_runner_frees_its_graphs_at_once(model_dirs):
     """A runner and its graphs form no reference cycle: dropping the runner destroys the captured
     graphs then, by reference count, not when the collector of cycles next runs.  (A collector run
