@@ -21,6 +21,7 @@ class PageAllocator:
             raise ValueError("PageAllocator: num_pages must be non-negative")
         self._free = list(range(num_pages - 1, -1, -1))
         self._refs = [0] * num_pages
+        self._issued = [0] * num_pages  # how often each page has been handed out
 
     @property
     def num_pages(self) -> int:
@@ -35,6 +36,7 @@ class PageAllocator:
             raise OutOfPages("PageAllocator: out of pages")
         page = self._free.pop()
         self._refs[page] = 1
+        self._issued[page] += 1
         return page
 
     def incref(self, page: int) -> None:
@@ -53,3 +55,12 @@ class PageAllocator:
 
     def ref_count(self, page: int) -> int:
         return self._refs[page]
+
+    @property
+    def pages_issued(self) -> int:
+        """How many times ``allocate`` has handed out a page since the pool was made."""
+        return sum(self._issued)
+
+    def pages_issued_again(self) -> list:
+        """Ids of the pages that have been handed out more than once."""
+        return [p for p, n in enumerate(self._issued) if n > 1]

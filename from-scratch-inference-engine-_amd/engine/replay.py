@@ -9,7 +9,9 @@ Input, one JSON object a line on standard input:
 
 All entries of a step are one batch.  For a step that wants logits, ``<out>/<step>.f32`` holds
 them as little-endian float32 [wanted, vocab] in the order of the entries and of ``want``.
-After every step a line ``done <step>`` is printed and flushed.
+After every step a line ``done <step>`` is printed and flushed.  When the input ends,
+``<out>/cache_stats.json`` says how many pages each group's pool has, how often a page was handed
+out, and how many pages were handed out more than once.
 """
 
 from __future__ import annotations
@@ -74,6 +76,12 @@ def main(argv=None) -> int:
             if rid in live:
                 runner.manager.close(live.pop(rid))
         print(f"done {step}", flush=True)
+    # what the cache manager did, for whoever wants to check that pages were used again
+    stats = {"page_size": page, "groups": [
+        {"pages": a.num_pages, "pages_issued": a.pages_issued, "pages_issued_again": len(a.pages_issued_again()),
+         "free_at_end": a.num_free} for a in runner.manager.allocators],
+        "steps": runner.steps, "tokens": runner.tokens}
+    (out_dir / "cache_stats.json").write_text(json.dumps(stats) + "\n")
     return 0
 
 

@@ -9,7 +9,8 @@ Policy (the reference's, src/engine/engine.cpp:53-178, plus a token budget and p
     not fit blocks those behind it;
   * a step holds at most ``max_tokens_per_step`` tokens: one for every request that has only
     its last token left (decoding), then portions of the remaining prompts, each cut to the
-    budget, to ``prefill_chunk`` and to the pages that are free;
+    budget, to ``prefill_chunk`` and to the pages that are free; no more requests run at once
+    than a step has tokens for, so a decoding request is never left out for want of budget;
   * a request whose next tokens find no free pages is left out of the step; if nothing at all
     fits and more than one request is running, the youngest running request that holds pages is
     preempted: its pages go back, it returns to the head of the waiting queue and later
@@ -101,7 +102,9 @@ class Scheduler:
         if max_batch < 1 or max_tokens_per_step < 1:
             raise ValueError("Scheduler: max_batch and max_tokens_per_step must be positive")
         self.manager = manager
-        self.max_batch = min(max_batch, manager.max_requests)
+        # never more running requests than a step has tokens for: every request that decodes
+        # gets its token in every step, nobody starves behind the budget
+        self.max_batch = min(max_batch, manager.max_requests, max_tokens_per_step)
         self.max_tokens_per_step = max_tokens_per_step
         self.prefill_chunk = prefill_chunk or max_tokens_per_step
         self.max_position = max_position

@@ -470,49 +470,6 @@ def test_prefill_with_the_library_kernel_selection(model_dirs):
                                           f"decode batch of 32 with library tuning, request {i} token {j}")
 
 
-def test_graphs_replay_the_librarys_timed_kernels_at_large_layer_sizes():
-    """Two layers of Qwen2.5-7B size (random weights made on the device), the library's kernels
-    chosen by timing: decode batches of 32, 64 and 128 through replayed graphs against eager
-    steps, twelve steps each with other work between the replays.  A library kernel that clears
-    its workspace with a memset node, or one that is not fit for capture in another way, shows as
-    a gross difference on a later replay; the kernels' own rounding stays below a bfloat16 step."""
-    from from_scratch_inference_engine_amd import ops
-    from from_scratch_inference_engine_amd.engine.context import StepEntry
-    from from_scratch_inference_engine_amd.engine.model import Model, Runner
-    from from_scratch_inference_engine_amd.models import parse_config
-
-    raw = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 3584, "num_hidden_layers": 2,
-           "num_attention_heads": 28, "num_key_value_heads": 4, "head_dim": 128, "intermediate_size": 18944,
-           "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
-           "max_position_embeddings": 4096}
-    cfg = parse_config(raw)
-    model = Model.from_random(cfg, seed=5, dtype="bfloat16")
-    gen = torch.Generator().manual_seed(5)
-    ops.enable_library_tuning(max_ms_per_candidate=5, iterations=2)
-    try:
-        for batch in (32, 64, 128):
-            runners = [Runner(model, page_size=16, num_pages=batch * 4 + 8, max_requests=batch, use_graphs=g)
-                       for g in (True, False)]
-            prompts = [torch.randint(0, cfg.vocab_size, (20 + i % 7,), generator=gen).tolist() for i in range(batch)]
-            caches = [[r.manager.open(i) for i in range(batch)] for r in runners]
-            for r, cs in zip(runners, caches):
-                r.step([StepEntry(c, p, []) for c, p in zip(cs, prompts)])
-            feed = torch.randint(0, cfg.vocab_size, (12, batch), generator=gen).tolist()
-            for t in range(12):
-                outs = []
-                for r, cs in zip(runners, caches):
-                    outs.append(r.step([StepEntry(c, [feed[t][i]], [0]) for i, c in enumerate(cs)]).float())
-                    torch.cuda.synchronize()
-                    _ = (torch.randn(128, 128, device="cuda") @ torch.randn(128, 128, device="cuda")).sum().item()
-                assert torch.isfinite(outs[0]).all()
-                worst = ((outs[0] - outs[1]).abs().max() / outs[1].abs().max()).item()
-                assert worst <= 2e-2, f"batch {batch}, step {t}: graphs against eager {worst:.3e}"
-            assert runners[0].graphs.captures == 1 and runners[0].graphs.replays == 11
-            del runners, caches
-    finally:
-        ops.disable_library_tuning()
-
-
 def test_a_dropped_runner_frees_its_graphs_at_once(model_dirs):
     """A runner and its graphs form no reference cycle: dropping the runner destroys the captured
     graphs then, by reference count, not when the collector of cycles next runs.  (A collector run
@@ -608,3 +565,139 @@ def test_sizes_the_fast_kernels_do_not_take_still_give_right_results(tmp_path, d
             got[i].append(out[at:at + n]); at += n; fed[i] += n
     for i in (0, 1):
         helpers.assert_close_to_plain(torch.cat(got[i]).numpy(), ref[i], dtype, f"odd sizes {dtype} page {page_size} request {i}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_of_thousands_of_tokens_in_portions_of_2048(tmp_path, dtype):
+    """4,600 tokens of the second tiny configuration (its position limit raised) fed in portions
+    of 2,048, 2,048 and 504 tokens, then 40 tokens decoded one by one: long portions behind
+    thousands of cached keys through the attention kernel that shares keys in LDS, a block table
+    of 290 pages, decode items that are split and merged."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    cfg = dict(helpers.TINY_B, max_position_embeddings=8192)
+    d = helpers.make_model_dir(tmp_path / "long", cfg, seed=31)
+    ids = helpers.token_ids(cfg["vocab_size"], 4640, 4640)
+    ref = plain.forward_dir(d, ids).numpy()
+    runner = Runner(load_model(d, dtype=dtype), page_size=16, num_pages=300, max_requests=2)
+    rc = runner.manager.open("long")
+    fed = 0
+    for n in (2048, 2048, 504):
+        want = sorted(set(range(0, n, 97)) | {n - 2, n - 1})
+        out = runner.step([StepEntry(rc, ids[fed:fed + n], want)]).float().cpu().numpy()
+        helpers.assert_close_to_plain(out, ref[[fed + w for w in want]], dtype, f"{dtype} portion at {fed}")
+        fed += n
+    rows = [runner.step([StepEntry(rc, ids[t:t + 1], [0])]).float().cpu().numpy() for t in range(fed, len(ids))]
+    helpers.assert_close_to_plain(np.concatenate(rows), ref[fed:], dtype, f"{dtype} decoding behind 4,600 tokens")
+    runner.manager.close(rc)
+    runner.manager.check_invariants()
+
+
+@pytest.mark.parametrize("run_ahead", [True, False])
+def test_batched_requests_that_meet_their_end_tokens_at_different_steps(llms, model_dirs, run_ahead):
+    """Five requests decode together, one step ahead of the host; each has an end-of-sequence
+    token of its own that the plain greedy continuation meets at another step (one never meets
+    it).  A request that ends has already been run one token too far by the step in flight: that
+    token is dropped, its pages go back, the others go on.  Outputs equal the plain continuation
+    cut at the end token, with and without running ahead; the manager's invariants hold after
+    every step."""
+    from from_scratch_inference_engine_amd import Engine, SamplingParams, SeqStatus
+
+    model = llms[("B", "float32")].model
+    prompts = [helpers.token_ids(509, n, 500 + n) for n in (4, 9, 17, 30, 6)]
+    free = [plain_greedy(model_dirs["B"], p, 14) for p in prompts]
+    eos = [free[0][2], free[1][5], free[2][9], -1, free[4][12]]
+    want = [f[:f.index(e) + 1] if e in f else f for f, e in zip(free, eos)]
+    assert len({len(w) for w in want}) >= 4  # they do end at different steps
+    engine = Engine(model, block_size=8, num_blocks=40, max_batch=8)
+    engine.run_ahead = run_ahead
+    ids = [engine.add_request(p, SamplingParams(temperature=0.0), max_tokens=14, eos_id=e) for p, e in zip(prompts, eos)]
+    steps = 0
+    while engine.has_work():
+        engine.step()
+        engine.runner.manager.check_invariants()
+        steps += 1
+        assert steps < 100
+    assert [engine.output(i) for i in ids] == want
+    assert all(engine.status(i) == SeqStatus.Finished for i in ids)
+    assert engine.free_blocks() == 40 and engine.runner.manager.free_slots == 8
+
+
+def test_more_requests_than_a_step_has_tokens_for(llms, model_dirs):
+    """A token budget smaller than the number of requests asked to run at once: the engine never
+    runs more requests than a step has tokens for, so nobody who decodes is left out of a step;
+    the others wait their turn.  Outputs are the plain continuations."""
+    from from_scratch_inference_engine_amd import Engine, SamplingParams
+
+    model = llms[("A", "float32")].model
+    engine = Engine(model, block_size=4, num_blocks=64, max_batch=6, max_tokens_per_step=4)
+    assert engine.scheduler.max_batch == 4
+    prompts = [helpers.token_ids(256, n, 600 + n) for n in (3, 5, 2, 7, 4, 6)]
+    got = engine.generate_batch(prompts, SamplingParams(temperature=0.0), max_tokens=8)
+    assert got == [plain_greedy(model_dirs["A"], p, 8) for p in prompts]
+    assert engine.free_blocks() == 64
+
+
+def _model_with_one_loud_key(tmp_path, special):
+    """The second tiny configuration with its first layer arranged so that every query gives
+    nearly all of its attention to the keys of one token, wherever it stands: dimension 15 of the
+    key (the slowest-turning rotary pair: the rotation leaves it alone over thousands of positions)
+    reads how much the normed input looks like that token's, and every query head carries a
+    large constant there.  Near-uniform attention, which random weights give, would hide a key
+    that is missed or taken from the wrong page; here the logits move by a whole unit."""
+    cfg = dict(helpers.TINY_B, max_position_embeddings=2048)
+    t = {k: v.float() for k, v in helpers.random_tensors(cfg, 1).items()}
+    n = plain.rms_norm(t["model.embed_tokens.weight"][special][None], t["model.layers.0.input_layernorm.weight"], 1e-5)[0]
+    t["model.layers.0.self_attn.k_proj.weight"][15] = 8.0 * n / (n @ n)
+    t["model.layers.0.self_attn.k_proj.bias"][15] = 0.0
+    for h in range(6):
+        t["model.layers.0.self_attn.q_proj.weight"][h * 32 + 15] = 0.0
+        t["model.layers.0.self_attn.q_proj.bias"][h * 32 + 15] = 40.0
+    return helpers.make_model_dir(tmp_path / "loud", cfg, 1, tensors={k: v.to(torch.bfloat16).contiguous() for k, v in t.items()})
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_the_model_finds_one_far_key_through_its_own_tables(tmp_path, dtype):
+    """Three requests whose loud token stands at position 2, at the last slot of a page and 1,200
+    tokens back: prefilled in portions beside each other's decoded tokens, then decoded together
+    (eagerly and through graphs).  What the step function's tables and the attention plan hand
+    to the kernels decides the logits here."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    special = 100
+    d = _model_with_one_loud_key(tmp_path, special)
+    seqs = []
+    for n, where, seed in ((700, 2, 1), (420, 335, 2), (1500, 287, 3)):
+        ids = [t if t != special else special + 1 for t in helpers.token_ids(509, n, 880 + seed)]
+        ids[where] = special
+        seqs.append(ids)
+    cfg, w = plain.read_config(d), plain.read_weights(d)
+    refs = [plain.forward(cfg, w, ids).numpy() for ids in seqs]
+    # the construction does what it says: without the loud token the later logits are far away
+    quiet = list(seqs[1])
+    quiet[335] = special + 1
+    assert np.abs(plain.forward(cfg, w, quiet).numpy()[400:] - refs[1][400:]).max() > 0.5
+    model = load_model(d, dtype=dtype)
+    for graphs in (False, True):
+        runner = Runner(model, page_size=16, num_pages=200, max_requests=4, use_graphs=graphs)
+        caches = [runner.manager.open(i) for i in range(3)]
+        fed = [0, 0, 0]
+        got = [[], [], []]
+        # portions of different sizes beside each other; request 1 is already decoding while 2 is in its prompt
+        plan = [[(0, 300), (1, 410)], [(0, 392), (1, 1), (2, 700)], [(1, 1), (2, 2)], [(0, 1), (1, 1), (2, 791)]]
+        plan += [[(0, 1), (1, 1), (2, 1)]] * 7
+        for step in plan:
+            entries = [StepEntry(caches[i], seqs[i][fed[i]:fed[i] + n], [n - 1]) for i, n in step]
+            out = runner.step(entries).float().cpu().numpy()
+            for row, (i, n) in enumerate(step):
+                fed[i] += n
+                got[i].append((fed[i] - 1, out[row]))
+        for i in range(3):
+            assert fed[i] == len(seqs[i])
+            pos = [p for p, _ in got[i]]
+            helpers.assert_close_to_plain(np.stack([r for _, r in got[i]]), refs[i][pos], dtype,
+                                          f"{dtype} graphs={graphs} request {i}")

@@ -267,6 +267,54 @@ def test_gemm_mfma_wide(ops, m, n, k, splits, waves):
         assert torch.equal(other.cpu(), out.cpu()), (blocks, wv)
 
 
+def _exact(x, w):
+    """x . w^T in float64 on the device: the exact sums of the bfloat16 products, to float32's last bits."""
+    return (x.cuda().double() @ w.cuda().double().t()).float().cpu()
+
+
+@pytest.mark.parametrize("n, k", [(3584, 18944), (5120, 13824), (5120, 27648), (3584, 3584), (152064, 3584)])
+def test_gemm_mfma_wide_at_the_large_models_shapes(ops, n, k):
+    """The residual projections and the logits at the layer sizes of the 7B, 14B and 32B shapes,
+    with the slices the engine's Linear picks there (K = 18944: seven slices of 2,432 and one of
+    1,920), at 8, 17 and 64 rows."""
+    from from_scratch_inference_engine_amd.parts.linear import Linear
+
+    splits = 1 if n == 152064 else Linear(k, n).wide_splits()
+    assert splits == (1 if n == 152064 else 4 if k == 3584 else 8)
+    w = rnd((n, k), 51, torch.bfloat16, 0.05)
+    for m in (8, 17, 64):
+        x = rnd((m, k), 50 + m, torch.bfloat16)
+        ref = _exact(x, w)
+        out = ops.gemm_mfma_wide(x.cuda(), w.cuda(), splits=splits).cpu()
+        total = out if splits == 1 else out.double().sum(0).float()
+        assert (total - ref).abs().max() <= 2e-5 * ref.abs().max(), (m, n, k)
+
+
+def test_gemm_mfma_skinny_at_the_large_models_shapes(ops):
+    """Logits of 1 and 7 rows at a vocabulary of 152,064; SiLU(gate) * up at the 32B shape's
+    2 x 27,648 rows of 5,120; the output projection's partial sums at hidden 5,120."""
+    w = rnd((152064, 3584), 52, torch.bfloat16, 0.05)
+    for m in (1, 7):
+        x = rnd((m, 3584), 53 + m, torch.bfloat16)
+        ref = _exact(x, w)
+        out = ops.gemm_mfma_skinny(x.cuda(), w.cuda(), out_dtype=torch.float32).cpu()
+        assert (out - ref).abs().max() <= 2e-5 * ref.abs().max(), m
+    w = rnd((2 * 27648, 5120), 54, torch.bfloat16, 0.03)
+    for m in (1, 16):
+        x = rnd((m, 5120), 55 + m, torch.bfloat16)
+        full = _exact(x, w)
+        ref = plain.silu_mul(full[:, 0::2], full[:, 1::2])
+        out = ops.gemm_mfma_skinny(x.cuda(), w.cuda(), epilogue="swiglu").float().cpu()
+        assert (out - ref).abs().max() <= tol(torch.bfloat16, ref), m
+    w = rnd((5120, 5120), 56, torch.bfloat16, 0.05)
+    x = rnd((8, 5120), 57, torch.bfloat16)
+    from from_scratch_inference_engine_amd.parts.linear import Linear
+    splits = Linear(5120, 5120).residual_splits(8)
+    assert splits > 1
+    out = ops.gemm_mfma_skinny(x.cuda(), w.cuda(), splits=splits).cpu().double().sum(0).float()
+    assert (out - _exact(x, w)).abs().max() <= 2e-5 * out.abs().max()
+
+
 def test_gemm_mfma_wide_refuses_what_it_does_not_take(ops):
     x, w = rnd((20, 200), 46, torch.bfloat16), rnd((32, 200), 47, torch.bfloat16)
     with pytest.raises(ops.KernelError, match="whole stages of 128"):
@@ -312,7 +360,9 @@ def test_rmsnorm_adds_partial_sums_at_odd_sizes(ops):
     (1, 14, 2, 64, 896, 1e6, True), (9, 3, 3, 48, 72, 1e4, True), (16, 5, 1, 256, 320, 5e5, False),
     (7, 28, 4, 128, 3584, 1e6, True), (33, 2, 1, 16, 64, 1e4, True),
     # on 256 compute units these deal 10 and 14 rotary pairs a workgroup; with a head size of 160 a block's pairs span two heads
-    (8, 24, 4, 160, 256, 1e4, True), (16, 40, 8, 128, 128, 1e6, False)])
+    (8, 24, 4, 160, 256, 1e4, True), (16, 40, 8, 128, 128, 1e6, False),
+    # the q/k/v projection of the 14B and 32B shapes (7,168 rows of 5,120)
+    (1, 40, 8, 128, 5120, 1e6, True), (8, 40, 8, 128, 5120, 1e6, True), (16, 40, 8, 128, 5120, 1e6, True)])
 def test_projection_with_rotary_epilogue(ops, m, heads, kv, hd, k, theta, use_bias):
     """q/k/v projection, bias, rotation and cache write in one kernel, against the plain formulas
     on the float32 product (one rounding to bfloat16, after the rotation)."""
@@ -422,12 +472,15 @@ def paged_case(seqs, heads, kv, hd, page, dtype, seed, window=None, shuffle=True
         edit(qs, ks, vs)
     for s, (p, n) in enumerate(seqs):
         total = p + n
-        for i in range(-(-total // page)):
+        held = -(-total // page)
+        for i in range(held):
             tables[s, i] = order.pop()
-        for j in range(total):
-            pg, off = tables[s, j // page].item(), j % page
-            k_pool[pg, :, off, :] = ks[s][j].reshape(kv, hd)
-            v_pool[pg, :, :, off] = vs[s][j].reshape(kv, hd)
+        mine = tables[s, :held].long()
+        k_all = torch.full((held * page, kv, hd), 7.0)  # the tail of the last page keeps stale content
+        v_all = torch.full((held * page, kv, hd), -9.0)
+        k_all[:total], v_all[:total] = ks[s].reshape(total, kv, hd), vs[s].reshape(total, kv, hd)
+        k_pool[mine] = k_all.reshape(held, page, kv, hd).permute(0, 2, 1, 3)
+        v_pool[mine] = v_all.reshape(held, page, kv, hd).permute(0, 2, 3, 1)
 
     class Host:
         n_seqs = len(seqs)
@@ -506,6 +559,30 @@ def test_attention_over_pages(ops, dtype, scalar, heads, kv, hd, page, window):
         assert 0 < case["plan"]["n_groups"] < case["plan"]["n_large"]
         alone = run_attention(ops, case, heads, kv, hd, window, share_keys=False)
         assert (alone - out).abs().max() <= 2.0 ** -7 * out.abs().max()
+
+
+@pytest.mark.parametrize("heads, kv, seqs", [
+    (28, 4, [(0, 4096)]),                # a whole long prompt: 32 groups of four tiles a kv head on the die-mapped grid
+    (28, 4, [(4096, 2048), (17000, 1)]),  # a portion behind thousands of cached keys; a decode of 67 splits and their merge
+    (40, 8, [(0, 4096)]),
+    (40, 8, [(4096, 2048), (12000, 1)]),
+])
+def test_attention_over_pages_at_the_lengths_that_are_timed(ops, heads, kv, seqs):
+    """The prompt and context lengths that the measurements quote, at the head geometries of the
+    large models (head size 128, page 16, bfloat16), against the plain attention."""
+    hd, page = 128, 16
+    case = paged_case(seqs, heads, kv, hd, page, torch.bfloat16, seed=heads)
+    plan = case["plan"]
+    assert plan["mfma"] and (plan["n_groups"] > 100 or plan["n_merges"])
+    out = run_attention(ops, case, heads, kv, hd)
+    row = 0
+    for (p, n), q, k, v in zip(seqs, case["qs"], case["ks"], case["vs"]):
+        ref = plain.attention(q, k, v, heads, kv, hd, query_offset=p)
+        err = (out[row:row + n] - ref).abs().max().item()
+        assert err <= 2.0 ** -7 * ref.abs().max().item(), f"seq past {p} new {n}: {err}"
+        row += n
+    if len(seqs) > 1:
+        assert max(m[2] for m in plan["merges"]) > (64 if heads == 28 else 40)  # splits of the long decode
 
 
 @pytest.mark.parametrize("dtype, scalar", [(torch.float32, True), (torch.bfloat16, False)])

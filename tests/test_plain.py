@@ -173,3 +173,128 @@ def test_sampler_vectors():
     # vocabulary order of the draw: small u gives the first kept token
     assert plain.sample(torch.tensor([1.0, 1.0, 1.0]), 1.0, 0, 1.0, 0.01) == 0
     assert plain.sample(torch.tensor([1.0, 1.0, 1.0]), 1.0, 0, 1.0, 0.99) == 2
+
+
+# ---- the whole model's composition (src/model/model.cpp:90-149), pinned without any package's
+# model code: special cases in which the model reduces to a few library routines, a second
+# composition written from torch's own routines only, and an invariant of the positions
+def _library_model(cfg, w, ids):
+    """The decoder put together from torch's library routines alone (embedding, rms_norm, linear,
+    silu, scaled_dot_product_attention, complex multiplication for the rotation), in float64 so
+    that it owes nothing to the plain implementation's choices of precision."""
+    import torch.nn.functional as F
+
+    nh, nkv, hd, eps = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["rms_norm_eps"]
+    w = {k: v.double() for k, v in w.items()}
+    s = len(ids)
+    x = F.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    ang = torch.arange(s, dtype=torch.float64)[:, None] * cfg["rope_theta"] ** (
+        -torch.arange(0, hd, 2, dtype=torch.float64) / hd)[None, :]
+    turn = torch.polar(torch.ones_like(ang), ang)[:, None, :]  # [S, 1, hd/2]
+
+    def rotate(t, heads):
+        t = t.reshape(s, heads, hd)
+        z = torch.complex(t[..., :hd // 2], t[..., hd // 2:]) * turn
+        return torch.cat([z.real, z.imag], dim=-1)
+
+    for l in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        h = F.rms_norm(x, (x.shape[-1],), w[p + "input_layernorm.weight"], eps)
+        q = rotate(F.linear(h, w[p + "self_attn.q_proj.weight"], w[p + "self_attn.q_proj.bias"]), nh)
+        k = rotate(F.linear(h, w[p + "self_attn.k_proj.weight"], w[p + "self_attn.k_proj.bias"]), nkv)
+        v = F.linear(h, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"]).reshape(s, nkv, hd)
+        k, v = k.repeat_interleave(nh // nkv, dim=1), v.repeat_interleave(nh // nkv, dim=1)
+        a = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+        x = x + F.linear(a.transpose(0, 1).reshape(s, nh * hd), w[p + "self_attn.o_proj.weight"])
+        h = F.rms_norm(x, (x.shape[-1],), w[p + "post_attention_layernorm.weight"], eps)
+        x = x + F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                         w[p + "mlp.down_proj.weight"])
+    x = F.rms_norm(x, (x.shape[-1],), w["model.norm.weight"], eps)
+    return F.linear(x, w.get("lm_head.weight", w["model.embed_tokens.weight"]))
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_whole_model_equals_a_composition_of_library_routines(model_dirs, name):
+    import helpers
+
+    cfg, w = plain.read_config(model_dirs[name]), plain.read_weights(model_dirs[name])
+    ids = helpers.token_ids(cfg["vocab_size"], 41, 123)
+    got, want = plain.forward(cfg, w, ids).double(), _library_model(cfg, w, ids)
+    assert (got - want).abs().max().item() <= 1e-5
+    assert torch.equal(got.argmax(-1), want.argmax(-1))
+
+
+def _one_layer(seed=0, **sizes):
+    """A one-layer model with larger weights than the tiny ones, so that every term is visible."""
+    cfg = {"hidden_size": 24, "num_hidden_layers": 1, "num_attention_heads": 3, "num_key_value_heads": 1,
+           "head_dim": 8, "intermediate_size": 20, "vocab_size": 31, "rope_theta": 100.0, "rms_norm_eps": 1e-3,
+           "qkv_bias": True}
+    cfg.update(sizes)
+    g = torch.Generator().manual_seed(seed)
+    h, nh, nkv, hd, it, v = (cfg[k] for k in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim",
+                                                "intermediate_size", "vocab_size"))
+    r = lambda *shape: torch.randn(*shape, generator=g) * 0.5
+    p = "model.layers.0."
+    w = {"model.embed_tokens.weight": r(v, h), "model.norm.weight": 1 + r(h), "lm_head.weight": r(v, h),
+         p + "input_layernorm.weight": 1 + r(h), p + "post_attention_layernorm.weight": 1 + r(h),
+         p + "self_attn.q_proj.weight": r(nh * hd, h), p + "self_attn.q_proj.bias": r(nh * hd),
+         p + "self_attn.k_proj.weight": r(nkv * hd, h), p + "self_attn.k_proj.bias": r(nkv * hd),
+         p + "self_attn.v_proj.weight": r(nkv * hd, h), p + "self_attn.v_proj.bias": r(nkv * hd),
+         p + "self_attn.o_proj.weight": r(h, nh * hd), p + "mlp.gate_proj.weight": r(it, h),
+         p + "mlp.up_proj.weight": r(it, h), p + "mlp.down_proj.weight": r(h, it)}
+    return cfg, w
+
+
+def test_model_special_cases_reduce_to_library_routines():
+    import torch.nn.functional as F
+
+    cfg, w = _one_layer()
+    p, eps, ids = "model.layers.0.", cfg["rms_norm_eps"], [5, 30, 5, 11]
+    x = w["model.embed_tokens.weight"][ids]
+    head = lambda t: F.linear(F.rms_norm(t, (t.shape[-1],), w["model.norm.weight"], eps), w["lm_head.weight"])
+    # both residual branches silenced: logits = head(norm(embedding)); no scaling of the embedding
+    w0 = dict(w)
+    w0[p + "self_attn.o_proj.weight"] = torch.zeros_like(w[p + "self_attn.o_proj.weight"])
+    w0[p + "mlp.down_proj.weight"] = torch.zeros_like(w[p + "mlp.down_proj.weight"])
+    assert torch.allclose(plain.forward(cfg, w0, ids), head(x), atol=1e-5)
+    # attention silenced: x + down(silu(gate(n2(x))) * up(n2(x))); swapping gate and up must show
+    w1 = dict(w)
+    w1[p + "self_attn.o_proj.weight"] = w0[p + "self_attn.o_proj.weight"]
+    n2 = F.rms_norm(x, (x.shape[-1],), w[p + "post_attention_layernorm.weight"], eps)
+    mlp = F.linear(F.silu(F.linear(n2, w[p + "mlp.gate_proj.weight"])) * F.linear(n2, w[p + "mlp.up_proj.weight"]),
+                   w[p + "mlp.down_proj.weight"])
+    got = plain.forward(cfg, w1, ids)
+    assert torch.allclose(got, head(x + mlp), atol=1e-5)
+    swapped = dict(w1)
+    swapped[p + "mlp.gate_proj.weight"], swapped[p + "mlp.up_proj.weight"] = w[p + "mlp.up_proj.weight"], w[p + "mlp.gate_proj.weight"]
+    assert (plain.forward(cfg, swapped, ids) - got).abs().max() > 1e-2
+    # feed-forward silenced, one token: attention over one key is its value, so the layer is
+    # x + o(v(n1(x)) + b_v) repeated for every head of the group: bias on v, none on o, the first
+    # norm before the projections, the residual taken from before the norm
+    w2 = dict(w)
+    w2[p + "mlp.down_proj.weight"] = w0[p + "mlp.down_proj.weight"]
+    x1 = x[:1]
+    n1 = F.rms_norm(x1, (x1.shape[-1],), w[p + "input_layernorm.weight"], eps)
+    v = F.linear(n1, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"])
+    a = v.reshape(1, cfg["num_key_value_heads"], cfg["head_dim"]).repeat_interleave(
+        cfg["num_attention_heads"] // cfg["num_key_value_heads"], dim=1).reshape(1, -1)
+    assert torch.allclose(plain.forward(cfg, w2, ids[:1]), head(x1 + F.linear(a, w[p + "self_attn.o_proj.weight"])), atol=1e-5)
+    # the biases of q and k count (a model that dropped them gives other logits for two tokens)
+    nob = dict(w2)
+    nob[p + "self_attn.q_proj.bias"] = torch.zeros_like(w[p + "self_attn.q_proj.bias"])
+    assert (plain.forward(cfg, nob, ids) - plain.forward(cfg, w2, ids)).abs().max() > 1e-4
+
+
+def test_model_depends_on_distances_only_and_rotates_q_and_k_but_not_v(monkeypatch):
+    """All positions shifted by a constant: the logits stay (only distances count), which a
+    rotation of the values, or of q alone, would break."""
+    cfg, w = _one_layer(seed=1, num_attention_heads=4, num_key_value_heads=2, hidden_size=32)
+    ids = [1, 2, 3, 4, 5, 6, 7]
+    base = plain.forward(cfg, w, ids)
+    real = plain.rope
+    monkeypatch.setattr(plain, "rope", lambda x, nh, hd, theta, pos: real(x, nh, hd, theta, [p + 1000 for p in pos]))
+    assert torch.allclose(plain.forward(cfg, w, ids), base, atol=2e-5)
+    # the check can fail: rotating only what has as many heads as q (q alone) changes the logits
+    monkeypatch.setattr(plain, "rope", lambda x, nh, hd, theta, pos:
+                        real(x, nh, hd, theta, [p + 1000 for p in pos]) if nh == 4 else real(x, nh, hd, theta, pos))
+    assert (plain.forward(cfg, w, ids) - base).abs().max() > 1e-3

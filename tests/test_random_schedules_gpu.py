@@ -67,3 +67,5 @@ def test_random_schedule_matches_plain(model_dirs, name, dtype, seed, page_size,
     assert checked > 50
     if num_pages * page_size <= 160:
         assert reused > 0  # the small pools did run out
+        alloc = runner.manager.allocators[0]
+        assert alloc.pages_issued > num_pages and len(alloc.pages_issued_again()) > num_pages // 2

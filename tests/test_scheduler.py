@@ -294,3 +294,22 @@ def test_pipelined_loop_gives_the_same_outputs_and_frees_everything():
         assert all(q.status == SeqStatus.Finished for q in s.sequences.values())
     assert outs[0] == outs[1]
     assert any(o[-1] == 7 and len(o) > 1 for o in outs[0].values())     # an eos was found one step late
+
+
+def test_no_more_running_requests_than_a_step_has_tokens_for():
+    """max_batch above the token budget is cut to it: six requests, three tokens a step; the three
+    that run each decode in every step, the others are admitted as those finish."""
+    m, s = make(num_pages=64, page_size=2, budget=3, max_batch=6)
+    assert s.max_batch == 3
+    ids = [s.add_request(Request([1 + i], max_tokens=4)) for i in range(6)]
+    seen = []
+    while s.has_work():
+        items = launch(m, s.schedule())
+        assert 0 < sum(len(it.tokens) for it in items) <= 3
+        running = [q for q in s.running]
+        assert sorted(it.seq.id for it in items) == sorted(running)  # nobody who runs is left out
+        seen.append([it.seq.id for it in items])
+        s.finish_step(items, [50] * len(items))
+    assert seen[0] == ids[:3] and seen[-1] == ids[3:]
+    assert all(len(s.sequences[i].output) == 4 for i in ids)
+    m.check_invariants()

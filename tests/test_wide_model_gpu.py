@@ -1,0 +1,220 @@
+"""The engine against the plain implementation at the layer sizes of Qwen2.5-7B: hidden 3584,
+28 query and 4 key/value heads of 128, intermediate 18944, vocabulary 152,064, untied head, page
+size 16.  Four layers instead of 28 (named here, so that the test fits the suite's time and the
+host's memory: 2.0 billion parameters, 8 GB as float32 for the plain side); every width, and so
+every kernel shape of the full model, is the real one.
+
+float32: prompts of 330, 301 and 77 tokens, whole; all but the last 32 tokens in one step and
+those one by one; in portions of changing size; and mixed in one pool so small that the second
+wave of requests gets the pages of the first.  Within 1e-4 of the plain logits, identical argmax
+wherever the plain choice is clear (the reference's own whole-model checks on its device path:
+tests/cpp/test_cuda_model.cpp:18-70, 113-218).
+
+bfloat16: the same families.  Random weights give small logits and rounding the activations to
+bfloat16 moves them by a few per cent of the largest one, in the plain model as well; so the
+bound is stated against that: the engine may differ from the plain float32 logits by at most
+twice (largest) and one and a half times (root mean square) what the plain model itself moves
+when its activations are rounded to bfloat16 where the engine rounds them, and it picks the
+plain token wherever that one leads by more than twice the largest difference.  Decode batches
+of 32, 64 and 128 through replayed graphs, with the library's kernels chosen by timing, are checked
+against the plain logits in the same way.
+"""
+
+import json
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_qwen2 as plain
+
+pytestmark = pytest.mark.gpu
+
+LAYERS = 4  # of the 28 that the 7B shape has
+WIDE = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": 3584,
+    "num_hidden_layers": LAYERS, "num_attention_heads": 28, "num_key_value_heads": 4, "head_dim": 128,
+    "intermediate_size": 18944, "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False, "max_position_embeddings": 4096, "use_sliding_window": False,
+}
+LENGTHS = [330, 301, 77]
+PORTIONS = [7, 2, 16, 3, 2, 33, 5, 2, 64, 9, 130]
+
+
+def _rounded_plain(cfg, w, ids):
+    """The plain model with its activations rounded to bfloat16 where the bfloat16 engine rounds
+    them: the inputs of every product, q and k after the rotation, the gated activation."""
+    r16 = lambda t: t.to(torch.bfloat16).float()
+    lin, rope, silu = plain.linear, plain.rope, plain.silu_mul
+    plain.linear = lambda x, wt, b=None: lin(r16(x), wt, b)
+    plain.rope = lambda *a, **k: r16(rope(*a, **k))
+    plain.silu_mul = lambda g, u: r16(silu(r16(g), r16(u)))
+    try:
+        return plain.forward(cfg, w, ids)
+    finally:
+        plain.linear, plain.rope, plain.silu_mul = lin, rope, silu
+
+
+@pytest.fixture(scope="module")
+def wide(tmp_path_factory):
+    """The model folder (bfloat16 values, drawn on the device by the test's own generator, so
+    that both precisions and the plain side read the same numbers) and the plain logits."""
+    from safetensors.torch import save_file
+
+    d = tmp_path_factory.mktemp("wide7b")
+    (d / "config.json").write_text(json.dumps(WIDE))
+    g = torch.Generator(device="cuda").manual_seed(11)
+    tensors = {}
+    for name, shape in sorted(helpers.expected_tensor_shapes(WIDE).items()):
+        t = torch.randn(shape, generator=g, device="cuda") * 0.02
+        if name.endswith("norm.weight") or name.endswith("layernorm.weight"):
+            t = t + 1.0
+        tensors[name] = t.to(torch.bfloat16).cpu()
+    save_file(tensors, str(d / "model.safetensors"))
+    del tensors
+    print("wide model written", flush=True)
+    cfg, w = plain.read_config(d), plain.read_weights(d)
+    prompts = [helpers.token_ids(WIDE["vocab_size"], n, 4000 + n) for n in LENGTHS]
+    ref = [plain.forward(cfg, w, p) for p in prompts]
+    print("plain logits done", flush=True)
+    moved = [(_rounded_plain(cfg, w, p) - r) for p, r in zip(prompts, ref)]
+    noise = [(m.abs().max().item(), m.pow(2).mean().sqrt().item()) for m in moved]
+    # short prompts of the decode batches (graphs): the first eight are compared with the plain model
+    short = [helpers.token_ids(WIDE["vocab_size"], 20 + i % 7 + 12, 5000 + i) for i in range(128)]
+    short_ref = [plain.forward(cfg, w, p) for p in short[:8]]
+    del w, moved
+    print("rounded plain logits done", flush=True)
+    return {"dir": d, "prompts": prompts, "ref": ref, "noise": noise, "short": short, "short_ref": short_ref}
+
+
+def _plans():
+    """{family: list of steps; a step is a list of (request key, prompt index, n tokens)}."""
+    n = LENGTHS
+    whole = [[(f"w{i}", i, n[i])] for i in range(3)]
+    decode = []
+    for i in range(3):
+        decode.append([(f"d{i}", i, n[i] - 32)])
+        decode += [[(f"d{i}", i, 1)] for _ in range(32)]
+    portions = []
+    for i in range(3):
+        fed, j = 0, i
+        while fed < n[i]:
+            k = min(PORTIONS[j % len(PORTIONS)], n[i] - fed)
+            portions.append([(f"p{i}", i, k)])
+            fed, j = fed + k, j + 1
+    # mixed: three live requests, portions of some beside single tokens of others; then the same
+    # prompts again under new names, cut otherwise, in the pages the first wave gave back
+    mixed = []
+    for wave, cuts in enumerate(([40, 5, 17], [3, 64, 2])):
+        fed = [0, 0, 0]
+        key = lambda i: f"m{wave}{i}"
+        step = 0
+        while any(f < m for f, m in zip(fed, n)):
+            entries = []
+            for i in range(3):
+                left = n[i] - fed[i]
+                if left <= 0 or (step + i) % 5 == 4:
+                    continue  # done, or left out of this step
+                k = 1 if left <= 24 else min(left - 24, cuts[(i + step) % 3] if step % 3 else cuts[i])
+                entries.append((key(i), i, k))
+                fed[i] += k
+            if entries:
+                mixed.append(entries)
+            step += 1
+    return {"whole": whole, "decode": decode, "portions": portions, "mixed": mixed}
+
+
+def _run(runner, prompts, plan):
+    """Runs the steps (every token's logits wanted); returns {request key: (prompt, logits [n, V])}."""
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+
+    caches, fed, rows, which = {}, {}, {}, {}
+    for step in plan:
+        entries = []
+        for key, i, k in step:
+            if key not in caches:
+                caches[key], fed[key], rows[key], which[key] = runner.manager.open(key), 0, [], i
+            entries.append(StepEntry(caches[key], prompts[i][fed[key]:fed[key] + k], list(range(k))))
+            fed[key] += k
+        out = runner.step(entries).float().cpu()
+        at = 0
+        for key, i, k in step:
+            rows[key].append(out[at:at + k])
+            at += k
+            if fed[key] == len(prompts[i]):
+                runner.manager.close(caches[key])  # its pages go back; a later request takes them
+        runner.manager.check_invariants()
+    return {key: (which[key], torch.cat(r)) for key, r in rows.items()}
+
+
+def test_float32_families_at_7b_widths(wide):
+    from from_scratch_inference_engine_amd.engine.model import Model, Runner
+
+    model = Model.from_pretrained(wide["dir"], dtype="float32")
+    # 46 pages hold the three prompts together (21 + 19 + 5 pages) and one more: the second wave
+    # of the mixed family can only run in the first wave's pages
+    runner = Runner(model, page_size=16, num_pages=46, max_requests=4)
+    worst = clear = rows = 0
+    for family, plan in _plans().items():
+        for key, (i, logits) in _run(runner, wide["prompts"], plan).items():
+            ref = wide["ref"][i].numpy()
+            assert logits.shape[0] == LENGTHS[i], f"{family} {key}: every position was asked for"
+            c, r = helpers.assert_close_to_plain(logits.numpy(), ref, "float32", f"float32 {family} {key}")
+            clear, rows = clear + c, rows + r
+            worst = max(worst, float(np.abs(logits.numpy() - ref).max()))
+    alloc = runner.manager.allocators[0]
+    print(f"float32 at 7B widths, {LAYERS} layers: largest difference {worst:.3e}; argmax compared on {clear} of {rows} rows; "
+          f"{alloc.pages_issued} pages handed out of a pool of {alloc.num_pages}")
+    assert 2 * clear >= rows
+    assert alloc.pages_issued > 4 * alloc.num_pages and len(alloc.pages_issued_again()) > alloc.num_pages * 3 // 4
+    assert alloc.num_free == alloc.num_pages
+
+
+def _assert_within_rounding(logits, ref, noise, what):
+    diff = (logits - ref)
+    worst, rms = diff.abs().max().item(), diff.pow(2).mean().sqrt().item()
+    assert torch.isfinite(logits).all(), what
+    assert worst <= 2.0 * noise[0], f"{what}: max|diff| {worst:.3e} against {noise[0]:.3e} from rounding alone"
+    assert rms <= 1.5 * noise[1], f"{what}: rms diff {rms:.3e} against {noise[1]:.3e} from rounding alone"
+    top2 = ref.topk(2, dim=-1).values
+    clear = (top2[:, 0] - top2[:, 1]) > 2 * worst
+    assert torch.equal(logits.argmax(-1)[clear], ref.argmax(-1)[clear]), f"{what}: argmax differs on a clear row"
+    return worst / noise[0], rms / noise[1]
+
+
+def test_bfloat16_families_and_graph_batches_at_7b_widths(wide):
+    from from_scratch_inference_engine_amd import ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Model, Runner
+
+    model = Model.from_pretrained(wide["dir"], dtype="bfloat16")
+    runner = Runner(model, page_size=16, num_pages=46, max_requests=4)
+    ratios = []
+    for family, plan in _plans().items():
+        for key, (i, logits) in _run(runner, wide["prompts"], plan).items():
+            ratios.append(_assert_within_rounding(logits, wide["ref"][i], wide["noise"][i], f"bfloat16 {family} {key}"))
+    print(f"bfloat16 at 7B widths: difference / rounding noise, largest {max(r[0] for r in ratios):.2f} (max), "
+          f"{max(r[1] for r in ratios):.2f} (rms)")
+    del runner
+    # decode batches of 32, 64 and 128 rows: the library's products (chosen by timing) inside replayed
+    # graphs, with other work between the replays; the first eight requests against the plain model
+    noise = max(n[0] for n in wide["noise"]), max(n[1] for n in wide["noise"])
+    short, short_ref = wide["short"], wide["short_ref"]
+    ops.enable_library_tuning(max_ms_per_candidate=5, iterations=2)
+    try:
+        for batch in (32, 64, 128):
+            runner = Runner(model, page_size=16, num_pages=batch * 3 + 8, max_requests=batch)
+            caches = [runner.manager.open(i) for i in range(batch)]
+            runner.step([StepEntry(c, p[:-12], []) for c, p in zip(caches, short)])
+            for t in range(12, 0, -1):
+                out = runner.step([StepEntry(c, [p[-t]], [0]) for c, p in zip(caches, short)]).float().cpu()
+                torch.cuda.synchronize()
+                _ = (torch.randn(128, 128, device="cuda") @ torch.randn(128, 128, device="cuda")).sum().item()
+                got = torch.stack([out[i] for i in range(8)])
+                ref = torch.stack([short_ref[i][len(short[i]) - t] for i in range(8)])
+                _assert_within_rounding(got, ref, noise, f"decode batch of {batch} through graphs, {t} from the end")
+            assert runner.graphs.captures == 1 and runner.graphs.replays == 11
+            del runner, caches
+    finally:
+        ops.disable_library_tuning()
