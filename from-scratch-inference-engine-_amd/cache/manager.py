@@ -1,9 +1,10 @@
 """Host side of the cache: who holds which page and which state slot.
 
-The manager knows nothing of models.  It is built from *needs*: a ``PagedNeed`` says that some
-layers keep one entry per token (all of them, or only a window of the latest), a ``StateNeed``
-says that a layer keeps a fixed-size state per request.  Layers with equal paged needs form a
-*group*; a group has its own pool of pages, and each request has one block table per group.
+The manager knows nothing of models.  It is built from *needs* (``cache.needs``): a per-token
+need says that some layers keep one entry per token (all of them, or only a window of the
+latest), a per-request need says that a layer keeps a fixed-size state per request.  Layers with
+equal per-token needs form a *group*; a group has its own pool of pages, and each request has one
+block table per group.  Of a need the manager reads the ``window`` only.
 Device memory is not touched here (``cache.storage`` holds the tensors), so every decision
 can be tested on the CPU.
 """
@@ -14,35 +15,11 @@ from dataclasses import dataclass, field
 from typing import Dict, Hashable, Iterable, List, Optional, Sequence, Tuple
 
 from .allocator import OutOfPages, PageAllocator
+from .needs import CacheNeed, PagedNeed, StateNeed  # noqa: F401  (PagedNeed and StateNeed are also named from here)
 
 
 class NoFreeSlot(RuntimeError):
     """All per-request state slots are taken."""
-
-
-@dataclass(frozen=True)
-class PagedNeed:
-    """One entry per token and layer: ``n_kv_heads * head_dim`` keys and as many values.
-    ``window`` = number of latest positions a query still reads (itself included); ``None``
-    means all of them."""
-
-    n_kv_heads: int
-    head_dim: int
-    window: Optional[int] = None
-
-    def __post_init__(self):
-        if self.n_kv_heads < 1 or self.head_dim < 1:
-            raise ValueError("PagedNeed: sizes must be positive")
-        if self.window is not None and self.window < 1:
-            raise ValueError("PagedNeed: window must be >= 1")
-
-
-@dataclass(frozen=True)
-class StateNeed:
-    """A tensor of fixed ``shape`` per request and layer (torch dtype name, e.g. 'float32')."""
-
-    shape: Tuple[int, ...]
-    dtype: str = "float32"
 
 
 @dataclass
@@ -62,7 +39,7 @@ class RequestCache:
 
 
 class CacheManager:
-    def __init__(self, paged_groups: Sequence[PagedNeed], page_size: int,
+    def __init__(self, paged_groups: Sequence[CacheNeed], page_size: int,
                  num_pages, max_requests: int):
         """``num_pages``: one number for every group or one per group."""
         if page_size < 1:
@@ -70,7 +47,7 @@ class CacheManager:
         if max_requests < 1:
             raise ValueError("CacheManager: max_requests must be positive")
         self.page_size = int(page_size)
-        self.groups: List[PagedNeed] = list(paged_groups)
+        self.groups: List[CacheNeed] = list(paged_groups)
         if isinstance(num_pages, int):
             num_pages = [num_pages] * len(self.groups)
         if len(num_pages) != len(self.groups):

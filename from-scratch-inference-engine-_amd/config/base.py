@@ -21,6 +21,17 @@ class ModelConfig:
 
     architecture: str
 
+    @property
+    def max_positions(self) -> int:
+        """The most positions a request may reach (0: no limit), from whichever key the
+        architecture's config.json keeps it under."""
+        return 0
+
+    @property
+    def end_token(self) -> int:
+        """The end-of-sequence token id of config.json, -1 if it names none."""
+        return -1
+
     @classmethod
     def from_dict(cls, raw: Mapping[str, Any]) -> "ModelConfig":  # pragma: no cover - abstract
         raise NotImplementedError
@@ -41,6 +52,30 @@ def read_config_json(model_dir) -> dict:
     if not isinstance(raw, dict):
         raise ConfigError(f"{path}: top level must be an object")
     return raw
+
+
+def end_token_of(raw: Mapping[str, Any]) -> int:
+    """``eos_token_id`` of a config.json or generation_config.json: an id, the first of a list of
+    ids, or -1 where there is none."""
+    eos = raw.get("eos_token_id")
+    if isinstance(eos, (list, tuple)):
+        eos = eos[0] if eos else None
+    if eos is None:
+        return -1
+    return checked_int(eos, "eos_token_id", -1)
+
+
+def generation_end_token(model_dir) -> int:
+    """The end token that the folder's generation_config.json names (it goes before config.json's,
+    as in the reference's python/engine/llm.py:18-30); -1 if the file or the key is missing."""
+    path = Path(model_dir) / "generation_config.json"
+    if not path.is_file():
+        return -1
+    try:
+        raw = json.loads(path.read_text(encoding="utf-8"))
+    except json.JSONDecodeError as e:
+        raise ConfigError(f"{path}: invalid JSON: {e}") from e
+    return end_token_of(raw) if isinstance(raw, dict) else -1
 
 
 def required_int(raw: Mapping[str, Any], key: str, minimum: int = 1) -> int:

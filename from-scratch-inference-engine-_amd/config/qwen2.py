@@ -5,7 +5,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Any, Mapping
 
-from .base import ConfigError, ModelConfig, checked_float, checked_int, required_int
+from .base import ConfigError, ModelConfig, checked_float, checked_int, end_token_of, required_int
 
 
 @dataclass(frozen=True)
@@ -34,6 +34,14 @@ class Qwen2Config(ModelConfig):
     hidden_act: str = "silu"
     model_type: str = "qwen2"
     eos_token_id: int = -1
+
+    @property
+    def max_positions(self) -> int:
+        return self.max_position_embeddings
+
+    @property
+    def end_token(self) -> int:
+        return self.eos_token_id
 
     @classmethod
     def from_dict(cls, raw: Mapping[str, Any]) -> "Qwen2Config":
@@ -64,11 +72,6 @@ class Qwen2Config(ModelConfig):
             raise ConfigError("config.json: rope_scaling is not supported")
         if raw.get("use_sliding_window", False):
             raise ConfigError("config.json: use_sliding_window=true is not supported")
-        eos = raw.get("eos_token_id", -1)
-        if isinstance(eos, list):
-            eos = eos[0] if eos else -1
-        if eos is None:
-            eos = -1
         qkv_bias = True if model_type == "qwen2" else bool(raw.get("attention_bias", False))
         return cls(
             architecture=str(archs[0]),
@@ -87,7 +90,7 @@ class Qwen2Config(ModelConfig):
             attention_qkv_bias=qkv_bias,
             hidden_act=act,
             model_type=model_type,
-            eos_token_id=int(eos),
+            eos_token_id=end_token_of(raw),
         )
 
     def to_dict(self) -> dict:

@@ -42,6 +42,12 @@ int fsie_embedding(const void* table, int dtype, const int32_t* ids, float* out,
 int fsie_rmsnorm(float* residual, const void* delta, const float* weight, void* out, const int32_t* rows,
                  int n_rows, int hidden, float eps, int dtype, int write_back, int n_parts, int total_rows,
                  hipStream_t stream);
+// RMSNorm of a plain tensor (no residual stream): every row holds `groups` runs of `width` values
+// (strides in elements), each run normalised by itself; `out` may be `x`.
+int fsie_rmsnorm_plain(const void* x, int64_t x_stride, const float* weight, void* out, int64_t out_stride, int n_rows,
+                       int groups, int width, float eps, int dtype, hipStream_t stream);
+// Rows slots[0..n) of a table of n_slots rows of row_bytes set to zero; a negative slot is skipped.
+int fsie_zero_rows(void* table, const int32_t* slots, int n, int64_t row_bytes, int n_slots, hipStream_t stream);
 int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream);
 int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream);
 int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream);

@@ -264,7 +264,78 @@ __global__ void bias_add_kernel(T* __restrict__ y, const float* __restrict__ bia
     if (i < total) y[i] = from_float<T>(to_float(y[i]) + bias[i % cols]);
 }
 
+// Rows of a table set to zero: row slots[i] of [n_slots, row_bytes / 4] words, negative = none.
+__global__ void zero_rows_kernel(uint32_t* __restrict__ table, const int32_t* __restrict__ slots, int64_t row_words,
+                                 int n_slots) {
+    const int slot = slots[blockIdx.x];
+    if (slot < 0 || slot >= n_slots) return;
+    uint32_t* row = table + static_cast<int64_t>(slot) * row_words;
+    for (int64_t i = static_cast<int64_t>(blockIdx.y) * blockDim.x + threadIdx.x; i < row_words;
+         i += static_cast<int64_t>(gridDim.y) * blockDim.x)
+        row[i] = 0u;
+}
+
+// RMSNorm of a plain tensor, no residual stream: every row of x holds `groups` runs of `width`
+// values, each normalised by itself (a whole row, or the heads of a row); one wave a run.
+template <typename T>
+__global__ void rmsnorm_plain_kernel(const T* __restrict__ x, int64_t x_stride, const float* __restrict__ weight,
+                                     T* __restrict__ out, int64_t out_stride, int64_t n_runs, int groups, int width,
+                                     float eps) {
+    const int lane = threadIdx.x & (FSIE_WAVE - 1);
+    const int64_t run = static_cast<int64_t>(blockIdx.x) * (blockDim.x / FSIE_WAVE) + threadIdx.x / FSIE_WAVE;
+    if (run >= n_runs) return;
+    const int64_t row = run / groups;
+    const int g = static_cast<int>(run % groups);
+    const T* src = x + row * x_stride + static_cast<int64_t>(g) * width;
+    T* dst = out + row * out_stride + static_cast<int64_t>(g) * width;
+    float sum = 0.f;
+    for (int i = lane; i < width; i += FSIE_WAVE) {
+        const float v = to_float(src[i]);
+        sum += v * v;
+    }
+    sum = wave_sum(sum);
+    const float r = 1.0f / sqrtf(sum / static_cast<float>(width) + eps);
+    for (int i = lane; i < width; i += FSIE_WAVE) dst[i] = from_float<T>(to_float(src[i]) * r * weight[i]);
+}
+
 }  // namespace
+
+extern "C" int fsie_zero_rows(void* table, const int32_t* slots, int n, int64_t row_bytes, int n_slots,
+                              hipStream_t stream) {
+    FSIE_REQUIRE(n >= 0 && n_slots >= 0 && row_bytes >= 0 && row_bytes % 4 == 0,
+                 "zero_rows: bad sizes n=%d slots=%d row_bytes=%lld", n, n_slots, static_cast<long long>(row_bytes));
+    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(table) % 4 == 0, "zero_rows: the table must be 4-byte aligned");
+    if (n == 0 || row_bytes == 0) return 0;
+    const int64_t words = row_bytes / 4;
+    const dim3 grid(n, static_cast<unsigned>(ceil_div64(words, 4 * kThreads) > 64 ? 64 : ceil_div64(words, 4 * kThreads)));
+    zero_rows_kernel<<<grid, kThreads, 0, stream>>>(static_cast<uint32_t*>(table), slots, words, n_slots);
+    FSIE_CHECK_LAUNCH("zero_rows");
+    return 0;
+}
+
+extern "C" int fsie_rmsnorm_plain(const void* x, int64_t x_stride, const float* weight, void* out, int64_t out_stride,
+                                  int n_rows, int groups, int width, float eps, int dtype, hipStream_t stream) {
+    FSIE_REQUIRE(n_rows >= 0 && groups > 0 && width > 0, "rmsnorm_plain: bad sizes rows=%d groups=%d width=%d", n_rows,
+                 groups, width);
+    FSIE_REQUIRE(x_stride >= static_cast<int64_t>(groups) * width && out_stride >= static_cast<int64_t>(groups) * width,
+                 "rmsnorm_plain: a row is shorter than its %d runs of %d", groups, width);
+    FSIE_REQUIRE(dtype == FSIE_F32 || dtype == FSIE_BF16, "rmsnorm_plain: unknown dtype %d", dtype);
+    const int64_t runs = static_cast<int64_t>(n_rows) * groups;
+    if (runs == 0) return 0;
+    const int per_block = kThreads / FSIE_WAVE;
+    const unsigned grid = static_cast<unsigned>(ceil_div64(runs, per_block));
+    if (dtype == FSIE_F32) {
+        rmsnorm_plain_kernel<float><<<grid, kThreads, 0, stream>>>(static_cast<const float*>(x), x_stride, weight,
+                                                                   static_cast<float*>(out), out_stride, runs, groups,
+                                                                   width, eps);
+    } else {
+        rmsnorm_plain_kernel<bf16_t><<<grid, kThreads, 0, stream>>>(static_cast<const bf16_t*>(x), x_stride, weight,
+                                                                    static_cast<bf16_t*>(out), out_stride, runs, groups,
+                                                                    width, eps);
+    }
+    FSIE_CHECK_LAUNCH("rmsnorm_plain");
+    return 0;
+}
 
 extern "C" int fsie_embedding(const void* table, int dtype, const int32_t* ids, float* out,
                               int n_tokens, int hidden, int vocab, hipStream_t stream) {

@@ -67,6 +67,8 @@ class HostBatch:
             self.q_starts.append(self.q_starts[-1] + n)
         self.n_tokens = self.q_starts[-1]
         self.seq_slots = [e.cache.slot for e in entries]
+        # the slots of the requests that start in this step (their per-request memory is reset), -1 for the others
+        self.reset_slots = [e.cache.slot if e.cache.length == 0 else -1 for e in entries]
         self.token_ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64,
                                      count=self.n_tokens)
         self.positions = np.concatenate(
@@ -138,7 +140,8 @@ class StepContext:
     """Passed to every part.  Device tensors are int32.
 
     ``token_ids`` [T], ``positions`` [T], ``want_rows`` [wanted], ``seq_slots`` [n] (state slot of
-    each request), ``q_starts`` [n+1], ``past_lens`` [n]; per paged group ``block_tables[g]``
+    each request), ``reset_slots`` [n] (the same for a request that starts in this step, else -1),
+    ``q_starts`` [n+1], ``past_lens`` [n]; per paged group ``block_tables[g]``
     [n, pages] and ``slots[g]`` [T]; ``host`` holds the same as Python lists/arrays.
     ``plan(planner)`` gives the tables a part asked for through its ``planner()``."""
 
@@ -149,7 +152,7 @@ class StepContext:
         self.n_tokens = host.n_tokens
         self.n_seqs = host.n_seqs
         self.token_ids = self.positions = self.want_rows = None
-        self.seq_slots = self.q_starts = self.past_lens = None
+        self.seq_slots = self.q_starts = self.past_lens = self.reset_slots = None
         # set by the model: every norm can add up a delta that comes as float32 partial sums
         self.partial_sums_ok = False
         self.block_tables: List[torch.Tensor] = []
@@ -184,6 +187,7 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
     i_pos = pk.add(host.positions)
     i_want = pk.add(host.want_rows)
     i_slots = pk.add(np.asarray(host.seq_slots, dtype=np.int32))
+    i_reset = pk.add(np.asarray(host.reset_slots, dtype=np.int32))
     i_qs = pk.add(np.asarray(host.q_starts, dtype=np.int32))
     i_past = pk.add(np.asarray(host.past_lens, dtype=np.int32))
     ps = manager.page_size
@@ -212,6 +216,7 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
     dev = pk.upload(staging, device, into)
     ctx.token_ids, ctx.positions, ctx.want_rows = dev[i_ids], dev[i_pos], dev[i_want]
     ctx.seq_slots, ctx.q_starts, ctx.past_lens = dev[i_slots], dev[i_qs], dev[i_past]
+    ctx.reset_slots = dev[i_reset]
     for it, isl in group_idx:
         ctx.block_tables.append(dev[it])
         ctx.slots.append(dev[isl])

@@ -109,14 +109,22 @@ class DecodeGraphs:
                 return None
             if len(self._graphs) >= self.max_graphs:
                 self._graphs.pop(next(iter(self._graphs)))
-            # eager run on the tables of this step first: allocates nothing the graph keeps, warms
-            # the library's kernel selection
+            # An eager run of the same shape first: it allocates what the graph must not, and warms
+            # the library's kernel selection.  It runs on rows that belong to no request (the spare
+            # page, the spare slot), so that the step itself is executed once and only once, by the
+            # replay below: a part whose cache is a running state would otherwise advance it twice.
+            warm = [filler_entry(runner.storage, 1, runner.manager.page_size) for _ in entries]
+            for w in warm:
+                w.want = (0,)
+            warm_ctx, _ = build_context(warm, runner.manager, runner.model.planners, runner._staging,
+                                        runner.model.dtype, runner.model.device, pad=pad)
+            runner.model.forward(warm_ctx, runner.storage)
+            torch.cuda.synchronize()
+            del warm_ctx
             ctx, tables = build_context(entries, runner.manager, runner.model.planners, runner._staging,
                                         runner.model.dtype, runner.model.device, pad=pad)
             if feed is not None:
                 ctx.token_ids[:n].copy_(feed)
-            runner.model.forward(ctx, runner.storage)
-            torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             # Nothing may free device or pinned memory while the stream is captured.  Dead cycles
             # of Python objects that hold such memory (or other graphs) are therefore collected
@@ -132,9 +140,7 @@ class DecodeGraphs:
                     gc.enable()
             self._graphs[key] = (graph, tables, logits, ctx.token_ids)
             self.captures += 1
-            # the eager run above already wrote this step's keys and values; replaying writes the
-            # same values again
-            graph.replay()
+            graph.replay()  # the step itself
             return logits[:n]
         graph, tables, logits, token_ids = hit
         build_context(entries, runner.manager, runner.model.planners, runner._staging, runner.model.dtype,

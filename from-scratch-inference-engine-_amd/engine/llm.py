@@ -3,29 +3,14 @@
 
 from __future__ import annotations
 
-import json
 from dataclasses import dataclass
 from pathlib import Path
 from typing import List, Optional, Sequence
 
+from ..config.base import generation_end_token
 from ..sampling.params import SamplingParams
 from .engine import Engine
 from .model import Model
-
-
-def _read_eos_id(model_dir: Path) -> int:
-    """generation_config.json, then config.json: ``eos_token_id``; a list gives its first
-    element; -1 if unspecified (python/engine/llm.py:18-30)."""
-    for name in ("generation_config.json", "config.json"):
-        path = model_dir / name
-        if not path.exists():
-            continue
-        eos = json.loads(path.read_text(encoding="utf-8")).get("eos_token_id")
-        if isinstance(eos, list):
-            eos = eos[0] if eos else None
-        if eos is not None:
-            return int(eos)
-    return -1
 
 
 @dataclass
@@ -62,7 +47,12 @@ class LLM:
         self.model = Model.from_pretrained(model_dir, dtype=dtype, device=device)
         self.engine = Engine(self.model, block_size, num_blocks, seed, max_batch, enable_prefix_cache,
                              max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk)
-        self.eos_id = _read_eos_id(model_dir) if eos_id is None else eos_id
+        if eos_id is None:
+            # the folder's generation_config.json, then the model's typed configuration
+            eos_id = generation_end_token(model_dir)
+            if eos_id < 0:
+                eos_id = self.model.config.end_token
+        self.eos_id = eos_id
         self._model_dir = model_dir
         self._tokenizer = None
 

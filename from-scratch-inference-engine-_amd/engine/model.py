@@ -15,7 +15,8 @@ import torch
 
 from .. import ops
 from ..cache.allocator import OutOfPages
-from ..cache.manager import CacheManager, PagedNeed, StateNeed
+from ..cache.manager import CacheManager
+from ..cache.needs import CacheNeed
 from ..cache.storage import CacheLayout, CacheStorage
 from ..config.base import ModelConfig, read_config_json
 from ..models.registry import build_model_spec, parse_config
@@ -69,19 +70,23 @@ class Model:
                 if not 0 <= call.cache_of < i or spec.schedule[call.cache_of].cache_of is not None:
                     raise ValueError(f"schedule entry {i}: cache_of must name an earlier call that keeps a cache")
                 self.call_cache.append(call.cache_of)
-        groups: List[PagedNeed] = []
+        # per-token needs that compare equal share a pool of pages (a group); a per-request need
+        # gets slots of its own.  What the memory looks like is the need's business.
+        groups: List[CacheNeed] = []
         group_caches: List[List[int]] = []
-        states: Dict[int, StateNeed] = {}
+        states: Dict[int, CacheNeed] = {}
         for cid, need in needs.items():
-            if isinstance(need, PagedNeed):
+            per_token = getattr(need, "per_token", None)
+            if not isinstance(per_token, bool) or not callable(getattr(need, "allocate", None)):
+                raise TypeError(f"cache_need() of call {cid} returned {type(need).__name__}, which is no cache need "
+                                f"(per_token, allocate, view)")
+            if per_token:
                 if need not in groups:
                     groups.append(need)
                     group_caches.append([])
                 group_caches[groups.index(need)].append(cid)
-            elif isinstance(need, StateNeed):
-                states[cid] = need
             else:
-                raise TypeError(f"cache_need() of call {cid} returned {type(need).__name__}")
+                states[cid] = need
         self.cache_layout = CacheLayout(groups, group_caches, states)
         self.cached_calls = set(needs)
         # planners of all mixers, one per distinct key
@@ -134,8 +139,7 @@ class Model:
         return manager, storage
 
     def cache_bytes_per_token(self) -> int:
-        item = torch.empty((), dtype=self.dtype).element_size()
-        return sum(2 * need.n_kv_heads * need.head_dim * item * len(ids)
+        return sum(need.bytes_per_token(self.dtype) * len(ids)
                    for need, ids in zip(self.cache_layout.paged_groups, self.cache_layout.group_caches))
 
     # ---------------------------------------------------------------- compute
@@ -144,6 +148,7 @@ class Model:
         spec = self.spec
         ctx.partial_sums_ok = self.partial_sums_ok
         ctx.memo.clear()  # a captured graph must hold whatever the layers share: nothing is kept from an earlier pass
+        storage.reset_states(ctx)  # requests that start in this step find their per-request memory zero
         hidden = HiddenState(spec.embedding.forward(ctx.token_ids))
         for i, call in enumerate(spec.schedule):
             cid = self.call_cache[i]
@@ -164,7 +169,7 @@ class Runner:
         self.manager, self.storage = model.make_cache(page_size, num_pages, max_requests)
         self._staging = PinnedStaging()
         self.vocab_size = model.spec.embedding.vocab_size
-        self.max_position = int(getattr(model.config, "max_position_embeddings", 0) or 0)
+        self.max_position = int(model.config.max_positions)  # 0: the architecture sets no limit
         self.steps = 0
         self.tokens = 0
         from .graphs import DecodeGraphs
@@ -194,7 +199,7 @@ class Runner:
                                      f"{e.cache.request_id!r}")
             if self.max_position and e.cache.length + n > self.max_position:
                 raise ValueError(f"step: request {e.cache.request_id!r} would reach {e.cache.length + n} "
-                                 f"positions, more than max_position_embeddings {self.max_position}")
+                                 f"positions, more than the model's limit of {self.max_position}")
 
     def step(self, entries: Sequence[StepEntry], keep: bool = True,
              feed: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -211,7 +216,6 @@ class Runner:
             raise OutOfPages("step: the batch needs more pages than the pool has free")
         for e in entries:
             self.manager.reserve(e.cache, len(e.tokens))
-        self.storage.reset_states([e.cache.slot for e in entries if e.cache.length == 0])
         pad = self.graphs.shape_of(entries) if self.graphs is not None else None
         logits = self.graphs.step(entries, pad, feed) if pad is not None else None
         if logits is not None:

@@ -90,6 +90,41 @@ def rmsnorm(residual: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype:
     return out
 
 
+def rmsnorm_plain(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm of a plain tensor ``x`` [T, W] (no residual stream), float32 sums: every run of
+    ``weight.shape[0]`` values of a row is normalised by itself and multiplied by ``weight``
+    (float32), so a weight as long as a head normalises every head of a row.  ``x`` may be a view
+    whose rows are a stride apart (the q columns of a q/k/v row); ``out`` may be ``x``."""
+    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
+        raise KernelError("rmsnorm_plain x: must be a 2-d tensor on the GPU whose rows are contiguous")
+    _need(weight, "rmsnorm_plain weight", dtype=torch.float32, ndim=1)
+    t, w = x.shape
+    width = weight.shape[0]
+    if width == 0 or w % width:
+        raise KernelError(f"rmsnorm_plain: rows of {w} values are not whole runs of {width}")
+    if out is None:
+        out = torch.empty((t, w), dtype=x.dtype, device=x.device)
+    if out.shape != x.shape or out.dtype != x.dtype or out.stride(1) != 1 or not out.is_cuda:
+        raise KernelError("rmsnorm_plain out: must have the shape and type of x and contiguous rows")
+    check(load().fsie_rmsnorm_plain(x.data_ptr(), x.stride(0), weight.data_ptr(), out.data_ptr(), out.stride(0), t,
+                                    w // width, width, float(eps), dtype_code(x.dtype), _stream()))
+    return out
+
+
+def zero_rows(table: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+    """``table[slots[i]] = 0`` for every non-negative entry of ``slots`` (int32); rows are whole
+    multiples of four bytes."""
+    _need(table, "zero_rows table")
+    _need(slots, "zero_rows slots", dtype=torch.int32, ndim=1)
+    if table.dim() < 1:
+        raise KernelError("zero_rows: the table needs a first dimension of slots")
+    row_bytes = (table.numel() // max(table.shape[0], 1)) * table.element_size()
+    if row_bytes % 4:
+        raise KernelError(f"zero_rows: rows of {row_bytes} bytes are not whole 4-byte words")
+    check(load().fsie_zero_rows(table.data_ptr(), slots.data_ptr(), slots.shape[0], row_bytes, table.shape[0], _stream()))
+    return table
+
+
 def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(x[:, 0::2]) * x[:, 1::2] for x [T, 2I] (gate and up interleaved)."""
     _need(x, "swiglu input", ndim=2)

@@ -9,9 +9,11 @@ Kinds and their interfaces (``ctx`` is the step's ``StepContext``):
   Norm             ``normed = norm(hidden)``; ``norm.rows(hidden, rows)`` for chosen rows.
                    ``hidden`` is a ``HiddenState``: the float32 residual stream plus a pending
                    delta that the next norm folds in (fused residual sum + norm).
+                   ``norm.plain(x)`` normalises a plain tensor (an output before it is added,
+                   the heads of q and k).
   Mixer            ``y = mixer.forward(x, ctx, cache)``; ``cache_need()`` says what it keeps per
-                   request: a ``PagedNeed`` (entries per token), a ``StateNeed`` (fixed size) or
-                   nothing; ``planner()`` may name per-step index tables it wants built on the host.
+                   request: a need of ``cache.needs`` (``PagedNeed``: keys and values per token,
+                   ``StateNeed``: fixed size, or one of its own that owns its memory) or nothing; ``planner()`` may name per-step index tables it wants built on the host.
   FeedForward      ``y = ffn.forward(x, ctx)``.
   PositionEncoding ``pos.apply(qkv, n_heads, n_kv, head_dim, ctx, store)`` rotates/marks q and k
                    in place and hands k and v to the cache through ``store``.
@@ -57,7 +59,9 @@ class Part:
     # True if the part takes everything that changes from step to step from device tensors (its
     # input and the context's device tables, never ctx.host) and never waits for the device, so
     # that a captured graph of a decode step can be replayed.  A model is replayed from graphs
-    # only if every part of every layer says so.
+    # only if every part of every layer says so.  A step is executed exactly once, also the one
+    # that captures a graph (the warm-up before a capture runs on rows of no request), so a part
+    # whose cache is a running state may set it.
     graph_safe = False
 
     def param_decls(self) -> Dict[str, ParamDecl]:
@@ -76,6 +80,12 @@ class Norm(Part):
         raise NotImplementedError
 
     def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        raise NotImplementedError
+
+    def plain(self, x: torch.Tensor) -> torch.Tensor:
+        """The norm of a plain tensor [T, W], away from the residual stream: a mixer's or a
+        feed-forward's output before it is added (sandwich and post-norm arrangements), or the
+        heads of q and k (a norm as wide as a head normalises every head of a row)."""
         raise NotImplementedError
 
 

@@ -35,3 +35,6 @@ class RMSNorm(Norm):
 
     def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
         return ops.rmsnorm(hidden.residual, self.weight, self.eps, out_dtype, delta=hidden.delta, rows=rows)
+
+    def plain(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.rmsnorm_plain(x, self.weight, self.eps)
