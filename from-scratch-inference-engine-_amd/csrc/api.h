@@ -102,6 +102,29 @@ int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const void* k_pool,
 int fsie_attention_mfma_tiles(int head_dim, int large);
 int fsie_attention_mfma_max_waves(int head_dim);
 
+// ---- an entry point that allocates nothing --------------------------------------------------
+// It has no counterpart in the reference.  It is for callers that cannot allocate device memory:
+// code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+//
+// fsie_attention_scalar / fsie_attention_mfma (small items) followed by fsie_attention_merge, as one
+// call, with the partial records of the key splits kept in a buffer of FSIE_STATIC_SCRATCH_BYTES
+// that the library itself holds on every GPU it runs on (a file-scope device array; nothing is
+// allocated or freed, here or in any routine called from here).  The caller passes the inputs, the
+// tables and the output as for those entry points; `n_partial_slots` is one more than the largest
+// partial slot that `items` and `merges` name (slot = one query token of one split); a step that
+// needs more than the buffer holds is refused with an error, never computed.  `mfma` != 0: the
+// matrix-core kernel (bfloat16), else the float32-arithmetic kernel.  Every call on a GPU uses
+// that GPU's one buffer, which keeps the last call's contents: calls that overlap on one GPU
+// (different streams, or threads) race; calls on one stream are ordered and safe.  Nothing needs
+// clearing between calls: an item writes every record that a merge reads.
+#define FSIE_STATIC_SCRATCH_BYTES (16 * 1024 * 1024)
+int64_t fsie_static_scratch_bytes(void);
+int fsie_attention_split_static(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
+                                const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,
+                                const int32_t* merges, int n_merges, int n_partial_slots, void* out, int n_heads,
+                                int n_kv, int head_dim, int page_size, int window, float scale, int dtype, int mfma,
+                                int waves, hipStream_t stream);
+
 int fsie_sample(const float* logits, int n_rows, int vocab, const float* temperature, const int32_t* top_k,
                 const float* top_p, const double* uniform, int32_t* out, hipStream_t stream);
 

@@ -55,6 +55,9 @@ _SIGNATURES = {
     "fsie_attention_mfma_tiles": ([c_int, c_int], c_int),
     "fsie_attention_merge": ([_P, _P, c_int, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_attention_scalar_tile_tokens": ([c_int, c_int], c_int),
+    "fsie_static_scratch_bytes": ([], c_int64),
+    "fsie_attention_split_static": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, c_int, c_int, _P, c_int, c_int,
+                                     c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P], c_int),
     "fsie_sample": ([_P, c_int, c_int, _P, _P, _P, _P, _P, _P], c_int),
 }
 

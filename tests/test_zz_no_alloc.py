@@ -1,0 +1,74 @@
+"""The entry point that allocates nothing (split-key attention and its merge with the partial
+records in the library's own buffer), called through ctypes, against the existing entry points
+(attention with a caller's workspace, then the merge) on two calls in a row, the second with a
+smaller input."""
+
+import ctypes
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _existing(ops, case, heads, kv, hd, mfma):
+    q = case["q"].cuda()
+    plan = case["plan"]
+    t = q.shape[0]
+    out = torch.zeros((t, heads * hd), dtype=q.dtype).cuda()
+    partials = torch.empty(max(plan["n_partial"], 1) * heads * (hd + 2), dtype=torch.float32).cuda()
+    items = torch.from_numpy(plan["items"]).cuda()
+    pools = (case["k_pool"].cuda(), case["v_pool"].cuda(), case["tables"].cuda())
+    args = (items, plan["n_small"], out, partials, heads, kv, hd, None, 1.0 / math.sqrt(hd), t)
+    if mfma:
+        ops.attention_mfma(q, heads * hd, *pools, *args, large=False, waves=plan["waves"])
+    else:
+        ops.attention_scalar(q, heads * hd, *pools, *args)
+    ops.attention_merge(partials, torch.from_numpy(plan["merges"]).cuda(), plan["n_merges"], out, heads, hd)
+    return out
+
+
+def _static(ops, case, heads, kv, hd, mfma, n_partial_slots=None):
+    lib = ops.load()
+    q = case["q"].cuda()
+    plan = case["plan"]
+    t = q.shape[0]
+    out = torch.zeros((t, heads * hd), dtype=q.dtype).cuda()
+    items = torch.from_numpy(plan["items"]).cuda()
+    merges = torch.from_numpy(plan["merges"]).cuda()
+    k_pool, v_pool, tables = case["k_pool"].cuda(), case["v_pool"].cuda(), case["tables"].cuda()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    rc = lib.fsie_attention_split_static(
+        q.data_ptr(), heads * hd, k_pool.data_ptr(), v_pool.data_ptr(), tables.data_ptr(), tables.shape[1],
+        items.data_ptr(), plan["n_small"], merges.data_ptr(), plan["n_merges"],
+        plan["n_partial"] if n_partial_slots is None else n_partial_slots, out.data_ptr(), heads, kv, hd,
+        k_pool.shape[2], 0, ctypes.c_float(1.0 / math.sqrt(hd)), 1 if q.dtype == torch.bfloat16 else 0, int(mfma),
+        plan["waves"], torch.cuda.current_stream().cuda_stream)
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+    return rc, out
+
+
+@pytest.mark.parametrize("dtype, mfma", [(torch.bfloat16, True), (torch.float32, False)])
+def test_split_attention_in_the_librarys_own_buffer(dtype, mfma):
+    from from_scratch_inference_engine_amd import ops
+    from test_kernels_gpu import paged_case
+
+    heads, kv, hd, page = 28, 4, 128, 16
+    first = [(2500, 1), (600, 1), (40, 1), (1300, 2)]
+    second = [(700, 1)]
+    for seqs, seed in ((first, 1), (second, 2)):
+        case = paged_case(seqs, heads, kv, hd, page, dtype, seed=seed, scalar=not mfma)
+        plan = case["plan"]
+        assert plan["mfma"] == mfma and plan["n_merges"] > 0 and plan["n_large"] == 0
+        want = _existing(ops, case, heads, kv, hd, mfma)
+        rc, got = _static(ops, case, heads, kv, hd, mfma)
+        assert rc == 0, ops.load().fsie_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"{seqs}: the two entry points give other bits"
+        assert got.float().abs().max() > 0
+    # more partial records than the buffer holds: refused, nothing runs
+    slots = ops.load().fsie_static_scratch_bytes() // (heads * (hd + 2) * 4) + 1
+    rc, _ = _static(ops, case, heads, kv, hd, mfma, n_partial_slots=slots)
+    assert rc != 0 and b"the library's buffer" in ops.load().fsie_last_error()
