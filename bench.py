@@ -3,10 +3,11 @@
     python bench.py --gpus 1 --steps K --warmup W
 
 A step is one decode step of the whole batch through the engine (scheduler, step function,
-sampling).  The default run has the layer sizes of BASELINE.json's configs[2], a batch of 8
-requests with 512-token prompts, and times K decode steps after W warm-up steps.  One JSON line
-is printed: decoded tokens a second, the prefill of 2,048 tokens, the decode step against the
-HBM roofline, and decode at batch 1 and 64.
+sampling).  The default run has 28 layers of hidden 3584 / intermediate 18944 with 28 query and 4
+key/value heads of 128 and a vocabulary of 152,064, a batch of 8 requests with 512-token prompts,
+and times K decode steps after W warm-up steps.  One JSON line is printed: decoded tokens a
+second, the prefill of 2,048 tokens, the decode step against the HBM roofline, decode at batch 1
+and 64, and the time of each class of kernels of a decode step.
 """
 
 from __future__ import annotations
@@ -32,7 +33,7 @@ QWEN25_7B = {
 }
 
 
-# the other shapes that BASELINE.json lists (configs[3] and [4]); the default run is configs[2]
+# the two larger shapes: 48 layers of 5120 / 13824 and 64 layers of 5120 / 27648, 40 query and 8 key/value heads
 QWEN25_14B = dict(QWEN25_7B, hidden_size=5120, num_hidden_layers=48, num_attention_heads=40, num_key_value_heads=8,
                   intermediate_size=13824, rms_norm_eps=1e-5, max_position_embeddings=8192)
 QWEN25_32B = dict(QWEN25_14B, num_hidden_layers=64, intermediate_size=27648, max_position_embeddings=16384)
@@ -63,8 +64,106 @@ def decode_bytes(c, layers: int, batch: int, context: float, itemsize: int) -> f
     return weights + cache
 
 
+def kernel_classes(runner, cfg, batch: int, prompt_len: int, itemsize: int) -> dict:
+    """Time of each class of kernels of one decode step: the calls of an eagerly run step are
+    recorded (kernel, operands), and each class's calls, over all layers with each layer's own
+    weights, are captured into a graph of their own and timed with events around its replays.
+    GB/s = the weights (for attention: the live cache) the class reads once a step / its time."""
+    import torch
+
+    from from_scratch_inference_engine_amd import ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.parts import linear as linear_module
+
+    h, inter, v = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    q = cfg.num_attention_heads * cfg.head_dim
+
+    def matrix_class(w):
+        n, k = w.shape
+        if n == v:
+            return "lm_head"
+        if n == 2 * inter:
+            return "gate_up"
+        if k == inter:
+            return "down"
+        if n == q + 2 * cfg.num_key_value_heads * cfg.head_dim:
+            return "qkv"
+        return "o" if (n, k) == (h, q) else "other"
+
+    classify = {
+        "gemm_mfma_skinny_rope": lambda a, k: "qkv", "rope_kv_write": lambda a, k: "qkv", "bias_add": lambda a, k: "qkv",
+        "attention_mfma": lambda a, k: "attention", "attention_mfma_lds": lambda a, k: "attention",
+        "attention_scalar": lambda a, k: "attention", "attention_merge": lambda a, k: "attention",
+        "gemm_mfma_skinny": lambda a, k: matrix_class(a[1]), "gemm_mfma_wide": lambda a, k: matrix_class(a[1]),
+        "gemm": lambda a, k: matrix_class(a[1]), "library_mm": lambda a, k: matrix_class(a[1]),
+        "swiglu": lambda a, k: "gate_up", "rmsnorm": lambda a, k: "norms", "embedding": lambda a, k: "other",
+        "rope_table": lambda a, k: "other", "residual_add": lambda a, k: "other",
+    }
+    calls = []
+    saved = {name: getattr(ops, name) for name in classify}
+    saved_mm = linear_module.library_mm
+
+    def recorder(name, fn):
+        def run(*a, **k):
+            calls.append((classify[name](a, k), fn, a, k))
+            return fn(*a, **k)
+        return run
+
+    gen = torch.Generator().manual_seed(1)
+    caches = [runner.manager.open(f"classes{i}") for i in range(batch)]
+    graphs, runner.graphs = runner.graphs, None
+    try:
+        for c in caches:  # their prompts, then one decode step with the recorder on
+            runner.step([StepEntry(c, torch.randint(0, v, (prompt_len,), generator=gen).tolist(), [])])
+        for name, fn in saved.items():
+            setattr(ops, name, recorder(name, fn))
+        linear_module.library_mm = recorder("library_mm", saved_mm)
+        runner.step([StepEntry(c, [7], [0]) for c in caches])
+    finally:
+        for name, fn in saved.items():
+            setattr(ops, name, fn)
+        linear_module.library_mm = saved_mm
+        runner.graphs = graphs
+    weights = {"qkv": h * (q + 2 * cfg.num_key_value_heads * cfg.head_dim), "o": q * h, "gate_up": 2 * h * inter,
+               "down": h * inter}
+    n_layers = sum(1 for c in calls if c[0] == "qkv" and c[1].__name__ in ("gemm_mfma_skinny_rope", "library_mm", "gemm"))
+    read = {k: n * itemsize * n_layers for k, n in weights.items()}
+    read["lm_head"] = h * v * itemsize
+    read["attention"] = batch * (prompt_len + 1) * 2 * cfg.num_key_value_heads * cfg.head_dim * itemsize * n_layers
+    out = {}
+    side = torch.cuda.Stream()
+    for cls in sorted({c[0] for c in calls}):
+        mine = [(fn, a, k) for c, fn, a, k in calls if c == cls]
+        with torch.cuda.stream(side):
+            for fn, a, k in mine:
+                fn(*a, **k)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for fn, a, k in mine:
+                fn(*a, **k)
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 10
+        e0.record()
+        for _ in range(reps):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        out[cls] = {"ms": round(ms, 4), "launches": len(mine)}
+        if cls in read:
+            out[cls]["GB/s"] = round(read[cls] / ms / 1e6, 1)
+        del graph
+    for c in caches:
+        runner.manager.close(c)
+    return out
+
+
 def other_workload(args, cfg, model, shape_name, layers, full_layers, page) -> int:
-    """The two workloads of BASELINE.json beside the default run; one JSON line each."""
+    """The two workloads beside the default run (many requests of mixed lengths through the
+    scheduler; one long prompt in portions); one JSON line each."""
     import torch
 
     from from_scratch_inference_engine_amd import Engine, SamplingParams
@@ -133,15 +232,16 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (named in config)")
-    ap.add_argument("--shape", choices=sorted(SHAPES), default="7b", help="layer sizes (default: BASELINE.json's configs[2])")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="7b", help="layer sizes (default: 28 layers of 3584 / 18944)")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the time of each class of kernels of a decode step")
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
     ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill"], default="decode",
                     help="decode: the default run.  mixed: --requests prompts of --min-prompt to --max-prompt tokens, "
-                         "--outputs tokens each, through the scheduler (BASELINE.json's configs[3] with --shape 14b).  "
+                         "--outputs tokens each, through the scheduler (made for --shape 14b).  "
                          "long-prefill: one prompt of --prefill-tokens tokens in portions of the token budget "
-                         "(configs[4] with --shape 32b)")
+                         "(made for --shape 32b)")
     ap.add_argument("--requests", type=int, default=32)
     ap.add_argument("--min-prompt", type=int, default=128)
     ap.add_argument("--max-prompt", type=int, default=4096)
@@ -246,6 +346,12 @@ def main() -> int:
             points[f"decode_b{b}"] = b * k / d
             print(f"[bench] decode batch {b}: {d / k * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
 
+    kernels = {}
+    if not args.no_kernels:
+        kernels = kernel_classes(runner, cfg, args.batch, args.prompt_len + args.warmup + args.steps // 2, itemsize)
+        print("[bench] kernel classes of a decode step, ms: "
+              + ", ".join(f"{k} {v['ms']:.3f}" for k, v in kernels.items()), file=sys.stderr, flush=True)
+
     line = {
         "metric": f"decode tok/s @ batch {args.batch}, {shape_name} (with prefill tok/s @ 2,048 tokens, decode @ batch 1/64)",
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -263,6 +369,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
                      "frac": achieved / (HBM_BYTES_PER_S / 1e9)},
         "points": points,
+        "kernels": kernels,
     }
     print(json.dumps(line))
     return 0

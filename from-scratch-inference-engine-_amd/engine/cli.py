@@ -25,6 +25,8 @@ def _common(p: argparse.ArgumentParser) -> None:
     p.add_argument("--num-blocks", type=int, default=2048)
     p.add_argument("--max-batch", type=int, default=256)
     p.add_argument("--max-tokens-per-step", type=int, default=2048)
+    p.add_argument("--prefill-chunk", type=int, default=None,
+                   help="longest portion of a prompt in one step (default: the step's token budget)")
     p.add_argument("--max-tokens", type=int, default=64)
     p.add_argument("--temperature", type=float, default=0.0)
     p.add_argument("--top-k", type=int, default=0)
@@ -49,12 +51,12 @@ def _llm(args):
             raw = json.load(f)
         return LLM.from_config(raw, args.random_weights, block_size=args.block_size, num_blocks=args.num_blocks,
                                seed=args.seed, max_batch=args.max_batch, dtype=args.dtype,
-                               max_tokens_per_step=args.max_tokens_per_step)
+                               max_tokens_per_step=args.max_tokens_per_step, prefill_chunk=args.prefill_chunk)
     if not args.model_dir:
         raise SystemExit("--model-dir (or $ENGINE_MODEL_DIR), or --config with --random-weights, is required")
     return LLM(args.model_dir, block_size=args.block_size, num_blocks=args.num_blocks, seed=args.seed,
                max_batch=args.max_batch, dtype=args.dtype, max_tokens_per_step=args.max_tokens_per_step,
-               tune_gemms=args.tune_gemms)
+               prefill_chunk=args.prefill_chunk, tune_gemms=args.tune_gemms)
 
 
 def _prompts(args, llm):

@@ -9,8 +9,9 @@ does not depend on the batch it shares.
 
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -38,6 +39,29 @@ def uniform_for(seed: int, request_id: int, index: int) -> float:
 class Sampler:
     def __init__(self, seed: int = 0):
         self.seed = int(seed)
+        # the parameters of a step's rows travel in one pinned buffer and one copy
+        self._pinned: Optional[torch.Tensor] = None
+        self._copied: Optional[torch.cuda.Event] = None
+
+    def _upload(self, uniform, temperature, top_k, top_p, device):
+        """One host-to-device copy for the four per-row arrays: [uniform float64 | temperature
+        float32 | top_k int32 | top_p float32], each n long; returns their device views."""
+        n = len(uniform)
+        if self._copied is not None:
+            self._copied.synchronize()  # the last copy has read the buffer
+        if self._pinned is None or self._pinned.numel() < 20 * n:
+            self._pinned = torch.empty((max(20 * n, 4096),), dtype=torch.uint8, pin_memory=True)
+        host = self._pinned.numpy()
+        host[:8 * n].view(np.float64)[:] = uniform
+        host[8 * n:12 * n].view(np.float32)[:] = temperature
+        host[12 * n:16 * n].view(np.int32)[:] = top_k
+        host[16 * n:20 * n].view(np.float32)[:] = top_p
+        dev = self._pinned[:20 * n].to(device, non_blocking=True)
+        if self._copied is None:
+            self._copied = torch.cuda.Event()
+        self._copied.record()
+        return (dev[:8 * n].view(torch.float64), dev[8 * n:12 * n].view(torch.float32),
+                dev[12 * n:16 * n].view(torch.int32), dev[16 * n:20 * n].view(torch.float32))
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], request_ids: Sequence[int],
                indices: Sequence[int]) -> List[int]:
@@ -55,10 +79,8 @@ class Sampler:
             raise ValueError("sample: one set of parameters, request id and index per row")
         if all(p.greedy for p in params):
             return ops.sample(logits)
-        dev = logits.device
-        temperature = torch.tensor([max(float(p.temperature), 0.0) for p in params], dtype=torch.float32, device=dev)
-        top_k = torch.tensor([int(p.top_k) for p in params], dtype=torch.int32, device=dev)
-        top_p = torch.tensor([float(p.top_p) for p in params], dtype=torch.float32, device=dev)
-        uniform = torch.tensor([uniform_for(self.seed, r, i) for r, i in zip(request_ids, indices)],
-                               dtype=torch.float64, device=dev)
+        uniform, temperature, top_k, top_p = self._upload(
+            [uniform_for(self.seed, r, i) for r, i in zip(request_ids, indices)],
+            [max(float(p.temperature), 0.0) for p in params], [int(p.top_k) for p in params],
+            [float(p.top_p) for p in params], logits.device)
         return ops.sample(logits, temperature, top_k, top_p, uniform)
