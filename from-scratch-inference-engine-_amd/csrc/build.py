@@ -63,11 +63,33 @@ def _writable_dir(path: Path) -> bool:
         return False
 
 
-def build_dirs():
-    """Candidate folders, in the order they are looked at."""
-    local = CSRC / "_build"
+def private_tmp_dir(name: str):
+    """``<tmp>/<name>-<uid>``, made with mode 0700 if it is not there; None unless it belongs to
+    this user and nobody else may write to it.  The system's temporary folder is shared: a library
+    or a file of results found in a folder that another user could have made or filled is not
+    loaded."""
     uid = os.getuid() if hasattr(os, "getuid") else 0
-    return [local, Path(tempfile.gettempdir()) / f"fsie-build-{uid}"]
+    path = Path(tempfile.gettempdir()) / f"{name}-{uid}"
+    try:
+        path.mkdir(mode=0o700, exist_ok=True)
+        st = path.lstat()
+    except OSError:
+        return None
+    import stat
+
+    if not stat.S_ISDIR(st.st_mode) or (hasattr(os, "getuid") and st.st_uid != uid) or (st.st_mode & 0o022):
+        return None
+    return path
+
+
+def build_dirs():
+    """Candidate folders, in the order they are looked at: the checkout's own, then a private
+    per-user folder under the system's temporary directory."""
+    dirs = [CSRC / "_build"]
+    tmp = private_tmp_dir("fsie-build")
+    if tmp is not None:
+        dirs.append(tmp)
+    return dirs
 
 
 def find_built():
@@ -98,7 +120,11 @@ def build(verbose: bool = True) -> Path:
     srcs = sources()
     if verbose:
         _say(f"compiling {len(srcs)} sources for {ARCH} into {out_dir}")
-    objs = [out_dir / (s.stem + ".o") for s in srcs]
+    # objects go to a folder of this process, so that two first builds at once (a test run beside a
+    # replay) do not write each other's files; only the finished library is moved into place
+    obj_dir = out_dir / f"obj{os.getpid()}"
+    obj_dir.mkdir(exist_ok=True)
+    objs = [obj_dir / (s.stem + ".o") for s in srcs]
     workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "8"))))
     failed = []
     with ThreadPoolExecutor(max_workers=workers) as pool:
@@ -108,11 +134,13 @@ def build(verbose: bool = True) -> Path:
             elif verbose:
                 _say(f"  {src.name} ({dt:.1f} s)")
     if failed:
+        shutil.rmtree(obj_dir, ignore_errors=True)
         text = "\n".join(f"--- {s.name}\n{err}" for s, err in failed)
         raise RuntimeError(f"hipcc failed:\n{text}")
     tmp = out_dir / (LIB_NAME + f".tmp{os.getpid()}")
     link = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *map(str, objs), "-o", str(tmp)],
                           capture_output=True, text=True)
+    shutil.rmtree(obj_dir, ignore_errors=True)
     if link.returncode != 0:
         raise RuntimeError(f"hipcc link failed:\n{link.stderr}")
     os.replace(tmp, out_dir / LIB_NAME)

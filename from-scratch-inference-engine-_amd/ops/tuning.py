@@ -14,10 +14,11 @@ them, or the heuristic.
 
 from __future__ import annotations
 
-import os
-import tempfile
+import hashlib
 
 import torch
+
+from ..csrc.build import private_tmp_dir
 
 _TUNED_ROWS, _TUNED_MAX_ROWS = 256, 4096
 _TUNED_DECODE_ROWS, _TUNED_DECODE_MAX = 16, 64   # decode batches are padded to these row counts ...
@@ -32,10 +33,16 @@ def enable_library_tuning(max_ms_per_candidate: int = 30, iterations: int = 10) 
     tunable.tuning_enable(False)
     tunable.set_max_tuning_duration(int(max_ms_per_candidate))
     tunable.set_max_tuning_iterations(int(iterations))
-    # torch also keeps the results in a file; it goes to the temporary folder, under the user's id
-    # (the working directory may be read-only), and a later process starts from it
-    name = f"fsie-tunableop-{os.getuid()}.csv"
-    tunable.set_filename(os.path.join(tempfile.gettempdir(), name))
+    # torch also keeps the results in a file, from which a later process starts: it goes to a
+    # private per-user folder under the temporary directory (the working directory may be
+    # read-only), named for the device and the library versions the timings belong to; without
+    # such a folder the results stay in the process
+    folder = private_tmp_dir("fsie-tunableop")
+    if folder is not None:
+        what = f"{torch.cuda.get_device_name(0) if torch.cuda.is_available() else 'none'}|{torch.__version__}|{torch.version.hip}"
+        tunable.set_filename(str(folder / f"results-{hashlib.sha256(what.encode()).hexdigest()[:12]}.csv"))
+    elif hasattr(tunable, "write_file_on_exit"):
+        tunable.write_file_on_exit(False)
     _state["on"] = True
 
 
