@@ -134,9 +134,9 @@ class CacheManager:
                 want[g] += k
         return all(w <= a.num_free for w, a in zip(want, self.allocators))
 
-    def reserve(self, rc: RequestCache, n_tokens: int) -> None:
+    def reserve(self, rc: RequestCache, n_tokens: int) -> List[List[int]]:
         """Grow the block tables to hold ``length + n_tokens``.  Checks every group first, so a
-        failure leaves the request as it was."""
+        failure leaves the request as it was.  Returns, per group, the pages just taken."""
         if rc.closed:
             raise RuntimeError(f"CacheManager: request {rc.request_id!r} is closed")
         if n_tokens < 0:
@@ -147,9 +147,12 @@ class CacheManager:
                 raise OutOfPages(
                     f"CacheManager: group {g} needs {k} pages for request {rc.request_id!r}, "
                     f"{self.allocators[g].num_free} free")
+        fresh: List[List[int]] = [[] for _ in need]
         for g, k in enumerate(need):
             for _ in range(k):
-                rc.tables[g].append(self.allocators[g].allocate())
+                fresh[g].append(self.allocators[g].allocate())
+            rc.tables[g].extend(fresh[g])
+        return fresh
 
     def commit(self, rc: RequestCache, n_tokens: int) -> None:
         """The step wrote ``n_tokens`` entries: advance the length and give back the pages

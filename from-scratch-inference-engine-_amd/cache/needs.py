@@ -15,8 +15,11 @@ Two ways of keeping:
   per request (``per_token = False``)  memory of fixed size in the request's *slot*, zero when the
       request starts.
 
-Interface (``units`` = pages of the pool + 1, or slots + 1: the last one belongs to no request and
-is where the rows that pad a batch read and write):
+Interface (``units``: for a per-token need the pages of the pool + 2: unit 0 is the *null page*,
+which nothing ever writes and which a table entry of -1 stands for (a kernel that reads a key
+without a page reads zeros there), units 1.. are the allocator's pages, the last one is the spare
+page where the rows that pad a batch read and write; the step's tables name units.  For a
+per-request need: the slots + 1, the last one the spare slot):
 
   allocate(n_caches, units, page_size, device, dtype) -> store    anything the need likes
   view(store, plane, ctx, group, writes) -> what the mixer's ``forward`` gets as ``cache``;
@@ -26,6 +29,10 @@ is where the rows that pad a batch read and write):
   store_bytes(store) -> int
   reset(store, ctx)                   per-request needs: zero the slots ``ctx.reset_slots`` names
       (int32 [requests], -1 = leave alone) with work queued on the current stream
+  clear_fresh(store, pages)           per-token needs: zero the units ``pages`` (int32 on the device,
+      -1 = none) that the step has just taken from the pool, in every plane, before anything is
+      written: what an earlier request left in a page (a NaN, an overflow) must not reach the
+      request that gets the page next through a probability of zero times a stale value
 """
 
 from __future__ import annotations
@@ -52,6 +59,9 @@ class CacheNeed:
 
     def reset(self, store, ctx) -> None:
         """Per-request needs only."""
+
+    def clear_fresh(self, store, pages) -> None:
+        """Per-token needs only."""
 
 
 class LayerCache:
@@ -93,8 +103,9 @@ class PagedNeed(CacheNeed):
     def allocate(self, n_caches, units, page_size, device, dtype):
         import torch
 
-        # The pools start as zeros and only ever hold what the kernels wrote: a probability of
-        # zero times a slot that no token has filled yet must be zero, not NaN.
+        # The pools start as zeros, a page is zeroed again when a request takes it, and the null
+        # page is never written: a probability of zero times a slot that no token of this request
+        # has filled is zero, whatever an earlier request computed.
         k = torch.zeros((n_caches, units, self.n_kv_heads, page_size, self.head_dim), dtype=dtype, device=device)
         v = torch.zeros((n_caches, units, self.n_kv_heads, self.head_dim, page_size), dtype=dtype, device=device)
         return k, v, page_size
@@ -105,6 +116,11 @@ class PagedNeed(CacheNeed):
         lc.k_pool, lc.v_pool, lc.page_size = store[0][plane], store[1][plane], store[2]
         lc.block_tables, lc.slots, lc.group = ctx.block_tables[group], ctx.slots[group], group
         return lc
+
+    def clear_fresh(self, store, pages) -> None:
+        from .. import ops
+
+        ops.zero_pages(store[0], store[1], pages)
 
     def bytes_per_token(self, dtype) -> int:
         import torch

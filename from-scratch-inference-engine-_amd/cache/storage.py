@@ -31,9 +31,11 @@ class CacheLayout:
 class CacheStorage:
     """Asks every need for its memory and for the views; knows no layout itself.
 
-    The last page of a pool and the last state slot belong to no request (the allocators do not
-    know them): they are where the rows that pad a batch to a captured graph's size read and
-    write."""
+    A pool has two pages more than its allocator: unit 0 is the null page (never written; what a
+    table entry of -1 reads), the allocator's page p is unit p + 1, and the last unit is the spare
+    page, which, like the last state slot, belongs to no request: the rows that pad a batch to a
+    captured graph's size read and write there.  ``spare_pages`` names the spare page as the
+    allocator would (its number of pages): the step's tables turn page ids into units."""
 
     def __init__(self, layout: CacheLayout, manager: CacheManager, device, dtype):
         self.layout = layout
@@ -42,7 +44,7 @@ class CacheStorage:
         self.dtype = dtype
         self.spare_pages: List[int] = [manager.allocators[g].num_pages for g in range(len(layout.paged_groups))]
         self.spare_slot = manager.max_requests
-        self.group_stores = [need.allocate(len(layout.group_caches[g]), self.spare_pages[g] + 1, self.page_size,
+        self.group_stores = [need.allocate(len(layout.group_caches[g]), self.spare_pages[g] + 2, self.page_size,
                                            device, dtype)
                              for g, need in enumerate(layout.paged_groups)]
         self.state_stores = {cid: need.allocate(1, manager.max_requests + 1, self.page_size, device, dtype)
@@ -57,6 +59,12 @@ class CacheStorage:
         stream like the rest of the step, from the step's own tables)."""
         for cid, store in self.state_stores.items():
             self.layout.state_caches[cid].reset(store, ctx)
+
+    def clear_fresh(self, ctx) -> None:
+        """Zero the pages that this step's requests have just taken from the pools."""
+        for g, need in enumerate(self.layout.paged_groups):
+            if ctx.fresh_pages[g] is not None:
+                need.clear_fresh(self.group_stores[g], ctx.fresh_pages[g])
 
     def view(self, cache_id: int, ctx, writes: bool):
         if cache_id in self.state_stores:

@@ -48,6 +48,9 @@ int fsie_rmsnorm_plain(const void* x, int64_t x_stride, const float* weight, voi
                        int groups, int width, float eps, int dtype, hipStream_t stream);
 // Rows slots[0..n) of a table of n_slots rows of row_bytes set to zero; a negative slot is skipped.
 int fsie_zero_rows(void* table, const int32_t* slots, int n, int64_t row_bytes, int n_slots, hipStream_t stream);
+// Pages pages[0..n) (negative: skipped) of two pools of [planes][n_pages][page_bytes] set to zero.
+int fsie_zero_pages(void* pool_a, void* pool_b, const int32_t* pages, int n, int planes, int n_pages,
+                    int64_t page_bytes, hipStream_t stream);
 int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream);
 int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream);
 int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream);

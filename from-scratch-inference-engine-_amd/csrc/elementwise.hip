@@ -275,6 +275,23 @@ __global__ void zero_rows_kernel(uint32_t* __restrict__ table, const int32_t* __
         row[i] = 0u;
 }
 
+// Pages pages[i] (negative = none) of two pools set to zero in every plane: the pools are
+// [planes][n_pages][page_words] words each.
+template <typename V>
+__global__ void zero_pages_kernel(uint32_t* __restrict__ a, uint32_t* __restrict__ b, const int32_t* __restrict__ pages,
+                                  int64_t page_words, int64_t plane_words, int n_pages) {
+    const int page = pages[blockIdx.x];
+    if (page < 0 || page >= n_pages) return;
+    uint32_t* pool = (blockIdx.z & 1) ? b : a;
+    V* dst = reinterpret_cast<V*>(pool + (blockIdx.z >> 1) * plane_words + static_cast<int64_t>(page) * page_words);
+    const int64_t n = page_words / static_cast<int64_t>(sizeof(V) / 4);
+    V zero;
+    memset(&zero, 0, sizeof(V));
+    for (int64_t i = static_cast<int64_t>(blockIdx.y) * blockDim.x + threadIdx.x; i < n;
+         i += static_cast<int64_t>(gridDim.y) * blockDim.x)
+        dst[i] = zero;
+}
+
 // RMSNorm of a plain tensor, no residual stream: every row of x holds `groups` runs of `width`
 // values, each normalised by itself (a whole row, or the heads of a row); one wave a run.
 template <typename T>
@@ -310,6 +327,30 @@ extern "C" int fsie_zero_rows(void* table, const int32_t* slots, int n, int64_t 
     const dim3 grid(n, static_cast<unsigned>(ceil_div64(words, 4 * kThreads) > 64 ? 64 : ceil_div64(words, 4 * kThreads)));
     zero_rows_kernel<<<grid, kThreads, 0, stream>>>(static_cast<uint32_t*>(table), slots, words, n_slots);
     FSIE_CHECK_LAUNCH("zero_rows");
+    return 0;
+}
+
+extern "C" int fsie_zero_pages(void* pool_a, void* pool_b, const int32_t* pages, int n, int planes, int n_pages,
+                               int64_t page_bytes, hipStream_t stream) {
+    FSIE_REQUIRE(n >= 0 && planes > 0 && n_pages > 0 && page_bytes > 0 && page_bytes % 4 == 0,
+                 "zero_pages: bad sizes n=%d planes=%d pages=%d page_bytes=%lld (pages are whole 4-byte words)", n,
+                 planes, n_pages, static_cast<long long>(page_bytes));
+    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(pool_a) % 16 == 0 && reinterpret_cast<uintptr_t>(pool_b) % 16 == 0,
+                 "zero_pages: the pools must be 16-byte aligned");
+    if (n == 0) return 0;
+    const int64_t page_words = page_bytes / 4;
+    const bool quads = page_bytes % 16 == 0;
+    const int64_t chunks = ceil_div64(quads ? page_words / 4 : page_words, kThreads);
+    const dim3 grid(n, static_cast<unsigned>(chunks > 16 ? 16 : chunks), 2 * planes);
+    if (quads) {
+        zero_pages_kernel<uint4><<<grid, kThreads, 0, stream>>>(static_cast<uint32_t*>(pool_a), static_cast<uint32_t*>(pool_b),
+                                                               pages, page_words, page_words * n_pages, n_pages);
+    } else {
+        zero_pages_kernel<uint32_t><<<grid, kThreads, 0, stream>>>(static_cast<uint32_t*>(pool_a),
+                                                                  static_cast<uint32_t*>(pool_b), pages, page_words,
+                                                                  page_words * n_pages, n_pages);
+    }
+    FSIE_CHECK_LAUNCH("zero_pages");
     return 0;
 }
 

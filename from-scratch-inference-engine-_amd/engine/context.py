@@ -24,6 +24,8 @@ class StepEntry:
     cache: RequestCache
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    # set by the step function: per group, the pages it has just reserved for these tokens
+    fresh: Sequence[Sequence[int]] = ()
 
 
 def filler_entry(storage, n_tokens: int, page_size: int):
@@ -142,7 +144,8 @@ class StepContext:
     ``token_ids`` [T], ``positions`` [T], ``want_rows`` [wanted], ``seq_slots`` [n] (state slot of
     each request), ``reset_slots`` [n] (the same for a request that starts in this step, else -1),
     ``q_starts`` [n+1], ``past_lens`` [n]; per paged group ``block_tables[g]``
-    [n, pages] and ``slots[g]`` [T]; ``host`` holds the same as Python lists/arrays.
+    [n, pages] (units of the pool: page + 1; -1 = none, which reads the null page) and ``slots[g]``
+    [T]; ``host`` holds the same as Python lists/arrays.
     ``plan(planner)`` gives the tables a part asked for through its ``planner()``."""
 
     def __init__(self, host: HostBatch, compute_dtype: torch.dtype, device):
@@ -157,6 +160,7 @@ class StepContext:
         self.partial_sums_ok = False
         self.block_tables: List[torch.Tensor] = []
         self.slots: List[torch.Tensor] = []
+        self.fresh_pages: List[Optional[torch.Tensor]] = []  # per group: units just taken from the pool, or None
         self._plans: Dict[Hashable, SimpleNamespace] = {}
         # what a part computes once per forward pass and its siblings in other layers use again
         # (keyed by whatever identifies it); emptied when a forward pass starts
@@ -192,7 +196,16 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
     i_past = pk.add(np.asarray(host.past_lens, dtype=np.int32))
     ps = manager.page_size
     group_idx = []
+    fresh_idx = []
     for g in range(len(manager.groups)):
+        # pages just taken from the pool (as units: page + 1), for the kernel that zeroes them; a
+        # replayed graph has room for one a request
+        fresh = [p + 1 for e in entries for p in (getattr(e, "fresh", None) or [[]] * (g + 1))[g]]
+        if pad is not None:
+            if len(fresh) > len(entries):
+                raise RuntimeError("more fresh pages than the captured graph has room for")
+            fresh += [-1] * (len(entries) - len(fresh))
+        fresh_idx.append(pk.add(np.asarray(fresh, dtype=np.int32)) if fresh else None)
         max_pages = max([len(e.cache.tables[g]) for e in entries] + [1])
         if pad is not None:
             if max_pages > pad["pages"]:
@@ -201,7 +214,9 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
         table = np.full((len(entries), max_pages), -1, dtype=np.int32)
         slot_map = np.full((host.n_tokens,), -1, dtype=np.int32)
         for s, e in enumerate(entries):
+            # page ids become units of the pool: unit 0 is the null page, page p is unit p + 1
             pages = np.asarray(e.cache.tables[g], dtype=np.int32)
+            pages = np.where(pages >= 0, pages + 1, -1)
             table[s, :pages.size] = pages
             pos = host.positions[host.q_starts[s]:host.q_starts[s + 1]]
             page_of = pages[pos // ps]
@@ -220,6 +235,7 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
     for it, isl in group_idx:
         ctx.block_tables.append(dev[it])
         ctx.slots.append(dev[isl])
+    ctx.fresh_pages = [None if i is None else dev[i] for i in fresh_idx]
     for key, arrays, scalars in plan_idx:
         ctx._plans[key] = SimpleNamespace(**{k: dev[i] for k, i in arrays.items()}, **scalars)
     base = dev[0]._base if dev and dev[0]._base is not None else (dev[0] if dev else None)

@@ -149,6 +149,7 @@ class Model:
         ctx.partial_sums_ok = self.partial_sums_ok
         ctx.memo.clear()  # a captured graph must hold whatever the layers share: nothing is kept from an earlier pass
         storage.reset_states(ctx)  # requests that start in this step find their per-request memory zero
+        storage.clear_fresh(ctx)   # and the pages taken from the pools for this step hold nothing of their last owner
         hidden = HiddenState(spec.embedding.forward(ctx.token_ids))
         for i, call in enumerate(spec.schedule):
             cid = self.call_cache[i]
@@ -215,7 +216,7 @@ class Runner:
         if not self.manager.can_reserve((e.cache, len(e.tokens)) for e in entries):
             raise OutOfPages("step: the batch needs more pages than the pool has free")
         for e in entries:
-            self.manager.reserve(e.cache, len(e.tokens))
+            e.fresh = self.manager.reserve(e.cache, len(e.tokens))
         pad = self.graphs.shape_of(entries) if self.graphs is not None else None
         logits = self.graphs.step(entries, pad, feed) if pad is not None else None
         if logits is not None:

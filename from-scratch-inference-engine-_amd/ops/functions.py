@@ -125,6 +125,19 @@ def zero_rows(table: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
     return table
 
 
+def zero_pages(pool_a: torch.Tensor, pool_b: torch.Tensor, pages: torch.Tensor) -> None:
+    """Pages ``pages`` (int32, negative = none) of two pools [planes, n_pages, ...] of equal page
+    size set to zero in every plane."""
+    _need(pool_a, "zero_pages pool")
+    _need(pool_b, "zero_pages pool", dtype=pool_a.dtype)
+    _need(pages, "zero_pages pages", dtype=torch.int32, ndim=1)
+    if pool_a.dim() < 3 or pool_b.dim() < 3 or pool_a.shape[:2] != pool_b.shape[:2] or pool_a[0, 0].numel() != pool_b[0, 0].numel():
+        raise KernelError(f"zero_pages: pools of shapes {tuple(pool_a.shape)} and {tuple(pool_b.shape)} do not go together")
+    page_bytes = pool_a[0, 0].numel() * pool_a.element_size()
+    check(load().fsie_zero_pages(pool_a.data_ptr(), pool_b.data_ptr(), pages.data_ptr(), pages.shape[0], pool_a.shape[0],
+                                 pool_a.shape[1], page_bytes, _stream()))
+
+
 def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(x[:, 0::2]) * x[:, 1::2] for x [T, 2I] (gate and up interleaved)."""
     _need(x, "swiglu input", ndim=2)

@@ -701,3 +701,39 @@ def test_the_model_finds_one_far_key_through_its_own_tables(tmp_path, dtype):
             pos = [p for p, _ in got[i]]
             helpers.assert_close_to_plain(np.stack([r for _, r in got[i]]), refs[i][pos], dtype,
                                           f"{dtype} graphs={graphs} request {i}")
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_what_an_earlier_request_left_in_its_pages_does_not_reach_the_next(model_dirs, dtype):
+    """Every page of the pools is filled with NaN, as a request whose activations overflowed would
+    leave them (all but the null page, which nothing ever writes).  A request that takes such a
+    page finds it zeroed, and keys it has no page for are read from the null page: a probability
+    of zero times what lies there is zero.  Portions, decoded tokens and a batch padded to a
+    graph's size (whose filler rows live in the spare page) all give the plain model's logits."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    model = load_model(model_dirs["A"], dtype=dtype)
+    seqs = [helpers.token_ids(256, n, 1300 + n) for n in (37, 22, 9)]
+    refs = [plain.forward_dir(model_dirs["A"], ids).numpy() for ids in seqs]
+    for graphs in (False, True):
+        runner = Runner(model, page_size=4, num_pages=24, max_requests=4, use_graphs=graphs)
+        k, v, _ = runner.storage.group_stores[0]
+        k[:, 1:] = float("nan")
+        v[:, 1:] = float("nan")
+        caches = [runner.manager.open(i) for i in range(3)]
+        fed = [0, 0, 0]
+        plan = [[(0, 30), (1, 2)], [(0, 1), (1, 13), (2, 3)], [(0, 1), (1, 1), (2, 1)], [(0, 1), (1, 1), (2, 1)],
+                [(0, 4), (1, 5), (2, 4)]]
+        for step in plan:
+            entries = [StepEntry(caches[i], seqs[i][fed[i]:fed[i] + n], list(range(n))) for i, n in step]
+            out = runner.step(entries).float().cpu().numpy()
+            row = 0
+            for i, n in step:
+                helpers.assert_close_to_plain(out[row:row + n], refs[i][fed[i]:fed[i] + n], dtype,
+                                              f"{dtype} graphs={graphs} request {i} at {fed[i]}")
+                row += n
+                fed[i] += n
+        assert fed == [len(s_) for s_ in seqs]
+        assert not torch.isnan(k[:, 0]).any() and (k[:, 0] == 0).all() and (v[:, 0] == 0).all()  # the null page stays empty

@@ -237,7 +237,7 @@ def test_a_per_token_cache_of_one_vector_and_a_sandwich_norm(tmp_path):
     assert layout.group_caches == [[0, 1]] and model.cache_bytes_per_token() == 2 * 4 * 12
     runner = Runner(model, page_size=4, num_pages=14, max_requests=3)
     store = runner.storage.group_stores[0]
-    assert store.shape == (2, 15, 4, 12) and store.dtype == torch.float32 and runner.storage.bytes() == store.numel() * 4
+    assert store.shape == (2, 16, 4, 12)  # null page, 14 pages, spare page and store.dtype == torch.float32 and runner.storage.bytes() == store.numel() * 4
     assert runner.max_position == 64  # read through the typed configuration, whatever the key is called
     seqs = {"a": helpers.token_ids(83, 30, 1), "b": helpers.token_ids(83, 11, 2), "c": helpers.token_ids(83, 17, 3)}
     ref = {k: plain_toy(raw, w, ids) for k, ids in seqs.items()}
