@@ -51,6 +51,8 @@ int fsie_zero_rows(void* table, const int32_t* slots, int n, int64_t row_bytes, 
 // Pages pages[0..n) (negative: skipped) of two pools of [planes][n_pages][page_bytes] set to zero.
 int fsie_zero_pages(void* pool_a, void* pool_b, const int32_t* pages, int n, int planes, int n_pages,
                     int64_t page_bytes, hipStream_t stream);
+// Counter-based random values (the random-weights mode): see elementwise.hip.
+int fsie_random_fill(void* out, int64_t n, uint64_t key, int kind, float std, hipStream_t stream);
 int fsie_swiglu(const void* x, void* out, int n_tokens, int inter, int dtype, hipStream_t stream);
 int fsie_residual_add(float* residual, const void* delta, int64_t total, int dtype, hipStream_t stream);
 int fsie_bias_add(void* y, const float* bias, int rows, int cols, int dtype, hipStream_t stream);

@@ -292,6 +292,38 @@ __global__ void zero_pages_kernel(uint32_t* __restrict__ a, uint32_t* __restrict
         dst[i] = zero;
 }
 
+// Counter-based random values, a pure function of (key, element index): see fsie_random_fill.
+__device__ __forceinline__ uint64_t splitmix_output(uint64_t key, uint64_t number) {
+    uint64_t x = key + (number + 1) * 0x9E3779B97F4A7C15ull;
+    uint64_t z = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+__global__ void random_fill_kernel(void* __restrict__ out, int64_t n, uint64_t key, int kind, float std) {
+#pragma clang fp contract(off)  // a product and a sum stay two roundings, as on the host
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+         i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const uint64_t a = splitmix_output(key, 2 * static_cast<uint64_t>(i));
+        if (kind == 2) {
+            static_cast<int32_t*>(out)[i] = static_cast<int32_t>((a >> 17) & 0x7FFF);
+            continue;
+        }
+        const uint64_t b = splitmix_output(key, 2 * static_cast<uint64_t>(i) + 1);
+        int total = 0;
+#pragma unroll
+        for (int shift = 0; shift < 64; shift += 16)
+            total += static_cast<int>((a >> shift) & 0xFFFF) + static_cast<int>((b >> shift) & 0xFFFF);
+        // single float32 operations, written out here so that the pragma above covers them (the
+        // library's rounding-mode wrappers are compiled where contraction is allowed): the host
+        // computes the same bits
+        const float z = static_cast<float>(total - 4 * 65535) * __uint_as_float(0x379cc471u);
+        const float v = z * std;
+        const float shifted = v + 1.0f;
+        static_cast<float*>(out)[i] = kind == 1 ? shifted : v;
+    }
+}
+
 // RMSNorm of a plain tensor, no residual stream: every row of x holds `groups` runs of `width`
 // values, each normalised by itself (a whole row, or the heads of a row); one wave a run.
 template <typename T>
@@ -327,6 +359,18 @@ extern "C" int fsie_zero_rows(void* table, const int32_t* slots, int n, int64_t 
     const dim3 grid(n, static_cast<unsigned>(ceil_div64(words, 4 * kThreads) > 64 ? 64 : ceil_div64(words, 4 * kThreads)));
     zero_rows_kernel<<<grid, kThreads, 0, stream>>>(static_cast<uint32_t*>(table), slots, words, n_slots);
     FSIE_CHECK_LAUNCH("zero_rows");
+    return 0;
+}
+
+// out[i] for i in [0, n): kind 0: std * z_i, kind 1: 1 + std * z_i (float32), kind 2: 15 random bits
+// (int32), where z_i is the centred, scaled sum of the eight 16-bit fields of the SplitMix64 outputs
+// number 2i and 2i + 1 of the sequence that starts at `key` (close to a standard normal).
+extern "C" int fsie_random_fill(void* out, int64_t n, uint64_t key, int kind, float std, hipStream_t stream) {
+    FSIE_REQUIRE(n >= 0 && kind >= 0 && kind <= 2, "random_fill: bad arguments n=%lld kind=%d", static_cast<long long>(n), kind);
+    if (n == 0) return 0;
+    const int64_t blocks = ceil_div64(n, kThreads);
+    random_fill_kernel<<<static_cast<unsigned>(blocks > 65536 ? 65536 : blocks), kThreads, 0, stream>>>(out, n, key, kind, std);
+    FSIE_CHECK_LAUNCH("random_fill");
     return 0;
 }
 

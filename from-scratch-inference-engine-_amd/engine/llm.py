@@ -62,13 +62,12 @@ class LLM:
                     max_tokens_per_step: int = 2048, prefill_chunk: Optional[int] = None) -> "LLM":
         """An engine over random weights made from ``config`` (the dictionary of a config.json, or a
         typed configuration) and ``weight_seed``: no folder, no tokenizer, token ids in and out.
-        The weights are those that ``write_random_model`` writes for the same seed (as float32):
-        they are drawn on the host, tensor by tensor, and sent to the device."""
+        The weights are those that ``write_random_model`` writes for the same seed (as float32)."""
         from ..models import parse_config
 
         typed = parse_config(config) if isinstance(config, dict) else config
         llm = cls.__new__(cls)
-        llm.model = Model.from_random(typed, weight_seed, dtype=dtype, device=device, as_written=True)
+        llm.model = Model.from_random(typed, weight_seed, dtype=dtype, device=device)
         llm.engine = Engine(llm.model, block_size, num_blocks, seed, max_batch,
                             max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk)
         llm.eos_id = eos_id

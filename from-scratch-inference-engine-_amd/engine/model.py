@@ -110,18 +110,15 @@ class Model:
         return model
 
     @classmethod
-    def from_random(cls, config: ModelConfig, seed: int = 0, dtype="bfloat16", device="cuda:0",
-                    as_written: bool = False) -> "Model":
-        """Random weights without a folder.  By default they are drawn on the device (gigabytes in
-        a fraction of a second; the device's generator gives other numbers than the host's).
-        ``as_written=True`` draws them on the host instead, tensor by tensor: the very values that
-        ``write_random_model`` writes for this seed (as float32), at the host generator's pace."""
+    def from_random(cls, config: ModelConfig, seed: int = 0, dtype="bfloat16", device="cuda:0") -> "Model":
+        """Random weights without a folder, drawn on the device (gigabytes in a fraction of a
+        second): the very values that ``write_random_model`` writes for this configuration and
+        seed (the generator is a function of seed, tensor name and element index)."""
         device = _require_gpu(device)
         model = cls(build_model_spec(config), dtype, device)
         specs = expected_tensors(model.spec.bindings)
-        where = "cpu" if as_written else device
         model.weight_bytes = fill_parts(
-            model.spec.bindings, lambda name: random_tensor(specs[name], seed, torch.float32, device=where),
+            model.spec.bindings, lambda name: random_tensor(specs[name], seed, torch.float32, device=device),
             model.dtype, device)
         model._prepare()
         return model

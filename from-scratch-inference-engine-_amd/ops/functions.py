@@ -138,6 +138,18 @@ def zero_pages(pool_a: torch.Tensor, pool_b: torch.Tensor, pages: torch.Tensor) 
                                  pool_a.shape[1], page_bytes, _stream()))
 
 
+def random_fill(out: torch.Tensor, key: int, init: str, std: float = 0.0) -> torch.Tensor:
+    """Fill ``out`` (float32, or int32 for ``init == 'int'``) with the counter-based random values
+    of the sequence ``key``: ``std * z`` ('weight', 'bias'), ``1 + std * z`` ('norm'), 15 random
+    bits ('int'); element i is a function of (key, i) alone."""
+    kind = {"weight": 0, "bias": 0, "norm": 1, "int": 2}.get(init)
+    if kind is None:
+        raise KernelError(f"random_fill: unknown init '{init}'")
+    _need(out, "random_fill out", dtype=torch.int32 if kind == 2 else torch.float32)
+    check(load().fsie_random_fill(out.data_ptr(), out.numel(), int(key) & ((1 << 64) - 1), kind, float(std), _stream()))
+    return out
+
+
 def swiglu(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(x[:, 0::2]) * x[:, 1::2] for x [T, 2I] (gate and up interleaved)."""
     _need(x, "swiglu input", ndim=2)

@@ -31,6 +31,7 @@ _SIGNATURES = {
     "fsie_rmsnorm_plain": ([_P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_float, c_int, _P], c_int),
     "fsie_zero_rows": ([_P, _P, c_int, c_int64, c_int, _P], c_int),
     "fsie_zero_pages": ([_P, _P, _P, c_int, c_int, c_int, c_int64, _P], c_int),
+    "fsie_random_fill": ([_P, c_int64, ctypes.c_uint64, c_int, c_float, _P], c_int),
     "fsie_swiglu": ([_P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_residual_add": ([_P, _P, c_int64, c_int, _P], c_int),
     "fsie_bias_add": ([_P, _P, c_int, c_int, c_int, _P], c_int),

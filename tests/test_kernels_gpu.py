@@ -732,3 +732,19 @@ def test_sampling_distribution(ops):
     out = ops.sample(logits, ones, torch.zeros(n, dtype=torch.int32).cuda(), ones, u).cpu()
     assert abs((out == 1).float().mean().item() - 0.7869) < 0.002
     assert (out[:400] == 0).all() and (out[-400:] == 2).all()  # vocabulary order of the draw
+
+
+def test_random_weights_are_the_same_bits_on_the_device_and_on_the_host(ops):
+    """The random-weights mode: the kernel and the host code of the counter-based generator agree
+    bit for bit (weights, norm weights, integer tables; float32 and rounded to bfloat16), so a
+    model made on the device is the model that the written folder holds."""
+    from from_scratch_inference_engine_amd.weights import random_init as r
+    from from_scratch_inference_engine_amd.weights.loader import TensorSpec
+
+    for name, shape, init in [("model.embed_tokens.weight", (509, 192), "weight"), ("model.norm.weight", (3584,), "norm"),
+                              ("a.bias", (7,), "bias"), ("ids", (33, 5), "int"), ("big", (1 << 21,), "weight")]:
+        spec = TensorSpec(name, shape, init)
+        for dtype in (torch.float32, torch.bfloat16):
+            host = r.random_tensor(spec, 41, dtype, "cpu")
+            dev = r.random_tensor(spec, 41, dtype, "cuda:0")
+            assert dev.is_cuda and dev.dtype == host.dtype and torch.equal(dev.cpu(), host), (name, dtype)

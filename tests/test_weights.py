@@ -4,6 +4,7 @@ import json
 import struct
 
 import pytest
+import numpy as np
 import torch
 
 import helpers
@@ -207,3 +208,33 @@ def test_random_model_folder(tmp_path):
     assert parse_config(json.loads((a / "config.json").read_text())) == cfg
     # the written folder loads without complaint
     load_weights(a / "model.safetensors", _spec(helpers.TINY_B).bindings, torch.bfloat16, "cpu")
+
+
+def test_random_values_are_a_function_of_seed_name_and_index():
+    """The counter-based generator on the host: an element does not depend on how many elements
+    are made with it or on other tensors; the values are close to normal with the stated
+    deviation; integer tables are 15-bit ids."""
+    from from_scratch_inference_engine_amd.weights import random_init as r
+    from from_scratch_inference_engine_amd.weights.loader import TensorSpec
+
+    key = r.stream_key(7, "model.layers.3.mlp.up_proj.weight")
+    whole = r.host_values(key, (1 << 20) + 77, "weight")       # more than one chunk of the host loop
+    assert np.array_equal(r.host_values(key, 1000, "weight"), whole[:1000])
+    assert np.array_equal(r.host_values(key, 50, "norm"), whole[:50] + np.float32(1.0))
+    assert not np.array_equal(r.host_values(r.stream_key(8, "model.layers.3.mlp.up_proj.weight"), 1000, "weight"), whole[:1000])
+    assert not np.array_equal(r.host_values(r.stream_key(7, "model.layers.3.mlp.gate_proj.weight"), 1000, "weight"), whole[:1000])
+    z = whole.astype(np.float64) / 0.02
+    assert abs(z.mean()) < 5e-3 and abs(z.std() - 1.0) < 5e-3 and abs((z ** 4).mean() - 3.0) < 0.2 and np.abs(z).max() < 4.9
+    assert abs((np.abs(z) < 1.0).mean() - 0.68) < 0.01  # (the sum of eight uniform fields: 0.677 where a normal has 0.683)
+    ids = r.host_values(key, 4096, "int")
+    assert ids.dtype == np.int32 and ids.min() >= 0 and ids.max() < 1 << 15 and len(set(ids.tolist())) > 3500
+    # element 0 written out by hand
+    def output(number):
+        x = (key + (number + 1) * 0x9E3779B97F4A7C15) & ((1 << 64) - 1)
+        x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & ((1 << 64) - 1)
+        x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & ((1 << 64) - 1)
+        return x ^ (x >> 31)
+    total = sum((w >> s) & 0xFFFF for w in (output(0), output(1)) for s in (0, 16, 32, 48))
+    assert whole[0] == np.float32(total - 262140) * np.float32(1.8688124e-05) * np.float32(0.02)
+    t = r.random_tensor(TensorSpec("model.layers.3.mlp.up_proj.weight", (10, 100)), 7, torch.bfloat16)
+    assert t.dtype == torch.bfloat16 and torch.equal(t, torch.from_numpy(whole[:1000]).reshape(10, 100).to(torch.bfloat16))
