@@ -26,8 +26,8 @@ class AttentionPlanner:
     keys (decoding against a long context) is split over the keys into several items and merged
     afterwards in the order of the splits: 256 keys an item for the float32-arithmetic kernel; for
     the matrix-core kernel, which gives every 128 keys to a wave of the item's workgroup and
-    combines those inside, 1,024 keys, or 512 or 256 while the step has fewer workgroups than the
-    device has compute units (every wave still sums the same 128 keys; only where their sums
+    combines those inside, 1,024 keys, or 512, 256 or 128 while the step has fewer workgroups than
+    the device has compute units (every wave still sums the same 128 keys; only where their sums
     meet changes).  Longer portions are cut into *large* tiles of ``large_tokens``; how they are
     cut depends on the portion alone, never on what else is in the batch.  The item table lists
     the small items first.
@@ -90,7 +90,8 @@ class AttentionPlanner:
         step with few requests is faster with more, shorter items, although they cost a merge
         (MI355X, 28/4 heads of 128, per layer: 8 requests of 640 keys 10.7 us with 256 keys an
         item against 12.2 with 1,024; one request of 3,550 keys 11.3 against 18.2; 64 requests of
-        640 keys 24.8 against 18.3, which is why a full device keeps the long items)."""
+        640 keys 24.8 against 18.3, which is why a full device keeps the long items; items of 128
+        keys, one wave each, gain another per cent of a decode step of one to eight requests)."""
         small_tokens, _, longest = self.geometry(mfma)
         if not mfma:
             return longest
@@ -100,7 +101,7 @@ class AttentionPlanner:
         rows = ops.attention_mfma_rows(self.head_dim, False)
         per_item = self.n_kv * -(-group // min(group, rows))  # workgroups of one item
         split = longest
-        while split > 256 and sum(-(-k // split) for k in keys) * per_item < units:
+        while split > 128 and sum(-(-k // split) for k in keys) * per_item < units:
             split //= 2
         return split
 

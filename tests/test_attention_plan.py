@@ -122,13 +122,13 @@ def test_plans_cover_every_key_once(dtype, page_size, heads, kv, hd, window):
 def test_decode_items_shorten_while_compute_units_are_idle():
     planner = AttentionPlanner(28, 4, 128, None)
     planner.compute_units = 256
-    for n_requests, keys, split in ((8, 640, 256), (1, 3550, 256), (64, 640, 1024), (8, 16000, 1024), (20, 3000, 512)):
+    for n_requests, keys, split in ((8, 640, 128), (1, 3550, 128), (64, 640, 1024), (8, 16000, 1024), (20, 3000, 512), (12, 1500, 256)):
         host = Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16)
         assert planner.split_keys(host, True) == split
         plan = planner.plan(host)
         check_plan(planner, host, plan)
         assert plan["n_small"] == n_requests * -(-keys // split)
-        assert plan["waves"] == {256: 2, 512: 4, 1024: 8}[split]  # one wave per 128 keys
+        assert plan["waves"] == {128: 1, 256: 2, 512: 4, 1024: 8}[split]  # one wave per 128 keys
         assert plan["n_merges"] == (n_requests if keys > split else 0)
     # the float32-arithmetic kernel keeps its 256 keys an item
     assert planner.split_keys(Host([(5000, 1)], 16, torch.float32), False) == 256

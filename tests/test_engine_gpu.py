@@ -509,7 +509,7 @@ ODD = {
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
 def test_decoding_against_contexts_that_are_split_and_merged(tmp_path, dtype):
     """Requests of 40, 300 and 700 tokens decode together: a device with idle compute units
-    gives the long ones to several work items of 256 keys whose partial results are merged, the
+    gives the long ones to several work items of 128 keys whose partial results are merged, the
     short one needs no merge, and the graph of the step pads both tables.  Eagerly and through
     graphs, against the plain implementation."""
     from from_scratch_inference_engine_amd import load_model
@@ -536,7 +536,7 @@ def test_decoding_against_contexts_that_are_split_and_merged(tmp_path, dtype):
     if dtype == "bfloat16":  # the step that was tested is one that splits
         from types import SimpleNamespace
         host = SimpleNamespace(n_seqs=3, q_lens=[1, 1, 1], past_lens=[len(ids) - 1 for ids in seqs])
-        assert model.planners[0].split_keys(host, True) == 256
+        assert model.planners[0].split_keys(host, True) == 128
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
