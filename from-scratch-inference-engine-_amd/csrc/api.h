@@ -73,6 +73,10 @@ int fsie_rope_table(const int32_t* positions, const double* inv_freq, int n_toke
 int fsie_gemm(const void* x, const void* w, const float* bias, void* y, int M, int N, int K, int dtype,
               int out_f32, int kind, hipStream_t stream);
 
+// True float32 on the matrix cores (v_mfma_f32_16x16x4_f32) for up to 64 rows: the 32-bit path's decoding.
+int fsie_gemm_mfma_fp32(const float* x, const float* w, const float* bias, float* y, int M, int N, int K, int waves,
+                        hipStream_t stream);
+
 int fsie_gemm_mfma_skinny(const void* x, const void* w, const float* bias, void* y, int M, int N, int K,
                           int out_f32, int waves, int blocks, int epilogue, int splits, hipStream_t stream);
 

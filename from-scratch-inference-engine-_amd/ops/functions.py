@@ -247,6 +247,25 @@ def gemm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = N
     return out
 
 
+def gemm_mfma_fp32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, waves: int = 0,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [M, K] . weight [N, K]^T + bias in true float32 on the matrix cores, for up to 64 rows and K a
+    multiple of 4 (the 32-bit path's decoding).  A row's sums do not depend on the other rows."""
+    _need(x, "gemm x", dtype=torch.float32, ndim=2)
+    _need(weight, "gemm weight", dtype=torch.float32, ndim=2)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"gemm: weight inner size {weight.shape[1]} does not match x's {k}")
+    if bias is not None:
+        _need(bias, "gemm bias", dtype=torch.float32, shape=(n,))
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    _need(out, "gemm out", dtype=torch.float32, shape=(m, n))
+    check(load().fsie_gemm_mfma_fp32(x.data_ptr(), weight.data_ptr(), _ptr(bias), out.data_ptr(), m, n, k, waves, _stream()))
+    return out
+
+
 def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      out_dtype: Optional[torch.dtype] = None, waves: int = 0, blocks: int = 0,
                      out: Optional[torch.Tensor] = None, epilogue: str = "plain", splits: int = 1) -> torch.Tensor:

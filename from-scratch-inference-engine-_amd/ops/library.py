@@ -40,6 +40,7 @@ _SIGNATURES = {
     "fsie_rope_kv_write_table": ([_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, _P],
                                  c_int),
     "fsie_gemm": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_gemm_mfma_fp32": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_gemm_mfma_skinny": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_gemm_mfma_skinny_rope": ([_P, _P, _P, _P, c_int, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
                                     c_int64, _P], c_int),

@@ -14,13 +14,16 @@ from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M, GEMM_MFMA_SKINNY_MAX_M, GEM
 class Linear:
     """Holds ``weight`` [N, K] in the compute dtype and an optional float32 ``bias`` [N].
 
-    float32: the engine's own kernels only (true 32-bit products and sums).
+    float32: the engine's own kernels only (true 32-bit products and sums): vector FMA kernels,
+    and for 3 to 64 rows (decoding) the matrix cores' float32 instruction, which rounds nothing.
     bfloat16: up to 16 rows (decoding) the engine's matrix-core kernel that streams the weight
     once; its sibling that shares x through LDS for float32 results of 8 to 64 rows (the logits; beyond 64 rows the library with a float32 result)
     and for the residual projections (``for_residual``: 17 to 64 rows, and any number where K is
     long); everything else the library product
     (hipBLASLt through torch, where the reference's engine calls cuBLAS) with float32
     accumulation, the bias added by a kernel of the engine."""
+
+    float32_on_matrix_cores = True  # up to 64 rows of float32: v_mfma_f32_16x16x4_f32 instead of vector FMAs
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False):
         self.in_features = in_features
@@ -36,6 +39,11 @@ class Linear:
         w = self.weight
         m = x.shape[0]
         if x.dtype == torch.float32:
+            if self.float32_on_matrix_cores and 2 < m <= GEMM_MFMA_SKINNY_MAX_M and self.in_features % 4 == 0:
+                # decoding in the 32-bit path: W streams once into true float32 matrix instructions
+                # (4 layers of 3584 / 18944 and the head on MI355X, ms a step against the vector
+                # kernels: 8 rows 1.9 / 2.8, 32 rows 3.1 / 23, 64 rows 5.0 / 25; one row 1.6 / 1.5)
+                return ops.gemm_mfma_fp32(x, w, bias)
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
         wants_f32 = out_dtype is not None and out_dtype != x.dtype
         if (wants_f32 and bias is None and 8 <= m <= GEMM_MFMA_SKINNY_MAX_M

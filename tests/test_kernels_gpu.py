@@ -748,3 +748,27 @@ def test_random_weights_are_the_same_bits_on_the_device_and_on_the_host(ops):
             host = r.random_tensor(spec, 41, dtype, "cpu")
             dev = r.random_tensor(spec, 41, dtype, "cuda:0")
             assert dev.is_cuda and dev.dtype == host.dtype and torch.equal(dev.cpu(), host), (name, dtype)
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 4864, 896), (5, 151, 100), (8, 1000, 4864), (17, 3584, 18944), (37, 300, 132),
+                                     (64, 896, 1000), (64, 37888, 3584), (3, 16, 4)])
+def test_gemm_mfma_fp32(ops, m, n, k):
+    """True float32 on the matrix cores: against the float64 product of the same float32 values
+    (no reduced-precision mode would pass 2e-6), with and without bias; a row's sums do not depend
+    on the other rows; whatever the number of waves that split K."""
+    x, w, b = rnd((m, k), 70), rnd((n, k), 71, scale=0.05), rnd((n,), 72)
+    ref = (x.cuda().double() @ w.cuda().double().t()).cpu()
+    out = ops.gemm_mfma_fp32(x.cuda(), w.cuda(), b.cuda()).cpu()
+    assert (out.double() - (ref + b.double())).abs().max() <= 2e-6 * max(1.0, ref.abs().max().item())
+    plain_out = ops.gemm_mfma_fp32(x.cuda(), w.cuda()).cpu()
+    assert (plain_out.double() - ref).abs().max() <= 2e-6 * max(1.0, ref.abs().max().item())
+    if m > 2:
+        fewer = ops.gemm_mfma_fp32(x[1:m - 1].contiguous().cuda(), w.cuda()).cpu()
+        assert torch.equal(fewer, plain_out[1:m - 1])
+    for waves in (1, 2, 8):
+        other = ops.gemm_mfma_fp32(x.cuda(), w.cuda(), waves=waves).cpu()
+        assert (other.double() - ref).abs().max() <= 2e-6 * max(1.0, ref.abs().max().item())
+    with pytest.raises(ops.KernelError, match="multiple of 4"):
+        ops.gemm_mfma_fp32(torch.zeros(2, 6).cuda(), torch.zeros(3, 6).cuda())
+    with pytest.raises(ops.KernelError, match="at most 64 rows"):
+        ops.gemm_mfma_fp32(torch.zeros(65, 8).cuda(), torch.zeros(3, 8).cuda())
