@@ -131,12 +131,14 @@ def kernel_classes(runner, cfg, batch: int, prompt_len: int, itemsize: int) -> d
     read["lm_head"] = h * v * itemsize
     read["attention"] = batch * (prompt_len + 1) * 2 * cfg.num_key_value_heads * cfg.head_dim * itemsize * n_layers
     out = {}
-    side = torch.cuda.Stream()
+    # The recorded step and the prompts before it are only queued so far.  Every call below reads that
+    # step's tables and intermediate tensors, so they must be complete first; and the calls run on the
+    # stream that filled them, never on another one that would not wait for it.
+    torch.cuda.synchronize()
     for cls in sorted({c[0] for c in calls}):
         mine = [(fn, a, k) for c, fn, a, k in calls if c == cls]
-        with torch.cuda.stream(side):
-            for fn, a, k in mine:
-                fn(*a, **k)
+        for fn, a, k in mine:  # once outside a capture: first launches, the allocator's blocks
+            fn(*a, **k)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

@@ -176,14 +176,16 @@ class StepContext:
 
 def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners: Sequence, staging: PinnedStaging,
                   compute_dtype: torch.dtype, device, pad: Optional[dict] = None,
-                  into: Optional[torch.Tensor] = None):
+                  into: Optional[torch.Tensor] = None, host: Optional[HostBatch] = None):
     """Tables of one step.  The entries' pages must have been reserved already.
 
     ``pad`` fixes the sizes of everything whose size depends on the requests' lengths (for a
     step that a captured graph replays): ``pad["pages"]`` = width of the block tables,
-    ``pad[planner.key]`` = what that planner's ``graph_bucket`` returned.  Returns the context
-    and the device buffer that holds all tables."""
-    host = HostBatch(entries, manager.page_size, compute_dtype)
+    ``pad[planner.key]`` = what that planner's ``graph_bucket`` returned.  ``host``: the host view
+    of these very entries, if the caller has made it already.  Returns the context and the
+    device buffer that holds all tables."""
+    if host is None:
+        host = HostBatch(entries, manager.page_size, compute_dtype)
     host.pad = pad
     ctx = StepContext(host, compute_dtype, device)
     pk = _Packer()

@@ -59,6 +59,7 @@ class DecodeGraphs:
         self.enabled = all(p.graph_safe for p in parts) and all(hasattr(p, "graph_bucket") for p in model.planners)
         self.replays = 0
         self.captures = 0
+        self._host = None  # the host view that shape_of made, for the step that follows
 
     @property
     def runner(self):
@@ -88,6 +89,7 @@ class DecodeGraphs:
             if bucket is None:
                 return None
             pad[planner.key] = bucket
+        self._host = host  # of the filled-up entries: the step that follows takes it instead of making it again
         return pad
 
     def step(self, entries: Sequence[StepEntry], pad: dict,
@@ -99,6 +101,9 @@ class DecodeGraphs:
         runner = self.runner
         n = len(entries)
         entries = self.filled_up(entries)
+        host, self._host = self._host, None
+        if host is not None and host.n_seqs != len(entries):
+            host = None
         key = (len(entries),) + tuple(sorted((str(k), v) for k, v in pad.items()))
         hit = self._graphs.get(key)
         if hit is None:
@@ -122,7 +127,7 @@ class DecodeGraphs:
             torch.cuda.synchronize()
             del warm_ctx
             ctx, tables = build_context(entries, runner.manager, runner.model.planners, runner._staging,
-                                        runner.model.dtype, runner.model.device, pad=pad)
+                                        runner.model.dtype, runner.model.device, pad=pad, host=host)
             if feed is not None:
                 ctx.token_ids[:n].copy_(feed)
             graph = torch.cuda.CUDAGraph()
@@ -144,7 +149,7 @@ class DecodeGraphs:
             return logits[:n]
         graph, tables, logits, token_ids = hit
         build_context(entries, runner.manager, runner.model.planners, runner._staging, runner.model.dtype,
-                      runner.model.device, pad=pad, into=tables)
+                      runner.model.device, pad=pad, into=tables, host=host)
         if feed is not None:
             token_ids[:n].copy_(feed)
         graph.replay()

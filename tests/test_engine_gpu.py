@@ -737,3 +737,48 @@ def test_what_an_earlier_request_left_in_its_pages_does_not_reach_the_next(model
                 fed[i] += n
         assert fed == [len(s_) for s_ in seqs]
         assert not torch.isnan(k[:, 0]).any() and (k[:, 0] == 0).all() and (v[:, 0] == 0).all()  # the null page stays empty
+
+
+def test_steps_filled_up_to_the_timed_row_counts_of_256_and_more(tmp_path):
+    """With the library's kernels chosen by timing, a step of 448 tokens (two requests' portions) is
+    filled up to 512 rows with the tokens of a request that does not exist, and a step of 300
+    stays as it is (512 would add more than a fifth); the real requests' logits are the plain
+    model's either way, and so is what they decode next."""
+    from from_scratch_inference_engine_amd import load_model, ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry, padded_tokens
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    assert padded_tokens(448) == 512 and padded_tokens(300) == 300 and padded_tokens(1000) == 1024
+    cfg = dict(helpers.TINY_B, max_position_embeddings=1024)
+    d = helpers.make_model_dir(tmp_path / "m", cfg, seed=41)
+    seqs = [helpers.token_ids(509, n, 1400 + n) for n in (301, 149, 302)]
+    refs = [plain.forward_dir(d, ids).numpy() for ids in seqs]
+    rows_seen = []
+    real_mm = ops.library_mm
+    ops.enable_library_tuning(max_ms_per_candidate=5, iterations=2)
+    try:
+        runner = Runner(load_model(d, dtype="bfloat16"), page_size=16, num_pages=80, max_requests=4)
+        import from_scratch_inference_engine_amd.parts.linear as linear_module
+        saved = linear_module.library_mm
+        linear_module.library_mm = lambda x, w, **k: (rows_seen.append(x.shape[0]), saved(x, w, **k))[1]
+        try:
+            caches = [runner.manager.open(i) for i in range(3)]
+            # 300 + 148 = 448 tokens: filled up to 512
+            out = runner.step([StepEntry(caches[0], seqs[0][:300], [299]), StepEntry(caches[1], seqs[1][:148], [0, 147])]).float().cpu().numpy()
+            helpers.assert_close_to_plain(out[:1], refs[0][299:300], "bfloat16", "filled-up step, request 0")
+            helpers.assert_close_to_plain(out[1:], refs[1][[0, 147]], "bfloat16", "filled-up step, request 1")
+            assert set(rows_seen) == {512}, set(rows_seen)
+            rows_seen.clear()
+            # 300 tokens alone: as they are
+            out = runner.step([StepEntry(caches[2], seqs[2][:300], [299])]).float().cpu().numpy()
+            helpers.assert_close_to_plain(out, refs[2][299:300], "bfloat16", "a step of 300 rows")
+            assert set(rows_seen) == {300}, set(rows_seen)
+            # the next tokens of all three, decoded together
+            out = runner.step([StepEntry(c, [s_[len(s_) - 1 - (len(s_) == 302)]], [0]) for c, s_ in zip(caches, seqs)]).float().cpu().numpy()
+            for i, (s_, at) in enumerate(zip(seqs, (300, 148, 300))):
+                helpers.assert_close_to_plain(out[i:i + 1], refs[i][at:at + 1], "bfloat16", f"decoding after it, request {i}")
+        finally:
+            linear_module.library_mm = saved
+    finally:
+        ops.disable_library_tuning()
+    assert ops.library_mm is real_mm
