@@ -95,7 +95,8 @@ def kernel_classes(runner, cfg, batch: int, prompt_len: int, itemsize: int) -> d
         "attention_mfma": lambda a, k: "attention", "attention_mfma_lds": lambda a, k: "attention",
         "attention_scalar": lambda a, k: "attention", "attention_merge": lambda a, k: "attention",
         "gemm_mfma_skinny": lambda a, k: matrix_class(a[1]), "gemm_mfma_wide": lambda a, k: matrix_class(a[1]),
-        "gemm": lambda a, k: matrix_class(a[1]), "library_mm": lambda a, k: matrix_class(a[1]),
+        "gemm": lambda a, k: matrix_class(a[1]), "gemm_mfma_fp32": lambda a, k: matrix_class(a[1]),
+        "library_mm": lambda a, k: matrix_class(a[1]),
         "swiglu": lambda a, k: "gate_up", "rmsnorm": lambda a, k: "norms", "embedding": lambda a, k: "other",
         "rope_table": lambda a, k: "other", "residual_add": lambda a, k: "other",
     }
@@ -126,7 +127,8 @@ def kernel_classes(runner, cfg, batch: int, prompt_len: int, itemsize: int) -> d
         runner.graphs = graphs
     weights = {"qkv": h * (q + 2 * cfg.num_key_value_heads * cfg.head_dim), "o": q * h, "gate_up": 2 * h * inter,
                "down": h * inter}
-    n_layers = sum(1 for c in calls if c[0] == "qkv" and c[1].__name__ in ("gemm_mfma_skinny_rope", "library_mm", "gemm"))
+    n_layers = sum(1 for c in calls if c[0] == "qkv" and c[1].__name__ in ("gemm_mfma_skinny_rope", "library_mm", "gemm",
+                                                                         "gemm_mfma_fp32"))
     read = {k: n * itemsize * n_layers for k, n in weights.items()}
     read["lm_head"] = h * v * itemsize
     read["attention"] = batch * (prompt_len + 1) * 2 * cfg.num_key_value_heads * cfg.head_dim * itemsize * n_layers
