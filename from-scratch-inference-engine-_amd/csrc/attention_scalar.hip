@@ -32,7 +32,21 @@ __device__ __forceinline__ float half_wave_sum(float v) {
     return v;
 }
 
-template <typename T>
+// Four consecutive elements as floats: one 16-byte (float32) or 8-byte (bfloat16) load.
+__device__ __forceinline__ void load4(const float* p, float (&f)[4]) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    f[0] = v.x, f[1] = v.y, f[2] = v.z, f[3] = v.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float (&f)[4]) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    f[0] = __uint_as_float(v.x << 16), f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16), f[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+
+// VEC: the head size and the page size are multiples of 4 and the pools are aligned for load4, so a
+// thread copies four values of a key (along the head) or of a dimension (four consecutive slots of a
+// page; only for items whose first key is a multiple of 4, else element by element) with one load.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void attention_scalar_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_pages, const int32_t* __restrict__ items,
@@ -89,19 +103,36 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
     const int n_chunks = (hd + 31) / 32;
     const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
 
+    const bool slots_by_four = VEC && (key_begin & 3) == 0;
     for (int kt = key_begin; kt < key_end; kt += kKeys) {
         __syncthreads();  // previous tile's values are no longer read (first pass: qs is written)
-        for (int e = tid; e < kKeys * hd; e += blockDim.x) {
-            const int j = e / hd, d = e - j * hd;
-            const int kj = kt + j;
-            float v = 0.f;
-            if (kj < key_end) {
-                const int page = table[kj / page_size];
-                if (page >= 0) {
-                    v = to_float(k_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + kj % page_size) * hd + d]);
+        if (VEC) {
+            const int per_key = hd >> 2;
+            for (int e = tid; e < kKeys * per_key; e += blockDim.x) {
+                const int j = e / per_key, d = (e - j * per_key) * 4;
+                const int kj = kt + j;
+                float f[4] = {0.f, 0.f, 0.f, 0.f};
+                if (kj < key_end) {
+                    const int page = table[kj / page_size];
+                    if (page >= 0)
+                        load4(k_pool + ((static_cast<int64_t>(page) * n_kv + kvh) * page_size + kj % page_size) * hd + d, f);
                 }
+                float* dst = kv + j * kv_stride + d;
+                dst[0] = f[0], dst[1] = f[1], dst[2] = f[2], dst[3] = f[3];
             }
-            kv[j * kv_stride + d] = v;
+        } else {
+            for (int e = tid; e < kKeys * hd; e += blockDim.x) {
+                const int j = e / hd, d = e - j * hd;
+                const int kj = kt + j;
+                float v = 0.f;
+                if (kj < key_end) {
+                    const int page = table[kj / page_size];
+                    if (page >= 0) {
+                        v = to_float(k_pool[((static_cast<int64_t>(page) * n_kv + kvh) * page_size + kj % page_size) * hd + d]);
+                    }
+                }
+                kv[j * kv_stride + d] = v;
+            }
         }
         __syncthreads();
         float corr[2];
@@ -129,17 +160,34 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
             ps[r * kKeys + lane32] = pe;
         }
         __syncthreads();  // scores done: the tile buffer can take the values
-        for (int e = tid; e < kKeys * hd; e += blockDim.x) {
-            const int j = e / hd, d = e - j * hd;
-            const int kj = kt + j;
-            float v = 0.f;
-            if (kj < key_end) {
-                const int page = table[kj / page_size];
-                if (page >= 0) {
-                    v = to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + kj % page_size]);
+        if (slots_by_four) {
+            // a page of values is [head_dim][page_size]: consecutive threads take the eight groups of
+            // four keys of a dimension, then the next dimension
+            for (int e = tid; e < (kKeys / 4) * hd; e += blockDim.x) {
+                const int g = e & (kKeys / 4 - 1), d = e / (kKeys / 4);
+                const int kj = kt + 4 * g;  // a multiple of 4: the four slots lie in one page
+                float f[4] = {0.f, 0.f, 0.f, 0.f};
+                if (kj < key_end) {
+                    const int page = table[kj / page_size];
+                    if (page >= 0)
+                        load4(v_pool + ((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + kj % page_size, f);
                 }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) kv[(4 * g + t) * kv_stride + d] = kj + t < key_end ? f[t] : 0.f;
             }
-            kv[j * kv_stride + d] = v;
+        } else {
+            for (int e = tid; e < kKeys * hd; e += blockDim.x) {
+                const int j = e / hd, d = e - j * hd;
+                const int kj = kt + j;
+                float v = 0.f;
+                if (kj < key_end) {
+                    const int page = table[kj / page_size];
+                    if (page >= 0) {
+                        v = to_float(v_pool[((static_cast<int64_t>(page) * n_kv + kvh) * hd + d) * page_size + kj % page_size]);
+                    }
+                }
+                kv[j * kv_stride + d] = v;
+            }
         }
         __syncthreads();
 #pragma unroll
@@ -285,13 +333,17 @@ extern "C" int fsie_attention_scalar(const void* q, int64_t q_stride, const void
     const int head_chunks = (group + gh - 1) / gh;
     const dim3 grid(n_items, n_kv * head_chunks);
     const size_t lds = sizeof(float) * (static_cast<size_t>(kRows) * head_dim + kKeys * (head_dim + 1) + kRows * kKeys);
+    const bool vec = head_dim % 4 == 0 && page_size % 4 == 0 && reinterpret_cast<uintptr_t>(k_pool) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(v_pool) % 16 == 0;
     if (dtype == FSIE_F32) {
-        attention_scalar_kernel<float><<<grid, 256, lds, stream>>>(
+        auto kernel = vec ? attention_scalar_kernel<float, true> : attention_scalar_kernel<float, false>;
+        kernel<<<grid, 256, lds, stream>>>(
             static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pool), static_cast<const float*>(v_pool),
             block_tables, max_pages, items, static_cast<float*>(out), partials, n_heads, n_kv, head_dim, page_size,
             window, scale, gh, head_chunks);
     } else {
-        attention_scalar_kernel<bf16_t><<<grid, 256, lds, stream>>>(
+        auto kernel = vec ? attention_scalar_kernel<bf16_t, true> : attention_scalar_kernel<bf16_t, false>;
+        kernel<<<grid, 256, lds, stream>>>(
             static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool),
             static_cast<const bf16_t*>(v_pool), block_tables, max_pages, items, static_cast<bf16_t*>(out), partials,
             n_heads, n_kv, head_dim, page_size, window, scale, gh, head_chunks);

@@ -24,7 +24,8 @@ class AttentionPlanner:
     the keys from the start of its window to its last token.  A portion of at most
     ``small_tokens`` tokens is one *small* item.  A small item that reads more than ``split_keys``
     keys (decoding against a long context) is split over the keys into several items and merged
-    afterwards in the order of the splits: 256 keys an item for the float32-arithmetic kernel; for
+    afterwards in the order of the splits: 256 keys an item for the float32-arithmetic kernel (128
+    or 64 while the step has fewer workgroups than the device has compute units); for
     the matrix-core kernel, which gives every 128 keys to a wave of the item's workgroup and
     combines those inside, 1,024 keys, or 512, 256 or 128 while the step has fewer workgroups than
     the device has compute units (every wave still sums the same 128 keys; only where their sums
@@ -93,15 +94,15 @@ class AttentionPlanner:
         640 keys 24.8 against 18.3, which is why a full device keeps the long items; items of 128
         keys, one wave each, gain another per cent of a decode step of one to eight requests)."""
         small_tokens, _, longest = self.geometry(mfma)
-        if not mfma:
-            return longest
         units = self.compute_units if self.compute_units is not None else ops.compute_units()
         keys = self._small_keys(host, small_tokens)
         group = self.n_heads // self.n_kv
-        rows = ops.attention_mfma_rows(self.head_dim, False)
+        # the float32-arithmetic kernel takes 32 keys a pass and up to 16 heads of a group a workgroup:
+        # its items shorten to 64 keys (two passes) while compute units are idle
+        rows, shortest = (ops.attention_mfma_rows(self.head_dim, False), 128) if mfma else (16, 64)
         per_item = self.n_kv * -(-group // min(group, rows))  # workgroups of one item
         split = longest
-        while split > 128 and sum(-(-k // split) for k in keys) * per_item < units:
+        while split > shortest and sum(-(-k // split) for k in keys) * per_item < units:
             split //= 2
         return split
 
@@ -127,7 +128,7 @@ class AttentionPlanner:
             step = host.n_seqs * max(1, 1024 // split_keys)
             return (-(-n // step) * step,
                     self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)), split_keys)
-        step = 4 * host.n_seqs
+        step = host.n_seqs * max(1, 1024 // split_keys)
         return (-(-n // step) * step, 1, split_keys)
 
     def plan(self, host) -> Dict[str, object]:

@@ -130,8 +130,13 @@ def test_decode_items_shorten_while_compute_units_are_idle():
         assert plan["n_small"] == n_requests * -(-keys // split)
         assert plan["waves"] == {128: 1, 256: 2, 512: 4, 1024: 8}[split]  # one wave per 128 keys
         assert plan["n_merges"] == (n_requests if keys > split else 0)
-    # the float32-arithmetic kernel keeps its 256 keys an item
-    assert planner.split_keys(Host([(5000, 1)], 16, torch.float32), False) == 256
+    # the float32-arithmetic kernel: 256 keys an item on a full device, down to 64 (two passes of 32) on an idle one
+    for n_requests, keys, split in ((1, 5000, 64), (8, 640, 64), (64, 640, 256), (4, 2000, 128)):
+        host = Host([(keys - 1, 1)] * n_requests, 16, torch.float32)
+        assert planner.split_keys(host, False) == split
+        plan = planner.plan(host)
+        check_plan(planner, host, plan)
+        assert plan["n_small"] == n_requests * -(-keys // split) and plan["waves"] == 1
 
 
 def test_graph_bucket_pads_plans_of_decode_steps():
