@@ -21,6 +21,15 @@
 #include "common.h"
 #include "api.h"
 
+// 32-wide steps of K per stage (a stage is what the pipeline keeps in flight per wave and lays into
+// LDS).  Measured on MI355X with 2, 4 and 8 (8 holds at most 32 rows in the 64 KB of static LDS): the
+// gate/up shape (N = 37888, K = 3584) does not care (32 rows: 57 to 62 us for the best launch shape of
+// each), so it is not the memory latency that bounds it there; the down shape (N = 3584, K = 18944 in
+// 8 slices, 8 rows) takes 29.6 / 25.6 / 29.0 us.
+#ifndef FSIE_WIDE_STEPS
+#define FSIE_WIDE_STEPS 4
+#endif
+
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -174,8 +183,12 @@ int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, 
     switch (mt) {
         case 1: return launch<1, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
         case 2: return launch<2, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
+#if FSIE_WIDE_STEPS <= 4
         case 3: return launch<3, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
         default: return launch<4, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
+#else
+        default: fsie_set_error("gemm_mfma_wide: stages of %d steps hold at most 32 rows", STEPS); return 1;
+#endif
     }
 }
 
@@ -184,7 +197,7 @@ int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, 
 // The length of a slice of K for `splits` slices, or 0 if K cannot be cut that way: K and every
 // slice must be a multiple of the stage (128 values), and no slice may be empty.
 extern "C" int fsie_gemm_mfma_wide_slice(int K, int splits) {
-    constexpr int kStage = 128;
+    constexpr int kStage = 32 * FSIE_WIDE_STEPS;
     if (K <= 0 || splits < 1 || splits > FSIE_GEMM_MAX_SPLITS || K % kStage) return 0;
     const int slice = ((K + splits - 1) / splits + kStage - 1) / kStage * kStage;
     if (static_cast<int64_t>(slice) * (splits - 1) >= K) return 0;
@@ -233,11 +246,11 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
     if (blocks == 2) {
-        if (waves == 8) return launch_mt<8, 4, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-        if (waves == 2) return launch_mt<2, 4, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-        return launch_mt<4, 4, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+        if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+        if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+        return launch_mt<4, FSIE_WIDE_STEPS, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
     }
-    if (waves == 8) return launch_mt<8, 4, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-    if (waves == 2) return launch_mt<2, 4, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-    return launch_mt<4, 4, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    return launch_mt<4, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
 }
