@@ -27,6 +27,10 @@
 // 77 us (V) against 70 us with 8; 16, 24 or 40 change nothing (178 to 184 us at 4,096 tokens for all
 // of them): with 8 the layout is free of the conflicts that cost time, and what the counter of
 // bank conflicts still shows does not bound the kernel.
+// 1: the second batch of a die's workgroups takes its groups in ascending length (see the kernel)
+#ifndef FSIE_LDS_PAIR
+#define FSIE_LDS_PAIR 1
+#endif
 #ifndef FSIE_LDS_KPAD
 #define FSIE_LDS_KPAD 8
 #endif
@@ -62,7 +66,8 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, const int32_t* __restrict__ groups, bf16_t* __restrict__ out, int n_heads,
-    int n_kv, int page_size_arg, int window, float scale, int gh, int head_chunks, int n_groups, int n_y) {
+    int n_kv, int page_size_arg, int window, float scale, int gh, int head_chunks, int n_groups, int n_y,
+    int units_per_die) {
     constexpr int HD = HDT * 16;
     const int page_size = PS > 0 ? PS : page_size_arg;
     constexpr int S32 = HDT / 2;       // 32-wide steps over the head dimension
@@ -84,7 +89,22 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     if (n_y > 0) {
         const int die = blockIdx.x & 7;
         by = die % n_y;
-        g_lin = (blockIdx.x >> 3) * (8 / n_y) + die / n_y;
+        const int per = 8 / n_y, sub = die / n_y;
+        int i = blockIdx.x >> 3;  // the i-th workgroup of this die
+#if FSIE_LDS_PAIR
+        // A die's first `units_per_die` workgroups get a compute unit each, the next as many join
+        // them there in the same order (two fit a unit), and only what follows waits for a free
+        // place.  The first batch takes the longest groups in descending order; the second batch is
+        // turned round, so that the unit with the longest group of the first gets the shortest of the
+        // second: with 2,048 tokens (56 workgroups a die) the fullest unit then has 32 blocks of
+        // keys to go through, not 46.
+        if (i >= units_per_die && i < 2 * units_per_die) {
+            const int n_local = (n_groups - sub + per - 1) / per;
+            const int hi = min(2 * units_per_die, n_local);
+            if (i < hi) i = units_per_die + (hi - 1 - i);
+        }
+#endif
+        g_lin = i * per + sub;
         if (g_lin >= n_groups) return;
     }
     const int g_idx = n_groups - 1 - g_lin;
@@ -403,7 +423,7 @@ int launch_lds(const bf16_t* q, int64_t q_stride, const bf16_t* k_pool, const bf
     attention_mfma_lds_kernel<HDT, PS><<<grid, kLdsThreads, 0, stream>>>(q, q_stride, k_pool, v_pool, block_tables, max_pages,
                                                                      items, groups, out, n_heads, n_kv, page_size,
                                                                      window, scale, gh, head_chunks, n_groups,
-                                                                     by_die ? ys : 0);
+                                                                     by_die ? ys : 0, max(1, fsie_compute_units() / 8));
     FSIE_CHECK_LAUNCH("attention_mfma_lds");
     return 0;
 }

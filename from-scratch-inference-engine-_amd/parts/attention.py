@@ -183,6 +183,10 @@ class AttentionPlanner:
                     groups[-1][1] += 1
                 else:
                     groups.append([i, 1])
+            # by the number of keys a group goes through, ascending: the kernel starts its workgroups
+            # from the back of this list, the longest first (with several requests in a step the
+            # order of the requests would otherwise decide)
+            groups.sort(key=lambda g: large[g[0] + g[1] - 1][5] - large[g[0]][4])
         n_long = 0
         if mfma and self.long_keys is not None:
             # large tiles that read more than ``long_keys`` keys go to workgroups of four waves

@@ -83,7 +83,9 @@ def check_plan(planner, host, plan):
             assert len({int(t[SEQ]) for t in tiles}) == 1
             assert all(int(a[POS]) + int(a[NQ]) == int(b[POS]) for a, b in zip(tiles, tiles[1:]))
             covered += list(range(first, first + count))
-        assert covered == list(range(len(large)))
+        assert sorted(covered) == list(range(len(large)))  # every tile in exactly one group
+        spans = [int(large[f + n - 1][KE]) - int(large[f][KB]) for f, n in plan["groups"]]
+        assert spans == sorted(spans)  # ascending by keys: the kernel starts from the back, longest first
     else:
         assert plan["n_groups"] == 0
 
