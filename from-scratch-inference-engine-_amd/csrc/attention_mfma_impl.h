@@ -65,7 +65,7 @@ constexpr int max_waves() {
 }
 
 template <int HDT, int NT, int MAXW, bool V16>
-__global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW == 1 ? 2 : 1))) void attention_mfma_kernel(
+__global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW == 1 && NT > 1 ? 2 : 1))) void attention_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, bf16_t* __restrict__ out, float* __restrict__ partials, int n_heads,
@@ -285,7 +285,25 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
     // its data is in flight while the matrix cores work on the present one (few waves run here,
     // so occupancy does not hide the latency).
     constexpr bool PREFETCH = NT == 1 && HDT <= 8;
-    if (kb_begin < kb_end) {
+    // A workgroup of one wave (items of up to 128 keys, what a step with idle compute units is cut
+    // into) has all 512 registers of its SIMD: the table reads of its four blocks go out together,
+    // then all their data reads, and the products follow; one trip to memory for the addresses and
+    // one for the data, where fetching a block ahead costs a trip per block (8.0 -> 7.3 us a layer for
+    // eight requests of 640 keys).
+    constexpr bool ALL_AHEAD = PREFETCH && MAXW == 1;
+    if constexpr (ALL_AHEAD) {
+        for (int kb0 = kb_begin; kb0 < kb_end; kb0 += 4 * 32) {
+            Where at[4];
+            Block blk[4];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) locate(kb0 + 32 * d, at[d]);  // past the end: page 0, masked below
+#pragma unroll
+            for (int d = 0; d < 4; ++d) load_block(at[d], blk[d]);
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                if (kb0 + 32 * d < kb_end) compute_block(kb0 + 32 * d, blk[d]);
+        }
+    } else if (kb_begin < kb_end) {
         Where at;
         locate(kb_begin, at);
         if (PREFETCH) {
