@@ -12,7 +12,7 @@
 #define FSIE_GEMM_SKINNY_MAX_M 8
 #define FSIE_GEMM_MFMA_SKINNY_MAX_M 64
 #define FSIE_GEMM_MFMA_SKINNY_BEST_M 16  // above this the library product is faster on MI355X
-#define FSIE_GEMM_MAX_SPLITS 8           // most slices of K a product may leave as partial sums
+#define FSIE_GEMM_MAX_SPLITS 16          // most slices of K a product may leave as partial sums
 
 // one attention work item = 8 int32
 #define FSIE_ATTN_ITEM_INTS 8
@@ -88,6 +88,7 @@ int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const float* bias, 
 
 // 17 to 64 rows (any number up to 64 is taken): X shared through LDS, float32 result or partial sums
 int fsie_gemm_mfma_wide_slice(int K, int splits);
+int fsie_gemm_mfma_wide_best_splits(int M, int N, int K);
 int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits, int waves,
                         int blocks, hipStream_t stream);
 

@@ -102,19 +102,21 @@ __global__ void embedding_vec_kernel(const T* __restrict__ table, const int32_t*
     Pack4<float>::store(out + static_cast<int64_t>(t) * hidden + j, ok ? v : float4{0.f, 0.f, 0.f, 0.f});
 }
 
-// DELTA: 0 = none, 1 = one array of T, 2 / 4 / 8 = that many float32 partial sums, added in order.
+// DELTA: 0 = none, 1 = one array of T, 2 / 3 / 4 / 6 / 8 / 9 = that many float32 partial sums, added in
+// order (every load of the row goes out before anything waits); -1 = `n_parts` of them (any other
+// number: a loop, four loads ahead).
 template <typename T, int ITERS, int DELTA, bool WRITE_BACK>
 __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta,
                                                                const float* __restrict__ weight, T* __restrict__ out,
                                                                const int32_t* __restrict__ rows, int hidden, float eps,
-                                                               int64_t part_stride) {
+                                                               int64_t part_stride, int n_parts) {
     __shared__ float scratch[16];
     constexpr bool HAS_DELTA = DELTA != 0;
     const int r = blockIdx.x;
     const int64_t row = rows ? rows[r] : r;
     float* res = residual + row * hidden;
     const T* del = DELTA == 1 ? delta + row * hidden : nullptr;
-    const float* parts = DELTA > 1 ? reinterpret_cast<const float*>(delta) + row * hidden : nullptr;
+    const float* parts = (DELTA > 1 || DELTA < 0) ? reinterpret_cast<const float*>(delta) + row * hidden : nullptr;
     // every load of the row goes out before anything waits: places past the end read the last
     // quad again and are masked out of the sum and the stores
     float4 v[ITERS], d[ITERS], w[ITERS];
@@ -135,6 +137,18 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict
                 d[it].z += p[s].z;
                 d[it].w += p[s].w;
             }
+        }
+        if (DELTA < 0) {
+            float4 a = Pack4<float>::load(parts + j);
+#pragma unroll 4
+            for (int s = 1; s < n_parts; ++s) {
+                const float4 p = Pack4<float>::load(parts + s * part_stride + j);
+                a.x += p.x;
+                a.y += p.y;
+                a.z += p.z;
+                a.w += p.w;
+            }
+            d[it] = a;
         }
         w[it] = Pack4<float>::load(weight + j);
     }
@@ -186,10 +200,10 @@ void launch_rmsnorm_delta(const NormCall& c) {
     T* o = static_cast<T*>(c.out);
     if (c.write_back) {
         rmsnorm_vec_kernel<T, ITERS, DELTA, DELTA != 0><<<c.n_rows, kThreads, 0, c.stream>>>(
-            c.residual, d, c.weight, o, c.rows, c.hidden, c.eps, c.part_stride);
+            c.residual, d, c.weight, o, c.rows, c.hidden, c.eps, c.part_stride, c.n_parts);
     } else {
         rmsnorm_vec_kernel<T, ITERS, DELTA, false><<<c.n_rows, kThreads, 0, c.stream>>>(
-            c.residual, d, c.weight, o, c.rows, c.hidden, c.eps, c.part_stride);
+            c.residual, d, c.weight, o, c.rows, c.hidden, c.eps, c.part_stride, c.n_parts);
     }
 }
 
@@ -199,8 +213,12 @@ void launch_rmsnorm_vec(const NormCall& c) {
     switch (c.n_parts) {
         case 0: return launch_rmsnorm_delta<T, ITERS, 1>(c);
         case 2: return launch_rmsnorm_delta<T, ITERS, 2>(c);
+        case 3: return launch_rmsnorm_delta<T, ITERS, 3>(c);
         case 4: return launch_rmsnorm_delta<T, ITERS, 4>(c);
-        default: return launch_rmsnorm_delta<T, ITERS, 8>(c);
+        case 6: return launch_rmsnorm_delta<T, ITERS, 6>(c);
+        case 8: return launch_rmsnorm_delta<T, ITERS, 8>(c);
+        case 9: return launch_rmsnorm_delta<T, ITERS, 9>(c);
+        default: return launch_rmsnorm_delta<T, ITERS, -1>(c);
     }
 }
 
@@ -208,8 +226,7 @@ template <typename T>
 void launch_rmsnorm(const NormCall& c) {
     const bool aligned = c.hidden % 4 == 0 && reinterpret_cast<uintptr_t>(c.residual) % 16 == 0 &&
                          reinterpret_cast<uintptr_t>(c.weight) % 16 == 0 && reinterpret_cast<uintptr_t>(c.delta) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(c.out) % 16 == 0 && c.part_stride % 4 == 0 &&
-                         (c.n_parts == 0 || c.n_parts == 2 || c.n_parts == 4 || c.n_parts == 8);
+                         reinterpret_cast<uintptr_t>(c.out) % 16 == 0 && c.part_stride % 4 == 0;
     // a thread holds `iters` quads of the row: as many as the row needs, so that a row of 5,120
     // values asks for five quads a thread and not for eight of which three repeat the last one
     const int per_iter = kThreads * 4;

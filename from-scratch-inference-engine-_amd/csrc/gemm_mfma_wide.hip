@@ -192,35 +192,8 @@ int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, 
     }
 }
 
-}  // namespace
-
-// The length of a slice of K for `splits` slices, or 0 if K cannot be cut that way: K and every
-// slice must be a multiple of the stage (128 values), and no slice may be empty.
-extern "C" int fsie_gemm_mfma_wide_slice(int K, int splits) {
-    constexpr int kStage = 32 * FSIE_WIDE_STEPS;
-    if (K <= 0 || splits < 1 || splits > FSIE_GEMM_MAX_SPLITS || K % kStage) return 0;
-    const int slice = ((K + splits - 1) / splits + kStage - 1) / kStage * kStage;
-    if (static_cast<int64_t>(slice) * (splits - 1) >= K) return 0;
-    return slice;
-}
-
-// bfloat16 operands, float32 result: y is [M, N] (splits == 1) or [splits, M, N] partial sums.
-// 1 <= M <= 64; K a multiple of 128 that `splits` slices of whole stages cover (see above);
-// x and w 16-byte aligned.  waves: 2, 4 or 8 waves per workgroup; blocks: 1 or 2 blocks of 16 rows
-// of W per wave; 0 = choose.
-extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits,
-                                   int waves, int blocks, hipStream_t stream) {
-    FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide: bad sizes M=%d N=%d K=%d", M, N, K);
-    FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide: at most %d rows, got %d",
-                 FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
-    const int k_slice = fsie_gemm_mfma_wide_slice(K, splits);
-    FSIE_REQUIRE(k_slice > 0, "gemm_mfma_wide: K=%d cannot be cut into %d slices of whole stages of 128", K, splits);
-    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
-                 "gemm_mfma_wide: operands must be 16-byte aligned");
-    FSIE_REQUIRE(waves == 0 || waves == 2 || waves == 4 || waves == 8, "gemm_mfma_wide: waves must be 0, 2, 4 or 8");
-    FSIE_REQUIRE(blocks == 0 || blocks == 1 || blocks == 2, "gemm_mfma_wide: blocks must be 0, 1 or 2");
-    if (M == 0) return 0;
-    const int mt = (M + 15) / 16;
+// Waves a workgroup and row blocks a wave where the caller leaves them open (0).
+void launch_shape(int mt, int N, int splits, int& waves, int& blocks) {
     if (blocks == 0) {
         // three or four tiles of X: two blocks of W a wave share the B fragments read from LDS,
         // where that still leaves a workgroup for most compute units (measured on MI355X, 64 rows,
@@ -243,6 +216,77 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
             if (fullest2 < fullest4) waves = 2;
         }
     }
+}
+
+}  // namespace
+
+// The length of a slice of K for `splits` slices, or 0 if K cannot be cut that way: K and every
+// slice must be a multiple of the stage (128 values), and no slice may be empty.
+extern "C" int fsie_gemm_mfma_wide_slice(int K, int splits) {
+    constexpr int kStage = 32 * FSIE_WIDE_STEPS;
+    if (K <= 0 || splits < 1 || splits > FSIE_GEMM_MAX_SPLITS || K % kStage) return 0;
+    const int slice = ((K + splits - 1) / splits + kStage - 1) / kStage * kStage;
+    if (static_cast<int64_t>(slice) * (splits - 1) >= K) return 0;
+    return slice;
+}
+
+// Into how many slices of K a product of M rows that leaves partial sums is best cut (1: not at
+// all, or this kernel does not take K).  A slice is at least 512 long.
+// Up to 16 rows: 8, 4 or 2, the most that K gives: many short workgroups, several a compute unit.
+// (Alone, N = K = 3584 at 8 rows takes 7.4 us in 7 slices against 8.4 for the few-rows kernel's 4; in
+// a whole decode step the norm that adds 7 parts instead of 4 costs more than that: 3.63 against
+// 3.56 ms a step of 28 layers.)
+// From 17 rows on a workgroup keeps its compute unit busy by itself (the reads of x from LDS and
+// the matrix instructions grow with the rows), and what counts is that all workgroups run at once
+// and leave few units idle: the cut that gives the most workgroups the device has units for
+// (64 rows on 256 units: N = 3584, K = 18944 in 9 slices, 252 workgroups, 32.4 us against 33.2 in 8;
+// N = 5120, K = 13824 in 6 slices, 240 workgroups, 32.4 against 43.5 in 8, 320 workgroups;
+// N = 5120, K = 27648 in 6 slices 60.4 against 75.3; N = K = 5120 in 6 slices 17.4 against 21.6).
+extern "C" int fsie_gemm_mfma_wide_best_splits(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 1;
+    const int mt = (M + 15) / 16;
+    const int units = fsie_compute_units();
+    if (mt <= 1 || units <= 0) {
+        for (int s = 8; s >= 2; s /= 2)
+            if (K / s >= 512 && fsie_gemm_mfma_wide_slice(K, s) > 0) return s;
+        return 1;
+    }
+    int best = 1;
+    int64_t best_groups = 0;
+    bool best_fits = false;
+    for (int s = 2; s <= FSIE_GEMM_MAX_SPLITS; ++s) {
+        if (K / s < 512 || fsie_gemm_mfma_wide_slice(K, s) <= 0) continue;
+        int waves = 0, blocks = 0;
+        launch_shape(mt, N, s, waves, blocks);
+        const int rows = 16 * blocks * waves;
+        const int64_t groups = static_cast<int64_t>((N + rows - 1) / rows) * s;
+        const bool fits = groups <= units;
+        // among the cuts that fit, the most workgroups (of equals, the more slices: shorter ones);
+        // if none fits, the fewest workgroups
+        const bool better = best == 1 || (fits && !best_fits) || (fits == best_fits && (fits ? groups >= best_groups : groups < best_groups));
+        if (better) best = s, best_groups = groups, best_fits = fits;
+    }
+    return best;
+}
+
+// bfloat16 operands, float32 result: y is [M, N] (splits == 1) or [splits, M, N] partial sums.
+// 1 <= M <= 64; K a multiple of 128 that `splits` slices of whole stages cover (see above);
+// x and w 16-byte aligned.  waves: 2, 4 or 8 waves per workgroup; blocks: 1 or 2 blocks of 16 rows
+// of W per wave; 0 = choose.
+extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits,
+                                   int waves, int blocks, hipStream_t stream) {
+    FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide: bad sizes M=%d N=%d K=%d", M, N, K);
+    FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide: at most %d rows, got %d",
+                 FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
+    const int k_slice = fsie_gemm_mfma_wide_slice(K, splits);
+    FSIE_REQUIRE(k_slice > 0, "gemm_mfma_wide: K=%d cannot be cut into %d slices of whole stages of 128", K, splits);
+    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
+                 "gemm_mfma_wide: operands must be 16-byte aligned");
+    FSIE_REQUIRE(waves == 0 || waves == 2 || waves == 4 || waves == 8, "gemm_mfma_wide: waves must be 0, 2, 4 or 8");
+    FSIE_REQUIRE(blocks == 0 || blocks == 1 || blocks == 2, "gemm_mfma_wide: blocks must be 0, 1 or 2");
+    if (M == 0) return 0;
+    const int mt = (M + 15) / 16;
+    launch_shape(mt, N, splits, waves, blocks);
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
     if (blocks == 2) {

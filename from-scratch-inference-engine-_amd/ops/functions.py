@@ -14,7 +14,8 @@ ATTN_MERGE_INTS = 4
 GEMM_SKINNY_MAX_M = 8
 GEMM_MFMA_SKINNY_MAX_M = 64
 GEMM_MFMA_SKINNY_BEST_M = 16
-GEMM_SPLITS = (2, 4, 8)  # slices of K that a product may leave as partial sums
+GEMM_SPLITS = (2, 4, 8)  # slices of K that the few-rows product may leave as partial sums
+GEMM_MAX_SPLITS = 16     # most slices of the product that shares x through LDS, and most that a norm adds up
 GEMM_AUTO, GEMM_TILED, GEMM_SKINNY = 0, 1, 2
 
 
@@ -74,8 +75,8 @@ def rmsnorm(residual: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype:
     if delta is not None and delta.ndim == 3:
         n_parts = delta.shape[0]
         _need(delta, "rmsnorm delta parts", dtype=torch.float32, shape=(n_parts, t, h))
-        if n_parts not in GEMM_SPLITS:
-            raise KernelError(f"rmsnorm: {n_parts} partial sums; offered are {GEMM_SPLITS}")
+        if not 2 <= n_parts <= GEMM_MAX_SPLITS:
+            raise KernelError(f"rmsnorm: {n_parts} partial sums; 2 to {GEMM_MAX_SPLITS} are taken")
     elif delta is not None:
         _need(delta, "rmsnorm delta", dtype=out_dtype, shape=(t, h))
     n_rows = t
@@ -310,6 +311,12 @@ def gemm_mfma_wide_splits_ok(k: int, splits: int) -> bool:
     return load().fsie_gemm_mfma_wide_slice(int(k), int(splits)) > 0
 
 
+def gemm_mfma_wide_best_splits(m: int, n: int, k: int) -> int:
+    """Into how many slices of K ``gemm_mfma_wide`` best cuts a product of ``m`` rows that leaves
+    partial sums (1: it does not cut, or does not take this K)."""
+    return int(load().fsie_gemm_mfma_wide_best_splits(int(m), int(n), int(k)))
+
+
 def gemm_mfma_wide(x: torch.Tensor, weight: torch.Tensor, splits: int = 1, waves: int = 0,
                    out: Optional[torch.Tensor] = None, blocks: int = 0) -> torch.Tensor:
     """x [M, K] . weight [N, K]^T for bfloat16 operands and up to 64 rows, the rows of x shared by
@@ -323,8 +330,8 @@ def gemm_mfma_wide(x: torch.Tensor, weight: torch.Tensor, splits: int = 1, waves
     n = weight.shape[0]
     if weight.shape[1] != k:
         raise KernelError(f"gemm: weight inner size {weight.shape[1]} does not match x's {k}")
-    if splits != 1 and splits not in GEMM_SPLITS:
-        raise KernelError(f"gemm_mfma_wide: splits must be 1 or one of {GEMM_SPLITS}, got {splits}")
+    if not 1 <= splits <= GEMM_MAX_SPLITS:
+        raise KernelError(f"gemm_mfma_wide: splits must be 1 to {GEMM_MAX_SPLITS}, got {splits}")
     shape = (m, n) if splits == 1 else (splits, m, n)
     if out is None:
         out = torch.empty(shape, dtype=torch.float32, device=x.device)

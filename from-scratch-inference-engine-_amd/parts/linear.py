@@ -31,7 +31,7 @@ class Linear:
         self.has_bias = bias
         self.weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
-        self._wide_splits: Optional[int] = None
+        self._wide_splits: dict = {}
 
     def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                  skip_bias: bool = False) -> torch.Tensor:
@@ -80,7 +80,7 @@ class Linear:
             # the kernel that shares x through LDS: above 16 rows, and at any number of rows where
             # K is long enough for eight slices (N = 3584, K = 18944: 26 against 28 us at 8 rows,
             # 27 against 32 at 16)
-            splits = self.wide_splits()
+            splits = self.wide_splits(m)
             if splits > 1 and (m > GEMM_MFMA_SKINNY_BEST_M or splits == 8):
                 return ops.gemm_mfma_wide(x, self.weight, splits=splits)
             splits = self.residual_splits(m)
@@ -88,18 +88,17 @@ class Linear:
                 return ops.gemm_mfma_skinny(x, self.weight, splits=splits)
         return self(x)
 
-    def wide_splits(self) -> int:
-        """Slices of K for 17 to 64 rows (the kernel that shares x through LDS): as many as it
-        takes, each at least 512 long (measured on MI355X at 64 rows: N = 3584, K = 18944 in 8
-        slices 38 us, against 68 for the few-rows kernel and 91 for the library; N = K = 3584 in
-        4 slices 11.6 against the library's 13.7).  1 = it does not take this K."""
-        if self._wide_splits is None:
-            self._wide_splits = 1
-            for splits in (8, 4, 2):
-                if self.in_features // splits >= 512 and ops.gemm_mfma_wide_splits_ok(self.in_features, splits):
-                    self._wide_splits = splits
-                    break
-        return self._wide_splits
+    def wide_splits(self, m: int) -> int:
+        """Slices of K for the kernel that shares x through LDS, by the tiles of 16 rows that ``m``
+        rows make (the kernel's own rule: 8, 4 or 2, the most that K gives, for up to 16 rows; from 17
+        rows on the cut that gives the most workgroups the device has compute units for).  1 = it does
+        not take this K.  (64 rows on MI355X: N = 3584, K = 18944 in 9 slices 32 us, against 68 for
+        the few-rows kernel and 91 for the library; N = K = 3584 in 4 slices 10.9 against the
+        library's 13.7.)"""
+        tiles = -(-m // 16)
+        if tiles not in self._wide_splits:
+            self._wide_splits[tiles] = ops.gemm_mfma_wide_best_splits(m, self.out_features, self.in_features)
+        return self._wide_splits[tiles]
 
     def residual_splits(self, m: int) -> int:
         """Slices of K for ``for_residual`` (1 = do not cut): as many as bring the workgroups to

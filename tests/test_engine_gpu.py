@@ -416,7 +416,8 @@ def test_batches_of_17_to_64_rows_share_x_through_lds(tmp_path):
         ops.gemm_mfma_wide = real
     rows = {m for m, _ in calls}
     assert 20 in rows and 40 in rows, rows                      # decode batch and the portion
-    assert {s for _, s in calls} == {1, 2}, calls                # logits whole, projections in two slices
+    used = {s for _, s in calls}
+    assert 1 in used and len(used) > 1 and all(1 <= s <= 16 for s in used), calls  # logits whole, projections in slices
 
 
 def test_prefill_with_the_library_kernel_selection(model_dirs):

@@ -275,19 +275,27 @@ def _exact(x, w):
 @pytest.mark.parametrize("n, k", [(3584, 18944), (5120, 13824), (5120, 27648), (3584, 3584), (152064, 3584)])
 def test_gemm_mfma_wide_at_the_large_models_shapes(ops, n, k):
     """The residual projections and the logits at the layer sizes of the 7B, 14B and 32B shapes,
-    with the slices the engine's Linear picks there (K = 18944: seven slices of 2,432 and one of
-    1,920), at 8, 17 and 64 rows."""
+    with the slices the engine's Linear picks there for 8, 17 and 64 rows (K = 18944 on 256 compute
+    units: eight slices, seven of 2,432 and one of 1,920, at 8 rows; nine at 64), and with 3, 7 and
+    16 slices where K gives them."""
     from from_scratch_inference_engine_amd.parts.linear import Linear
 
-    splits = 1 if n == 152064 else Linear(k, n).wide_splits()
-    assert splits == (1 if n == 152064 else 4 if k == 3584 else 8)
     w = rnd((n, k), 51, torch.bfloat16, 0.05)
+    picked = {}
     for m in (8, 17, 64):
         x = rnd((m, k), 50 + m, torch.bfloat16)
         ref = _exact(x, w)
-        out = ops.gemm_mfma_wide(x.cuda(), w.cuda(), splits=splits).cpu()
-        total = out if splits == 1 else out.double().sum(0).float()
-        assert (total - ref).abs().max() <= 2e-5 * ref.abs().max(), (m, n, k)
+        picked[m] = 1 if n == 152064 else Linear(k, n).wide_splits(m)
+        for splits in {picked[m]} | ({3, 7, 16} if n != 152064 and m == 17 else set()):
+            if not ops.gemm_mfma_wide_splits_ok(k, splits):
+                continue
+            out = ops.gemm_mfma_wide(x.cuda(), w.cuda(), splits=splits).cpu()
+            total = out if splits == 1 else out.double().sum(0).float()
+            assert (total - ref).abs().max() <= 2e-5 * ref.abs().max(), (m, n, k, splits)
+    if n != 152064:
+        assert picked[8] == (4 if k == 3584 else 8), picked           # 8, 4 or 2 slices of 512 or more
+        if ops.compute_units() == 256:
+            assert picked[64] == {(3584, 18944): 9, (5120, 13824): 6, (5120, 27648): 6, (3584, 3584): 4}[(n, k)], picked
 
 
 def test_gemm_mfma_skinny_at_the_large_models_shapes(ops):
@@ -331,10 +339,11 @@ def test_gemm_mfma_wide_refuses_what_it_does_not_take(ops):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_rmsnorm_at_every_row_length_class(ops, dtype):
     """A thread of the vector kernel holds one to eight quads of the row (1,024 values a quad):
-    row lengths in every class, at its upper edge and just inside it, with eight partial sums."""
-    for hidden in (1024, 1028, 2560, 3072, 3584, 5120, 5124, 6144, 7000, 8192):
+    row lengths in every class, at its upper edge and just inside it, with eight partial sums (one of
+    the counts the kernel is made for, as 3, 6 and 9 are) or with 5, 7 or 16 (its loop over any count)."""
+    for i, hidden in enumerate((1024, 1028, 2560, 3072, 3584, 5120, 5124, 6144, 7000, 8192)):
         x, g = rnd((2, hidden), 40), rnd((hidden,), 41) + 1.0
-        parts = rnd((8, 2, hidden), 42)
+        parts = rnd(((8, 3, 5, 6, 9, 7, 16, 8, 9, 6)[i], 2, hidden), 42)
         summed = x + parts.double().sum(0).float()
         want = plain.rms_norm(summed, g, 1e-6)
         res = x.clone().cuda()
@@ -345,7 +354,7 @@ def test_rmsnorm_at_every_row_length_class(ops, dtype):
 
 def test_rmsnorm_adds_partial_sums_at_odd_sizes(ops):
     """Sizes the vector kernel does not take: hidden not a multiple of 4 and larger than its registers hold."""
-    for hidden, n_parts in [(102, 2), (9001 * 4, 4), (4099, 8)]:
+    for hidden, n_parts in [(102, 2), (9001 * 4, 4), (4099, 8), (4099, 9), (102, 5)]:
         x, g = rnd((3, hidden), 28), rnd((hidden,), 29) + 1.0
         parts = rnd((n_parts, 3, hidden), 30)
         summed = x + parts.double().sum(0).float()
