@@ -102,7 +102,7 @@ __global__ void embedding_vec_kernel(const T* __restrict__ table, const int32_t*
     Pack4<float>::store(out + static_cast<int64_t>(t) * hidden + j, ok ? v : float4{0.f, 0.f, 0.f, 0.f});
 }
 
-// DELTA: 0 = none, 1 = one array of T, 2 / 3 / 4 / 6 / 8 / 9 = that many float32 partial sums, added in
+// DELTA: 0 = none, 1 = one array of T, 2 to 9 = that many float32 partial sums, added in
 // order (every load of the row goes out before anything waits); -1 = `n_parts` of them (any other
 // number: a loop, four loads ahead).
 template <typename T, int ITERS, int DELTA, bool WRITE_BACK>
@@ -215,7 +215,9 @@ void launch_rmsnorm_vec(const NormCall& c) {
         case 2: return launch_rmsnorm_delta<T, ITERS, 2>(c);
         case 3: return launch_rmsnorm_delta<T, ITERS, 3>(c);
         case 4: return launch_rmsnorm_delta<T, ITERS, 4>(c);
+        case 5: return launch_rmsnorm_delta<T, ITERS, 5>(c);
         case 6: return launch_rmsnorm_delta<T, ITERS, 6>(c);
+        case 7: return launch_rmsnorm_delta<T, ITERS, 7>(c);
         case 8: return launch_rmsnorm_delta<T, ITERS, 8>(c);
         case 9: return launch_rmsnorm_delta<T, ITERS, 9>(c);
         default: return launch_rmsnorm_delta<T, ITERS, -1>(c);

@@ -236,10 +236,13 @@ extern "C" int fsie_gemm_mfma_wide_slice(int K, int splits) {
 // (Alone, N = K = 3584 at 8 rows takes 7.4 us in 7 slices against 8.4 for the few-rows kernel's 4; in
 // a whole decode step the norm that adds 7 parts instead of 4 costs more than that: 3.63 against
 // 3.56 ms a step of 28 layers.)
-// From 17 rows on a workgroup keeps its compute unit busy by itself (the reads of x from LDS and
-// the matrix instructions grow with the rows), and what counts is that all workgroups run at once
-// and leave few units idle: the cut that gives the most workgroups the device has units for
-// (64 rows on 256 units: N = 3584, K = 18944 in 9 slices, 252 workgroups, 32.4 us against 33.2 in 8;
+// From 17 rows on the workgroups keep a compute unit busy by themselves (the reads of x from LDS
+// and the matrix instructions grow with the rows): two of them with up to 32 rows, one beyond, and
+// what counts is that all workgroups run at once and leave few units idle: the cut that gives the
+// most workgroups the device has room for
+// (32 rows on 256 units: N = 3584, K = 18944 in 9 slices, 504 workgroups, 28.1 us against 29.2 in 8
+// and 38.5 in 4; N = 5120, K = 13824 in 6 slices, 480 workgroups, 29.2 against 35.2 in 8;
+// 64 rows: N = 3584, K = 18944 in 9 slices, 252 workgroups, 32.4 us against 33.2 in 8;
 // N = 5120, K = 13824 in 6 slices, 240 workgroups, 32.4 against 43.5 in 8, 320 workgroups;
 // N = 5120, K = 27648 in 6 slices 60.4 against 75.3; N = K = 5120 in 6 slices 17.4 against 21.6).
 extern "C" int fsie_gemm_mfma_wide_best_splits(int M, int N, int K) {
@@ -260,7 +263,7 @@ extern "C" int fsie_gemm_mfma_wide_best_splits(int M, int N, int K) {
         launch_shape(mt, N, s, waves, blocks);
         const int rows = 16 * blocks * waves;
         const int64_t groups = static_cast<int64_t>((N + rows - 1) / rows) * s;
-        const bool fits = groups <= units;
+        const bool fits = groups <= static_cast<int64_t>(units) * (mt == 2 ? 2 : 1);
         // among the cuts that fit, the most workgroups (of equals, the more slices: shorter ones);
         // if none fits, the fewest workgroups
         const bool better = best == 1 || (fits && !best_fits) || (fits == best_fits && (fits ? groups >= best_groups : groups < best_groups));

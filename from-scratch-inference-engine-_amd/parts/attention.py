@@ -25,11 +25,11 @@ class AttentionPlanner:
     ``small_tokens`` tokens is one *small* item.  A small item that reads more than ``split_keys``
     keys (decoding against a long context) is split over the keys into several items and merged
     afterwards in the order of the splits: 256 keys an item for the float32-arithmetic kernel (128
-    or 64 while the step has fewer workgroups than the device has compute units); for
+    or 64 by the same rule as below); for
     the matrix-core kernel, which gives every 128 keys to a wave of the item's workgroup and
-    combines those inside, 1,024 keys, or 512, 256 or 128 while the step has fewer workgroups than
-    the device has compute units (every wave still sums the same 128 keys; only where their sums
-    meet changes).  Longer portions are cut into *large* tiles of ``large_tokens``; how they are
+    combines those inside, 1,024 keys, or 512, 256 or 128 while that leaves the step with at most
+    as many workgroups as the device has compute units (every wave still sums the same 128 keys;
+    only where their sums meet changes).  Longer portions are cut into *large* tiles of ``large_tokens``; how they are
     cut depends on the portion alone, never on what else is in the batch.  The item table lists
     the small items first.
 
@@ -99,10 +99,15 @@ class AttentionPlanner:
         group = self.n_heads // self.n_kv
         # the float32-arithmetic kernel takes 32 keys a pass and up to 16 heads of a group a workgroup:
         # its items shorten to 64 keys (two passes) while compute units are idle
-        rows, shortest = (ops.attention_mfma_rows(self.head_dim, False), 128) if mfma else (16, 64)
+        rows, shortest, room = (ops.attention_mfma_rows(self.head_dim, False), 128, 1) if mfma else (16, 64, 2)
         per_item = self.n_kv * -(-group // min(group, rows))  # workgroups of one item
         split = longest
-        while split > shortest and sum(-(-k // split) for k in keys) * per_item < units:
+        # halved while the halves' workgroups still number at most the compute units: beyond that a
+        # split only adds a merge (48 requests of 600 keys, 192 workgroups whole: 4.59 ms a step;
+        # 384 of 512 keys each: 4.86).  The float32-arithmetic kernel's workgroups are slower and
+        # several share a unit: twice the units (8 requests of 640 keys, 28 layers of the 32-bit
+        # path: 8.5 ms a step with 64 keys an item, 9.1 with 128)
+        while split > shortest and sum(-(-k // (split // 2)) for k in keys) * per_item <= units * room:
             split //= 2
         return split
 

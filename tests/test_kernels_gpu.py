@@ -340,10 +340,10 @@ def test_gemm_mfma_wide_refuses_what_it_does_not_take(ops):
 def test_rmsnorm_at_every_row_length_class(ops, dtype):
     """A thread of the vector kernel holds one to eight quads of the row (1,024 values a quad):
     row lengths in every class, at its upper edge and just inside it, with eight partial sums (one of
-    the counts the kernel is made for, as 3, 6 and 9 are) or with 5, 7 or 16 (its loop over any count)."""
+    the counts the kernel is made for, as all from 2 to 9 are) or with 10, 12 or 16 (its loop over any count)."""
     for i, hidden in enumerate((1024, 1028, 2560, 3072, 3584, 5120, 5124, 6144, 7000, 8192)):
         x, g = rnd((2, hidden), 40), rnd((hidden,), 41) + 1.0
-        parts = rnd(((8, 3, 5, 6, 9, 7, 16, 8, 9, 6)[i], 2, hidden), 42)
+        parts = rnd(((8, 3, 5, 6, 9, 7, 16, 12, 10, 2)[i], 2, hidden), 42)
         summed = x + parts.double().sum(0).float()
         want = plain.rms_norm(summed, g, 1e-6)
         res = x.clone().cuda()
@@ -579,8 +579,14 @@ def test_attention_over_pages(ops, dtype, scalar, heads, kv, hd, page, window):
 def test_attention_over_pages_at_the_lengths_that_are_timed(ops, heads, kv, seqs):
     """The prompt and context lengths that the measurements quote, at the head geometries of the
     large models (head size 128, page 16, bfloat16), against the plain attention."""
+    from from_scratch_inference_engine_amd.parts.attention import AttentionPlanner
+
     hd, page = 128, 16
-    case = paged_case(seqs, heads, kv, hd, page, torch.bfloat16, seed=heads)
+    AttentionPlanner.compute_units = 4096  # as on a device with so many idle units: the decode is cut into items of 128 keys
+    try:
+        case = paged_case(seqs, heads, kv, hd, page, torch.bfloat16, seed=heads)
+    finally:
+        AttentionPlanner.compute_units = None
     plan = case["plan"]
     assert plan["mfma"] and (plan["n_groups"] > 100 or plan["n_merges"])
     out = run_attention(ops, case, heads, kv, hd)
