@@ -125,7 +125,7 @@ def test_decode_items_shorten_while_compute_units_are_idle():
     planner = AttentionPlanner(28, 4, 128, None)
     planner.compute_units = 256
     for n_requests, keys, split in ((8, 640, 128), (1, 3550, 128), (64, 640, 1024), (8, 16000, 1024), (20, 3000, 1024), (12, 1500, 512),
-                                   (48, 600, 1024), (8, 3550, 512)):
+                                   (48, 600, 1024), (8, 3550, 512), (32, 600, 1024), (24, 600, 1024), (16, 640, 256)):
         host = Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16)
         assert planner.split_keys(host, True) == split
         plan = planner.plan(host)
@@ -134,7 +134,7 @@ def test_decode_items_shorten_while_compute_units_are_idle():
         assert plan["waves"] == {128: 1, 256: 2, 512: 4, 1024: 8}[split]  # one wave per 128 keys
         assert plan["n_merges"] == (n_requests if keys > split else 0)
     # the float32-arithmetic kernel: 256 keys an item on a full device, down to 64 (two passes of 32) on an idle one
-    for n_requests, keys, split in ((1, 5000, 64), (8, 640, 64), (64, 640, 256), (4, 2000, 64), (16, 2000, 256)):
+    for n_requests, keys, split in ((1, 5000, 64), (8, 640, 64), (64, 640, 256), (4, 2000, 128), (16, 2000, 256)):
         host = Host([(keys - 1, 1)] * n_requests, 16, torch.float32)
         assert planner.split_keys(host, False) == split
         plan = planner.plan(host)
