@@ -95,6 +95,7 @@ def kernel_classes(runner, cfg, batch: int, prompt_len: int, itemsize: int) -> d
         "attention_mfma": lambda a, k: "attention", "attention_mfma_lds": lambda a, k: "attention",
         "attention_scalar": lambda a, k: "attention", "attention_merge": lambda a, k: "attention",
         "gemm_mfma_skinny": lambda a, k: matrix_class(a[1]), "gemm_mfma_wide": lambda a, k: matrix_class(a[1]),
+        "gemm_mfma_wide_swiglu": lambda a, k: "gate_up",
         "gemm": lambda a, k: matrix_class(a[1]), "gemm_mfma_fp32": lambda a, k: matrix_class(a[1]),
         "library_mm": lambda a, k: matrix_class(a[1]),
         "swiglu": lambda a, k: "gate_up", "rmsnorm": lambda a, k: "norms", "embedding": lambda a, k: "other",

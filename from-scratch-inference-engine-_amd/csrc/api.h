@@ -91,6 +91,9 @@ int fsie_gemm_mfma_wide_slice(int K, int splits);
 int fsie_gemm_mfma_wide_best_splits(int M, int N, int K);
 int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits, int waves,
                         int blocks, hipStream_t stream);
+// the rows of w are gate and up in turn: y is bfloat16 [M, N / 2], silu(gate) * up
+int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int N, int K, int waves, int blocks,
+                               hipStream_t stream);
 
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,

@@ -45,7 +45,9 @@ union Frag {
 // MT tiles of 16 rows of X; WAVES waves of NB blocks of 16 rows of W each per workgroup (a wave's
 // blocks share the B fragments it reads from LDS: with four tiles of X one block a wave would be
 // bound by those reads); STEPS 32-wide MFMA steps per stage (KS = 32 * STEPS values of K).
-template <int MT, int WAVES, int STEPS, int NB>
+// SWIGLU: the rows of W are gate and up interleaved and y is bfloat16 [M, N / 2], silu(gate) * up
+// from the accumulators (a lane holds rows 4 kg .. 4 kg + 3 of a block: two pairs); one slice only.
+template <int MT, int WAVES, int STEPS, int NB, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t* __restrict__ x,
                                                                    const bf16_t* __restrict__ w,
                                                                    float* __restrict__ y, int M, int N, int K,
@@ -152,6 +154,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
     }
 
     // lane holds D[n0 + 16 nb + 4 kg + r][m = 16 t + row]
+    if constexpr (SWIGLU) {
+        uint32_t* out = reinterpret_cast<uint32_t*>(y);  // two bfloat16 results a store: columns nn / 2 and nn / 2 + 1
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const int m = t * 16 + row;
+                const int nn = n0 + nb * 16 + kg * 4;  // a multiple of 4: gate, up, gate, up
+                if (m >= M || nn >= N) continue;      // N is a multiple of 4 here (checked by the host)
+                const float g0 = acc[nb][t][0], u0 = acc[nb][t][1], g1 = acc[nb][t][2], u1 = acc[nb][t][3];
+                out[(static_cast<int64_t>(m) * (N / 2) + nn / 2) / 2] =
+                    pack2_bf16((g0 / (1.0f + expf(-g0))) * u0, (g1 / (1.0f + expf(-g1))) * u1);
+            }
+        return;
+    }
     float* part = y + static_cast<int64_t>(blockIdx.y) * M * N;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
@@ -167,25 +184,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
         }
 }
 
-template <int MT, int WAVES, int STEPS, int NB>
+template <int MT, int WAVES, int STEPS, int NB, bool SWIGLU>
 int launch(const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
            hipStream_t stream) {
     const int rows = 16 * NB * WAVES;
     const dim3 grid(static_cast<unsigned>((N + rows - 1) / rows), static_cast<unsigned>(splits));
-    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB><<<grid, WAVES * 64, 0, stream>>>(x, w, y, M, N, K, k_slice);
+    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB, SWIGLU><<<grid, WAVES * 64, 0, stream>>>(x, w, y, M, N, K, k_slice);
     FSIE_CHECK_LAUNCH("gemm_mfma_wide");
     return 0;
 }
 
-template <int WAVES, int STEPS, int NB>
+template <int WAVES, int STEPS, int NB, bool SWIGLU = false>
 int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
               hipStream_t stream) {
     switch (mt) {
-        case 1: return launch<1, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
-        case 2: return launch<2, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 1: return launch<1, WAVES, STEPS, NB, SWIGLU>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 2: return launch<2, WAVES, STEPS, NB, SWIGLU>(x, w, y, M, N, K, splits, k_slice, stream);
 #if FSIE_WIDE_STEPS <= 4
-        case 3: return launch<3, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
-        default: return launch<4, WAVES, STEPS, NB>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 3: return launch<3, WAVES, STEPS, NB, SWIGLU>(x, w, y, M, N, K, splits, k_slice, stream);
+        default: return launch<4, WAVES, STEPS, NB, SWIGLU>(x, w, y, M, N, K, splits, k_slice, stream);
 #else
         default: fsie_set_error("gemm_mfma_wide: stages of %d steps hold at most 32 rows", STEPS); return 1;
 #endif
@@ -193,12 +210,18 @@ int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, 
 }
 
 // Waves a workgroup and row blocks a wave where the caller leaves them open (0).
-void launch_shape(int mt, int N, int splits, int& waves, int& blocks) {
+void launch_shape(int mt, int N, int splits, int& waves, int& blocks, bool gate_up = false) {
     if (blocks == 0) {
         // three or four tiles of X: two blocks of W a wave share the B fragments read from LDS,
         // where that still leaves a workgroup for most compute units (measured on MI355X, 64 rows,
         // N = 3584, K = 18944 in 8 slices: 33.6 against 37.7 us)
         blocks = (mt >= 3 && static_cast<int64_t>((N + 127) / 128) * splits >= 128) ? 2 : 1;
+        // gate and up of one or two tiles at a very large N: two blocks a wave once that still gives
+        // every compute unit a workgroup and a half (N = 55296, K = 5120, 8 rows: 107 against 112 us;
+        // N = 27648: 56.6 against 52.5, N = 37888: 65 against 54, so not there)
+        const int units = fsie_compute_units();
+        if (gate_up && mt < 3 && units > 0 && static_cast<int64_t>((N + 127) / 128) * 2 >= 3 * static_cast<int64_t>(units))
+            blocks = 2;
     }
     if (waves == 0) {
         // eight waves a workgroup halve the reads of X, but only a large N leaves enough
@@ -300,4 +323,35 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
     if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
     if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
     return launch_mt<4, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+}
+
+// The same product with the rows of w as gate and up in turn: y is bfloat16 [M, N / 2], silu(gate) * up.
+// N a multiple of 4; one slice of K.
+extern "C" int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int N, int K, int waves,
+                                          int blocks, hipStream_t stream) {
+    FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide_swiglu: bad sizes M=%d N=%d K=%d", M, N, K);
+    FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide_swiglu: at most %d rows, got %d",
+                 FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
+    FSIE_REQUIRE(N % 4 == 0, "gemm_mfma_wide_swiglu: N=%d must be a multiple of 4 (gate and up rows in turn)", N);
+    const int k_slice = fsie_gemm_mfma_wide_slice(K, 1);
+    FSIE_REQUIRE(k_slice > 0, "gemm_mfma_wide_swiglu: K=%d must be a multiple of the stage of %d", K, 32 * FSIE_WIDE_STEPS);
+    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(y) % 4 == 0,
+                 "gemm_mfma_wide_swiglu: operands must be 16-byte aligned, the result 4-byte");
+    FSIE_REQUIRE(waves == 0 || waves == 2 || waves == 4 || waves == 8, "gemm_mfma_wide_swiglu: waves must be 0, 2, 4 or 8");
+    FSIE_REQUIRE(blocks == 0 || blocks == 1 || blocks == 2, "gemm_mfma_wide_swiglu: blocks must be 0, 1 or 2");
+    if (M == 0) return 0;
+    const int mt = (M + 15) / 16;
+    launch_shape(mt, N, 1, waves, blocks, true);
+    const bf16_t* xp = static_cast<const bf16_t*>(x);
+    const bf16_t* wq = static_cast<const bf16_t*>(w);
+    float* yp = static_cast<float*>(y);
+    if (blocks == 2) {
+        if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 2, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
+        if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 2, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
+        return launch_mt<4, FSIE_WIDE_STEPS, 2, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
+    }
+    if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 1, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
+    if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 1, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
+    return launch_mt<4, FSIE_WIDE_STEPS, 1, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
 }

@@ -311,6 +311,26 @@ def gemm_mfma_wide_splits_ok(k: int, splits: int) -> bool:
     return load().fsie_gemm_mfma_wide_slice(int(k), int(splits)) > 0
 
 
+def gemm_mfma_wide_swiglu(x: torch.Tensor, weight: torch.Tensor, waves: int = 0, blocks: int = 0,
+                          out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """silu(gate) * up [M, N/2] (bfloat16) of x [M, K] and a weight [N, K] whose rows are gate and up
+    in turn, by the kernel that shares x through LDS; up to 64 rows, N a multiple of 4, K of 128."""
+    _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
+    _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
+    m, k = x.shape
+    n = weight.shape[0]
+    if weight.shape[1] != k:
+        raise KernelError(f"gemm: weight inner size {weight.shape[1]} does not match x's {k}")
+    if n % 4:
+        raise KernelError(f"gemm_mfma_wide_swiglu: the number of weight rows {n} must be a multiple of 4")
+    if out is None:
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+    _need(out, "gemm out", dtype=torch.bfloat16, shape=(m, n // 2))
+    check(load().fsie_gemm_mfma_wide_swiglu(x.data_ptr(), weight.data_ptr(), out.data_ptr(), m, n, k, waves, blocks,
+                                            _stream()))
+    return out
+
+
 def gemm_mfma_wide_best_splits(m: int, n: int, k: int) -> int:
     """Into how many slices of K ``gemm_mfma_wide`` best cuts a product of ``m`` rows that leaves
     partial sums (1: it does not cut, or does not take this K)."""
@@ -321,7 +341,7 @@ def gemm_mfma_wide(x: torch.Tensor, weight: torch.Tensor, splits: int = 1, waves
                    out: Optional[torch.Tensor] = None, blocks: int = 0) -> torch.Tensor:
     """x [M, K] . weight [N, K]^T for bfloat16 operands and up to 64 rows, the rows of x shared by
     a workgroup's waves through LDS (made for 17 rows and more).  The result is float32: [M, N],
-    or with ``splits`` in (2, 4, 8) the partial sums [splits, M, N] of the slices of K, for
+    or with ``splits`` of 2 to 16 the partial sums [splits, M, N] of the slices of K, for
     ``rmsnorm`` to add up.  K must be a multiple of 128 that the slices cover in whole stages
     (``gemm_mfma_wide_splits_ok``)."""
     _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)

@@ -48,7 +48,15 @@ class SwiGLU(FeedForward):
         self.down.weight = t
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        if (x.dtype == torch.bfloat16 and x.shape[0] <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 8 == 0):
+        m = x.shape[0]
+        if (x.dtype == torch.bfloat16 and 3 <= m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 128 == 0
+                and self.gate_up.out_features % 4 == 0 and self.gate_up.out_features // 64 >= ops.compute_units()):
+            # three rows and more of a matrix that gives every compute unit a workgroup: the kernel that
+            # shares x through LDS (MI355X, 8 rows: N = 37888, K = 3584 49.3 against 51.2 us; N = 27648,
+            # K = 5120 57.2 against 62.4; N = 55296, K = 5120 110.5 against 118.7, at 16 rows 106 against
+            # 129; one or two rows, and N = 9728, K = 896, are faster in the other)
+            act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.weight)
+        elif x.dtype == torch.bfloat16 and m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 8 == 0:
             act = ops.gemm_mfma_skinny(x, self.gate_up.weight, epilogue="swiglu")
         else:
             act = ops.swiglu(self.gate_up(x))

@@ -430,6 +430,25 @@ def test_gemm_mfma_skinny_with_swiglu_epilogue(ops, m, n, k):
     assert (out.float().cpu() - ref).abs().max() <= tol(torch.bfloat16, ref)
 
 
+@pytest.mark.parametrize("m, n, k", [(3, 9728, 896), (8, 356, 128), (13, 644, 384), (16, 37888, 3584), (40, 1028, 256),
+                                     (64, 27648, 5120), (9, 55296, 5120)])
+def test_gemm_mfma_wide_with_swiglu_epilogue(ops, m, n, k):
+    """The kernel that shares x through LDS with silu(gate) * up from its accumulators: every number of
+    16-row tiles, an N that ends inside a block of rows, one and two blocks a wave, and the gate/up
+    shapes of the large models."""
+    from from_scratch_inference_engine_amd.ops import KernelError
+
+    x, w = rnd((m, k), 17, torch.bfloat16), rnd((n, k), 18, torch.bfloat16, 0.05)
+    full = (x.cuda().double() @ w.cuda().double().t()).float().cpu()
+    ref = plain.silu_mul(full[:, 0::2], full[:, 1::2])
+    for waves, blocks in ((0, 0), (2, 2), (8, 1)):
+        out = ops.gemm_mfma_wide_swiglu(x.cuda(), w.cuda(), waves=waves, blocks=blocks)
+        assert out.shape == (m, n // 2) and out.dtype == torch.bfloat16
+        assert (out.float().cpu() - ref).abs().max() <= tol(torch.bfloat16, ref), (waves, blocks)
+    with pytest.raises(KernelError, match="multiple of 4"):
+        ops.gemm_mfma_wide_swiglu(x.cuda(), w[:n - 2].contiguous().cuda())
+
+
 def test_refusals(ops):
     from from_scratch_inference_engine_amd.ops import KernelError
 
