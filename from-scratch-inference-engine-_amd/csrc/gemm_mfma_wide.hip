@@ -255,10 +255,11 @@ extern "C" int fsie_gemm_mfma_wide_slice(int K, int splits) {
 
 // Into how many slices of K a product of M rows that leaves partial sums is best cut (1: not at
 // all, or this kernel does not take K).  A slice is at least 512 long.
-// Up to 16 rows: 8, 4 or 2, the most that K gives: many short workgroups, several a compute unit.
-// (Alone, N = K = 3584 at 8 rows takes 7.4 us in 7 slices against 8.4 for the few-rows kernel's 4; in
-// a whole decode step the norm that adds 7 parts instead of 4 costs more than that: 3.63 against
-// 3.56 ms a step of 28 layers.)
+// Up to 16 rows: as many slices as K gives, up to 8: many short workgroups, several a compute unit
+// (N = K = 3584 on MI355X, 8 rows: 7 slices 7.4 us, 6 7.2, 4 9.3, the few-rows kernel's 4 8.4; the
+// norm that then adds 7 parts instead of 4 takes 0.6 us longer, which leaves 0.03 ms of a decode
+// step of 28 layers; with a norm that loops over the parts instead of asking for all at once it
+// cost 0.07 ms more than it brought).
 // From 17 rows on the workgroups keep a compute unit busy by themselves (the reads of x from LDS
 // and the matrix instructions grow with the rows): two of them with up to 32 rows, one beyond, and
 // what counts is that all workgroups run at once and leave few units idle: the cut that gives the
@@ -273,7 +274,7 @@ extern "C" int fsie_gemm_mfma_wide_best_splits(int M, int N, int K) {
     const int mt = (M + 15) / 16;
     const int units = fsie_compute_units();
     if (mt <= 1 || units <= 0) {
-        for (int s = 8; s >= 2; s /= 2)
+        for (int s = 8; s >= 2; --s)
             if (K / s >= 512 && fsie_gemm_mfma_wide_slice(K, s) > 0) return s;
         return 1;
     }

@@ -78,10 +78,10 @@ class Linear:
         if (getattr(ctx, "partial_sums_ok", False) and x.dtype == torch.bfloat16 and self.bias is None
                 and self.in_features % 8 == 0 and 0 < m <= GEMM_MFMA_SKINNY_MAX_M):
             # the kernel that shares x through LDS: above 16 rows, and at any number of rows where
-            # K is long enough for eight slices (N = 3584, K = 18944: 26 against 28 us at 8 rows,
-            # 27 against 32 at 16)
+            # K is long enough for six slices or more (N = 3584, K = 18944 in 8: 26 against 28 us at 8
+            # rows, 27 against 32 at 16; N = K = 3584 in 7: 7.4 against 8.4 at 8 rows)
             splits = self.wide_splits(m)
-            if splits > 1 and (m > GEMM_MFMA_SKINNY_BEST_M or splits == 8):
+            if splits > 1 and (m > GEMM_MFMA_SKINNY_BEST_M or splits >= 6):
                 return ops.gemm_mfma_wide(x, self.weight, splits=splits)
             splits = self.residual_splits(m)
             if splits > 1:
@@ -90,8 +90,8 @@ class Linear:
 
     def wide_splits(self, m: int) -> int:
         """Slices of K for the kernel that shares x through LDS, by the tiles of 16 rows that ``m``
-        rows make (the kernel's own rule: 8, 4 or 2, the most that K gives, for up to 16 rows; from 17
-        rows on the cut that gives the most workgroups the device has compute units for).  1 = it does
+        rows make (the kernel's own rule: as many as K gives, up to 8, for up to 16 rows; from 17
+        rows on the cut that gives the most workgroups the device has room for).  1 = it does
         not take this K.  (64 rows on MI355X: N = 3584, K = 18944 in 9 slices 32 us, against 68 for
         the few-rows kernel and 91 for the library; N = K = 3584 in 4 slices 10.9 against the
         library's 13.7.)"""

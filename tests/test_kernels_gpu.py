@@ -293,7 +293,7 @@ def test_gemm_mfma_wide_at_the_large_models_shapes(ops, n, k):
             total = out if splits == 1 else out.double().sum(0).float()
             assert (total - ref).abs().max() <= 2e-5 * ref.abs().max(), (m, n, k, splits)
     if n != 152064:
-        assert picked[8] == (4 if k == 3584 else 8), picked           # 8, 4 or 2 slices of 512 or more
+        assert picked[8] == (7 if k == 3584 else 8), picked           # as many slices of 512 or more as K gives, up to 8
         if ops.compute_units() == 256:
             assert picked[64] == {(3584, 18944): 9, (5120, 13824): 6, (5120, 27648): 6, (3584, 3584): 4}[(n, k)], picked
 
