@@ -219,6 +219,32 @@ def test_graft_entry_smoke():
     entry.smoke()
 
 
+def test_bench_prints_its_line():
+    """bench.py as it is run for the record, at a small shape (two layers of 896 / 4864): the library's
+    kernels chosen by timing, prefill, decode at batch 8, 1 and 64 through the engine, the time of each
+    class of kernels; one JSON line with the fields of the contract.  More than one GPU: one line, exit 2."""
+    cmd = [sys.executable, "bench.py", "--shape", "0.5b", "--layers", "2", "--steps", "8", "--warmup", "4"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300, cwd=str(helpers.ROOT))
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = proc.stdout.strip().splitlines()
+    assert len(lines) == 1, lines
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "prefill", "roofline", "points", "kernels"):
+        assert key in rec, key
+    assert rec["n_gpus"] == 1 and rec["steps"] == 8 and rec["warmup"] == 4 and rec["dtype"] == "bf16"
+    assert rec["value"] > 0 and abs(rec["value"] - 8 / (rec["ms_per_step"] * 1e-3)) <= 1e-6 * rec["value"]
+    assert len(rec["config"]) <= 20 and all(not isinstance(v, (dict, list)) for v in rec["config"].values())
+    assert rec["config"]["layers"] == 2 and rec["config"]["layers_of_config"] == 24
+    assert rec["prefill"]["tokens"] == 2048 and 0 < rec["prefill"]["frac"] < 1
+    assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0 and 0 < rec["roofline"]["frac"] < 1
+    assert set(rec["points"]) == {"decode_b1", "decode_b64"}
+    assert {"attention", "qkv", "gate_up", "down", "o", "norms", "lm_head"} <= set(rec["kernels"])
+    assert all(v["ms"] > 0 and v["launches"] > 0 for v in rec["kernels"].values())
+    two = subprocess.run(cmd[:2] + ["--gpus", "2"], capture_output=True, text=True, timeout=120, cwd=str(helpers.ROOT))
+    assert two.returncode == 2 and len(two.stdout.strip().splitlines()) == 1
+
+
 def test_graph_replays_equal_eager_steps(model_dirs):
     """Decode steps run as replayed graphs.  Two runners over the same model, one with graphs and
     one without, decode the same 20 requests (more rows than the engine's own small-matrix kernel
