@@ -89,11 +89,17 @@ int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const float* bias, 
 // 17 to 64 rows (any number up to 64 is taken): X shared through LDS, float32 result or partial sums
 int fsie_gemm_mfma_wide_slice(int K, int splits);
 int fsie_gemm_mfma_wide_best_splits(int M, int N, int K);
+// (frags: w is the copy of the matrix in the order of the A fragments, made by fsie_fragment_order)
 int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits, int waves,
-                        int blocks, hipStream_t stream);
+                        int blocks, int frags, hipStream_t stream);
 // the rows of w are gate and up in turn: y is bfloat16 [M, N / 2], silu(gate) * up
 int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int N, int K, int waves, int blocks,
-                               hipStream_t stream);
+                               int frags, hipStream_t stream);
+// A bfloat16 matrix [N, K] (K a multiple of 32) copied so that the 64 16-byte units of a block of 16
+// rows and 32 values of K lie together in the order of the lanes that hold them: a wave's load of W
+// is then one piece of 1 KB.  The copy has fsie_fragment_order_size values (N rounded up to 16 rows).
+int64_t fsie_fragment_order_size(int N, int K);
+int fsie_fragment_order(const void* w, void* out, int N, int K, hipStream_t stream);
 
 int fsie_attention_scalar(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                           const int32_t* block_tables, int max_pages, const int32_t* items, int n_items,

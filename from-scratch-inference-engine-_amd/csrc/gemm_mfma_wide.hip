@@ -18,6 +18,14 @@
 //
 // blockIdx.y selects a slice of K (a multiple of KS); with more than one slice y is
 // [slices][M][N], float32 partial sums for the consumer to add in the order of the slices.
+//
+// W may also come in the order of the A fragments (fsie_fragment_order): the 64 16-byte units of a
+// block of 16 rows and a step of 32 values of K lie together, in the order of the lanes that hold
+// them, block after block along K and then along N.  A wave's load is then one piece of 1 KB
+// instead of 16 pieces of 64 bytes, and W can be read with streaming (non-temporal) loads.  Measured
+// on MI355X with kernels that only read 272 MB (N = 37888, K = 3584): rows, plain loads 48 us
+// (this kernel's product takes as long); rows, streaming loads 52; fragment order, plain 46.5;
+// fragment order, streaming 41.3.
 #include "common.h"
 #include "api.h"
 
@@ -47,7 +55,7 @@ union Frag {
 // bound by those reads); STEPS 32-wide MFMA steps per stage (KS = 32 * STEPS values of K).
 // SWIGLU: the rows of W are gate and up interleaved and y is bfloat16 [M, N / 2], silu(gate) * up
 // from the accumulators (a lane holds rows 4 kg .. 4 kg + 3 of a block: two pairs); one slice only.
-template <int MT, int WAVES, int STEPS, int NB, bool SWIGLU>
+template <int MT, int WAVES, int STEPS, int NB, bool SWIGLU, bool FRAGS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t* __restrict__ x,
                                                                    const bf16_t* __restrict__ w,
                                                                    float* __restrict__ y, int M, int N, int K,
@@ -72,10 +80,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
     const int n_stages = (k_end - k_begin) / KS;  // the host makes every slice a multiple of KS
 
     // rows of W past the end repeat the last one; their results are never written
+    // W_STEP: values between a lane's fragments of consecutive steps
+    constexpr int W_STEP = FRAGS ? 512 : 32;
     const bf16_t* wp[NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-        wp[nb] = w + static_cast<int64_t>(min(n0 + nb * 16 + row, N - 1)) * K + k_begin + kg * 8;
+    for (int nb = 0; nb < NB; ++nb) {
+        if constexpr (FRAGS)  // blocks past the end repeat the last one (the copy is padded to whole blocks)
+            wp[nb] = w + (static_cast<int64_t>(min(n0 / 16 + nb, (N - 1) / 16)) * (K / 32) + k_begin / 32) * 512 + lane * 8;
+        else
+            wp[nb] = w + static_cast<int64_t>(min(n0 + nb * 16 + row, N - 1)) * K + k_begin + kg * 8;
+    }
+    auto load_w = [](const bf16_t* p) -> u32x4 {
+        if constexpr (FRAGS) return __builtin_nontemporal_load((GlobalVec)p);
+        else return *(GlobalVec)p;
+    };
     // staging: unit u = (row of X, j = step * 4 + k group); consecutive threads take consecutive
     // 16 bytes of a row
     const bf16_t* xsrc[PER_THREAD];
@@ -104,7 +122,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) wa[s][nb].q = *(GlobalVec)(wp[nb] + s * 32);
+        for (int nb = 0; nb < NB; ++nb) wa[s][nb].q = load_w(wp[nb] + s * W_STEP);
 #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i) xs[0][xdst[i]] = xr[i];
     __syncthreads();
@@ -133,7 +151,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
 #pragma unroll
         for (int s = 0; s < STEPS; ++s)
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) wn[s][nb].q = *(GlobalVec)(wp[nb] + k1 + s * 32);
+            for (int nb = 0; nb < NB; ++nb) wn[s][nb].q = load_w(wp[nb] + k1 * (W_STEP / 32) + s * W_STEP);
         __builtin_amdgcn_sched_barrier(0);
         products(buf, wc);
         __builtin_amdgcn_sched_barrier(0);
@@ -184,33 +202,80 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
         }
 }
 
-template <int MT, int WAVES, int STEPS, int NB, bool SWIGLU>
+template <int MT, int WAVES, int STEPS, int NB, bool SWIGLU, bool FRAGS>
 int launch(const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
            hipStream_t stream) {
     const int rows = 16 * NB * WAVES;
     const dim3 grid(static_cast<unsigned>((N + rows - 1) / rows), static_cast<unsigned>(splits));
-    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB, SWIGLU><<<grid, WAVES * 64, 0, stream>>>(x, w, y, M, N, K, k_slice);
+    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB, SWIGLU, FRAGS><<<grid, WAVES * 64, 0, stream>>>(x, w, y, M, N, K, k_slice);
     FSIE_CHECK_LAUNCH("gemm_mfma_wide");
     return 0;
 }
 
-template <int WAVES, int STEPS, int NB, bool SWIGLU = false>
+template <int WAVES, int STEPS, int NB, bool SWIGLU, bool FRAGS>
 int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int splits, int k_slice,
               hipStream_t stream) {
     switch (mt) {
-        case 1: return launch<1, WAVES, STEPS, NB, SWIGLU>(x, w, y, M, N, K, splits, k_slice, stream);
-        case 2: return launch<2, WAVES, STEPS, NB, SWIGLU>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 1: return launch<1, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 2: return launch<2, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
 #if FSIE_WIDE_STEPS <= 4
-        case 3: return launch<3, WAVES, STEPS, NB, SWIGLU>(x, w, y, M, N, K, splits, k_slice, stream);
-        default: return launch<4, WAVES, STEPS, NB, SWIGLU>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 3: return launch<3, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+        default: return launch<4, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
 #else
         default: fsie_set_error("gemm_mfma_wide: stages of %d steps hold at most 32 rows", STEPS); return 1;
 #endif
     }
 }
 
+template <bool SWIGLU, bool FRAGS>
+int launch_shape_of(int mt, int waves, int blocks, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K,
+                    int splits, int k_slice, hipStream_t stream) {
+    if (blocks == 2) {
+        if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+        if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+        return launch_mt<4, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+    }
+    if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+    if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+    return launch_mt<4, FSIE_WIDE_STEPS, 1, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+}
+
+// One thread a 16-byte unit of the copy: unit ((block, step), lane) holds the 8 values at row
+// 16 block + (lane & 15), k = 32 step + 8 (lane >> 4); rows past N are zeros.
+__global__ __launch_bounds__(256) void fragment_order_kernel(const u32x4* __restrict__ w, u32x4* __restrict__ out,
+                                                             int N, int K, int64_t units) {
+    const int64_t u = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (u >= units) return;
+    const int lane = static_cast<int>(u & 63);
+    const int64_t bs = u >> 6;
+    const int steps = K / 32;
+    const int64_t block = bs / steps;
+    const int step = static_cast<int>(bs - block * steps);
+    const int64_t n = block * 16 + (lane & 15);
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (n < N) v = w[(n * K + step * 32 + (lane >> 4) * 8) / 8];
+    out[u] = v;
+}
+
 // Waves a workgroup and row blocks a wave where the caller leaves them open (0).
 void launch_shape(int mt, int N, int splits, int& waves, int& blocks, bool gate_up = false) {
+    if (gate_up && mt >= 2 && waves == 0 && blocks == 0) {
+        // 17 rows and more, one slice: the products and the reads of x from LDS bound a workgroup, so
+        // a compute unit with two workgroups takes twice as long as one with one.  The largest
+        // workgroups (they lay x into LDS least often) that still occupy more than half of the units,
+        // one each (MI355X, 256 units, 64 rows, fragment-ordered W: N = 37888, K = 3584 in 148
+        // workgroups of 256 rows 52.5 us, in 296 of 128 rows 62.1; N = 27648, K = 5120 in 216 of 128
+        // rows 48.8, in 108 of 256 rows 69.3; N = 55296, K = 5120 in 216 of 256 rows 86.6, in 432 of
+        // 128 rows 96.1)
+        const int units = fsie_compute_units();
+        static const int shapes[4][2] = {{8, 2}, {4, 2}, {2, 2}, {2, 1}};
+        for (const auto& shape : shapes) {
+            const int rows = 16 * shape[0] * shape[1];
+            waves = shape[0], blocks = shape[1];
+            if (static_cast<int64_t>((N + rows - 1) / rows) * 20 >= static_cast<int64_t>(units) * 11) break;
+        }
+        return;
+    }
     if (blocks == 0) {
         // three or four tiles of X: two blocks of W a wave share the B fragments read from LDS,
         // where that still leaves a workgroup for most compute units (measured on MI355X, 64 rows,
@@ -300,8 +365,9 @@ extern "C" int fsie_gemm_mfma_wide_best_splits(int M, int N, int K) {
 // 1 <= M <= 64; K a multiple of 128 that `splits` slices of whole stages cover (see above);
 // x and w 16-byte aligned.  waves: 2, 4 or 8 waves per workgroup; blocks: 1 or 2 blocks of 16 rows
 // of W per wave; 0 = choose.
+// frags: w is the copy that fsie_fragment_order made of the [N, K] matrix.
 extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits,
-                                   int waves, int blocks, hipStream_t stream) {
+                                   int waves, int blocks, int frags, hipStream_t stream) {
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide: bad sizes M=%d N=%d K=%d", M, N, K);
     FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide: at most %d rows, got %d",
                  FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
@@ -316,20 +382,14 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
     launch_shape(mt, N, splits, waves, blocks);
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
-    if (blocks == 2) {
-        if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-        if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-        return launch_mt<4, FSIE_WIDE_STEPS, 2>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-    }
-    if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-    if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
-    return launch_mt<4, FSIE_WIDE_STEPS, 1>(mt, xp, wq, y, M, N, K, splits, k_slice, stream);
+    if (frags) return launch_shape_of<false, true>(mt, waves, blocks, xp, wq, y, M, N, K, splits, k_slice, stream);
+    return launch_shape_of<false, false>(mt, waves, blocks, xp, wq, y, M, N, K, splits, k_slice, stream);
 }
 
 // The same product with the rows of w as gate and up in turn: y is bfloat16 [M, N / 2], silu(gate) * up.
 // N a multiple of 4; one slice of K.
 extern "C" int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int N, int K, int waves,
-                                          int blocks, hipStream_t stream) {
+                                          int blocks, int frags, hipStream_t stream) {
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide_swiglu: bad sizes M=%d N=%d K=%d", M, N, K);
     FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide_swiglu: at most %d rows, got %d",
                  FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
@@ -347,12 +407,26 @@ extern "C" int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y,
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
     float* yp = static_cast<float*>(y);
-    if (blocks == 2) {
-        if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 2, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
-        if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 2, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
-        return launch_mt<4, FSIE_WIDE_STEPS, 2, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
-    }
-    if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 1, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
-    if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 1, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
-    return launch_mt<4, FSIE_WIDE_STEPS, 1, true>(mt, xp, wq, yp, M, N, K, 1, k_slice, stream);
+    if (frags) return launch_shape_of<true, true>(mt, waves, blocks, xp, wq, yp, M, N, K, 1, k_slice, stream);
+    return launch_shape_of<true, false>(mt, waves, blocks, xp, wq, yp, M, N, K, 1, k_slice, stream);
+}
+
+// The copy of a bfloat16 matrix w [N, K] in the order of the matrix instruction's A fragments, for
+// the products above with frags set: out holds ceil(N / 16) * 16 * K values (fsie_fragment_order_size),
+// the rows past N zeros.  K a multiple of 32; w and out 16-byte aligned and distinct.
+extern "C" int64_t fsie_fragment_order_size(int N, int K) {
+    if (N <= 0 || K <= 0 || K % 32) return 0;
+    return static_cast<int64_t>((N + 15) / 16) * 16 * K;
+}
+
+extern "C" int fsie_fragment_order(const void* w, void* out, int N, int K, hipStream_t stream) {
+    FSIE_REQUIRE(N > 0 && K > 0 && K % 32 == 0, "fragment_order: N=%d, K=%d: K must be a multiple of 32", N, K);
+    FSIE_REQUIRE(reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 && w != out,
+                 "fragment_order: both matrices must be 16-byte aligned, and two");
+    const int64_t units = fsie_fragment_order_size(N, K) / 8;
+    FSIE_REQUIRE((units + 255) / 256 <= 0x7fffffff, "fragment_order: N=%d, K=%d is too large", N, K);
+    fragment_order_kernel<<<static_cast<unsigned>((units + 255) / 256), 256, 0, stream>>>(
+        static_cast<const u32x4*>(w), static_cast<u32x4*>(out), N, K, units);
+    FSIE_CHECK_LAUNCH("fragment_order");
+    return 0;
 }

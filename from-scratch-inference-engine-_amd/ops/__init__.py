@@ -5,9 +5,9 @@ kernel and its grid assume, then queues the kernel on torch's current stream.  N
 computes with torch; a missing kernel library is an error, not a reason to fall back.
 """
 
-from .functions import (attention_merge, attention_mfma, attention_mfma_lds, attention_mfma_lds_ok,
+from .functions import (FragmentOrdered, attention_merge, attention_mfma, attention_mfma_lds, attention_mfma_lds_ok,
                         attention_mfma_max_waves, attention_mfma_rows, attention_scalar,
-                        attention_tile_tokens, bias_add, compute_units, dtype_code, embedding, gemm, gemm_mfma_fp32, gemm_mfma_skinny,
+                        attention_tile_tokens, bias_add, compute_units, dtype_code, embedding, fragment_order, gemm, gemm_mfma_fp32, gemm_mfma_skinny,
                         gemm_mfma_skinny_rope, gemm_mfma_wide, gemm_mfma_wide_best_splits, gemm_mfma_wide_splits_ok,
                         gemm_mfma_wide_swiglu, random_fill,
                         residual_add,
@@ -15,9 +15,9 @@ from .functions import (attention_merge, attention_mfma, attention_mfma_lds, att
 from .library import KernelError, KernelLibraryMissing, load
 from .tuning import disable_library_tuning, enable_library_tuning, library_mm, library_tuning_enabled
 
-__all__ = ["KernelError", "KernelLibraryMissing", "attention_merge", "attention_mfma", "attention_mfma_lds",
+__all__ = ["FragmentOrdered", "KernelError", "KernelLibraryMissing", "attention_merge", "attention_mfma", "attention_mfma_lds",
            "attention_mfma_lds_ok", "attention_mfma_max_waves", "attention_mfma_rows", "attention_scalar",
            "attention_tile_tokens", "bias_add", "compute_units", "disable_library_tuning", "dtype_code", "embedding",
-           "enable_library_tuning", "gemm", "gemm_mfma_fp32", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "gemm_mfma_wide",
+           "enable_library_tuning", "fragment_order", "gemm", "gemm_mfma_fp32", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "gemm_mfma_wide",
            "gemm_mfma_wide_best_splits", "gemm_mfma_wide_splits_ok", "gemm_mfma_wide_swiglu", "library_mm", "library_tuning_enabled", "load", "random_fill", "residual_add",
            "rmsnorm", "rmsnorm_plain", "rope_kv_write", "rope_table", "sample", "swiglu", "zero_pages", "zero_rows"]

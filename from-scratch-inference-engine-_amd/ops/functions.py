@@ -305,6 +305,49 @@ def gemm_mfma_skinny(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     return out
 
 
+class FragmentOrdered:
+    """The copy of a bfloat16 matrix [rows, cols] in the order of the matrix instruction's A
+    fragments (``fragment_order``): the 64 16-byte units of a block of 16 rows and 32 columns lie
+    together in the order of the lanes that hold them, so that a wave's load of the weight is one
+    piece of 1 KB and can be a streaming load.  ``gemm_mfma_wide`` and ``gemm_mfma_wide_swiglu``
+    take it in place of the matrix."""
+
+    __slots__ = ("data", "rows", "cols")
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int):
+        self.data, self.rows, self.cols = data, rows, cols
+
+    @property
+    def shape(self):
+        return (self.rows, self.cols)
+
+
+def fragment_order(weight: torch.Tensor) -> FragmentOrdered:
+    """The copy of ``weight`` [N, K] (bfloat16, K a multiple of 32) in fragment order; the rows that
+    fill N up to a multiple of 16 are zeros."""
+    _need(weight, "fragment_order weight", dtype=torch.bfloat16, ndim=2)
+    n, k = weight.shape
+    size = int(load().fsie_fragment_order_size(n, k))
+    if size <= 0:
+        raise KernelError(f"fragment_order: the inner size {k} must be a multiple of 32")
+    data = torch.empty(size, dtype=torch.bfloat16, device=weight.device)
+    check(load().fsie_fragment_order(weight.data_ptr(), data.data_ptr(), n, k, _stream()))
+    return FragmentOrdered(data, n, k)
+
+
+def _wide_weight(weight, k: int):
+    """(pointer, N, whether it is in fragment order) of a weight given to the wide products."""
+    if isinstance(weight, FragmentOrdered):
+        _need(weight.data, "gemm weight", dtype=torch.bfloat16, ndim=1)
+        n, kw, ptr, frags = weight.rows, weight.cols, weight.data.data_ptr(), 1
+    else:
+        _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
+        n, kw, ptr, frags = weight.shape[0], weight.shape[1], weight.data_ptr(), 0
+    if kw != k:
+        raise KernelError(f"gemm: weight inner size {kw} does not match x's {k}")
+    return ptr, n, frags
+
+
 def gemm_mfma_wide_splits_ok(k: int, splits: int) -> bool:
     """Whether ``gemm_mfma_wide`` can cut an inner size ``k`` into ``splits`` slices (whole stages
     of 128 values each)."""
@@ -314,19 +357,17 @@ def gemm_mfma_wide_splits_ok(k: int, splits: int) -> bool:
 def gemm_mfma_wide_swiglu(x: torch.Tensor, weight: torch.Tensor, waves: int = 0, blocks: int = 0,
                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(gate) * up [M, N/2] (bfloat16) of x [M, K] and a weight [N, K] whose rows are gate and up
-    in turn, by the kernel that shares x through LDS; up to 64 rows, N a multiple of 4, K of 128."""
+    in turn (or its ``FragmentOrdered`` copy), by the kernel that shares x through LDS; up to 64
+    rows, N a multiple of 4, K of 128."""
     _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
-    _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
     m, k = x.shape
-    n = weight.shape[0]
-    if weight.shape[1] != k:
-        raise KernelError(f"gemm: weight inner size {weight.shape[1]} does not match x's {k}")
+    wptr, n, frags = _wide_weight(weight, k)
     if n % 4:
         raise KernelError(f"gemm_mfma_wide_swiglu: the number of weight rows {n} must be a multiple of 4")
     if out is None:
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     _need(out, "gemm out", dtype=torch.bfloat16, shape=(m, n // 2))
-    check(load().fsie_gemm_mfma_wide_swiglu(x.data_ptr(), weight.data_ptr(), out.data_ptr(), m, n, k, waves, blocks,
+    check(load().fsie_gemm_mfma_wide_swiglu(x.data_ptr(), wptr, out.data_ptr(), m, n, k, waves, blocks, frags,
                                             _stream()))
     return out
 
@@ -340,24 +381,22 @@ def gemm_mfma_wide_best_splits(m: int, n: int, k: int) -> int:
 def gemm_mfma_wide(x: torch.Tensor, weight: torch.Tensor, splits: int = 1, waves: int = 0,
                    out: Optional[torch.Tensor] = None, blocks: int = 0) -> torch.Tensor:
     """x [M, K] . weight [N, K]^T for bfloat16 operands and up to 64 rows, the rows of x shared by
-    a workgroup's waves through LDS (made for 17 rows and more).  The result is float32: [M, N],
+    a workgroup's waves through LDS (made for 17 rows and more); ``weight`` may be the matrix's
+    ``FragmentOrdered`` copy.  The result is float32: [M, N],
     or with ``splits`` of 2 to 16 the partial sums [splits, M, N] of the slices of K, for
     ``rmsnorm`` to add up.  K must be a multiple of 128 that the slices cover in whole stages
     (``gemm_mfma_wide_splits_ok``)."""
     _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
-    _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
     m, k = x.shape
-    n = weight.shape[0]
-    if weight.shape[1] != k:
-        raise KernelError(f"gemm: weight inner size {weight.shape[1]} does not match x's {k}")
+    wptr, n, frags = _wide_weight(weight, k)
     if not 1 <= splits <= GEMM_MAX_SPLITS:
         raise KernelError(f"gemm_mfma_wide: splits must be 1 to {GEMM_MAX_SPLITS}, got {splits}")
     shape = (m, n) if splits == 1 else (splits, m, n)
     if out is None:
         out = torch.empty(shape, dtype=torch.float32, device=x.device)
     _need(out, "gemm out", dtype=torch.float32, shape=shape)
-    check(load().fsie_gemm_mfma_wide(x.data_ptr(), weight.data_ptr(), out.data_ptr(), m, n, k, splits, waves,
-                                     blocks, _stream()))
+    check(load().fsie_gemm_mfma_wide(x.data_ptr(), wptr, out.data_ptr(), m, n, k, splits, waves, blocks, frags,
+                                     _stream()))
     return out
 
 

@@ -255,6 +255,7 @@ class GQAttention(Mixer):
 
     def prepare(self, device, compute_dtype) -> None:
         self.position.prepare(device, compute_dtype)
+        self.o.prepare()
 
     # cache and plan ---------------------------------------------------------------------
     def cache_need(self) -> PagedNeed:

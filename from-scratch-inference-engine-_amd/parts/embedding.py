@@ -49,5 +49,8 @@ class LMHead(Part):
     def weight(self, t):
         self.linear.weight = t
 
+    def prepare(self, device, compute_dtype) -> None:
+        self.linear.prepare()
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.linear(x, out_dtype=torch.float32)

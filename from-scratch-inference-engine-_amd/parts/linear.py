@@ -24,14 +24,45 @@ class Linear:
     accumulation, the bias added by a kernel of the engine."""
 
     float32_on_matrix_cores = True  # up to 64 rows of float32: v_mfma_f32_16x16x4_f32 instead of vector FMAs
+    # A bfloat16 weight of at least this many bytes is kept a second time, in the order of the matrix
+    # instruction's fragments, for the products of up to 64 rows (decoding): a wave then loads 1 KB in
+    # one piece with streaming loads, where rows give it 16 pieces of 64 bytes (MI355X, 8 rows: N = 37888,
+    # K = 3584, 272 MB, 43.7 against 49.3 us; N = 3584, K = 18944, 136 MB, 23.2 against 27.2; N = 152064,
+    # K = 3584 179 against 194; N = K = 3584, 26 MB, 7.0 against 6.6, so small ones are not copied).  The
+    # rows stay for the library's products of many rows (prefill).  The device has 288 GB: twice the
+    # large matrices of a 32B model are 120.  None: no copies.
+    streamed_copy_from = 64 << 20
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False):
         self.in_features = in_features
         self.out_features = out_features
         self.has_bias = bias
-        self.weight: Optional[torch.Tensor] = None
+        self._weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
+        self.streamed = None  # the weight in fragment order (ops.FragmentOrdered), if prepare() made one
         self._wide_splits: dict = {}
+
+    @property
+    def weight(self) -> Optional[torch.Tensor]:
+        return self._weight
+
+    @weight.setter
+    def weight(self, t: Optional[torch.Tensor]) -> None:
+        self._weight = t
+        self.streamed = None  # a copy of the weight that was here says nothing about this one
+
+    def prepare(self) -> None:
+        """Called by the owning part once the weight is set."""
+        w = self.weight
+        self.streamed = None
+        if (self.streamed_copy_from is not None and w is not None and w.dtype == torch.bfloat16 and w.is_cuda
+                and w.numel() * 2 >= self.streamed_copy_from and ops.gemm_mfma_wide_splits_ok(self.in_features, 1)):
+            self.streamed = ops.fragment_order(w)
+
+    @property
+    def wide_weight(self):
+        """What the products that share x through LDS read: the fragment-ordered copy if there is one."""
+        return self.weight if self.streamed is None else self.streamed
 
     def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                  skip_bias: bool = False) -> torch.Tensor:
@@ -46,11 +77,12 @@ class Linear:
                 return ops.gemm_mfma_fp32(x, w, bias)
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
         wants_f32 = out_dtype is not None and out_dtype != x.dtype
-        if (wants_f32 and bias is None and 8 <= m <= GEMM_MFMA_SKINNY_MAX_M
+        if (wants_f32 and bias is None and (8 if self.streamed is None else 2) <= m <= GEMM_MFMA_SKINNY_MAX_M
                 and ops.gemm_mfma_wide_splits_ok(self.in_features, 1)):
             # logits of 8 to 64 rows: x shared through LDS (N = 152064, K = 3584 on MI355X: 200
-            # against 215 us at 8 rows, 242 against 486 at 64)
-            return ops.gemm_mfma_wide(x, w)
+            # against 215 us at 8 rows, 242 against 486 at 64); from the fragment-ordered copy from
+            # two rows on (174 against 179 us; one row 182 against 176)
+            return ops.gemm_mfma_wide(x, self.wide_weight)
         if (wants_f32 and bias is None and m > GEMM_MFMA_SKINNY_MAX_M and out_dtype == torch.float32
                 and self.in_features % 8 == 0 and self.out_features % 8 == 0):
             # logits of more rows than the engine's kernels take (a decode batch beyond 64, a replay
@@ -81,8 +113,8 @@ class Linear:
             # K is long enough for six slices or more (N = 3584, K = 18944 in 8: 26 against 28 us at 8
             # rows, 27 against 32 at 16; N = K = 3584 in 7: 7.4 against 8.4 at 8 rows)
             splits = self.wide_splits(m)
-            if splits > 1 and (m > GEMM_MFMA_SKINNY_BEST_M or splits >= 6):
-                return ops.gemm_mfma_wide(x, self.weight, splits=splits)
+            if splits > 1 and (m > GEMM_MFMA_SKINNY_BEST_M or splits >= 6 or self.streamed is not None):
+                return ops.gemm_mfma_wide(x, self.wide_weight, splits=splits)
             splits = self.residual_splits(m)
             if splits > 1:
                 return ops.gemm_mfma_skinny(x, self.weight, splits=splits)

@@ -47,9 +47,22 @@ class SwiGLU(FeedForward):
     def down_weight(self, t):
         self.down.weight = t
 
+    def prepare(self, device, compute_dtype) -> None:
+        self.gate_up.prepare()
+        self.down.prepare()
+
+    # rows up to which silu(gate) * up comes from the product that shares x through LDS when the weight
+    # has a fragment-ordered copy (beyond: the library's product and a kernel for SiLU*up)
+    streamed_swiglu_max_rows = 64
+
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         m = x.shape[0]
-        if (x.dtype == torch.bfloat16 and 3 <= m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 128 == 0
+        if (x.dtype == torch.bfloat16 and self.gate_up.streamed is not None and 0 < m <= self.streamed_swiglu_max_rows
+                and self.gate_up.out_features % 4 == 0):
+            # from the fragment-ordered copy at any number of rows up to 64 (MI355X, N = 37888, K = 3584:
+            # 44 us for 1 to 16 rows, where the few-rows kernel takes 49 to 55 on rows)
+            act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.streamed)
+        elif (x.dtype == torch.bfloat16 and 3 <= m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 128 == 0
                 and self.gate_up.out_features % 4 == 0 and self.gate_up.out_features // 64 >= ops.compute_units()):
             # three rows and more of a matrix that gives every compute unit a workgroup: the kernel that
             # shares x through LDS (MI355X, 8 rows: N = 37888, K = 3584 49.3 against 51.2 us; N = 27648,

@@ -446,6 +446,74 @@ def test_batches_of_17_to_64_rows_share_x_through_lds(tmp_path):
     assert 1 in used and len(used) > 1 and all(1 <= s <= 16 for s in used), calls  # logits whole, projections in slices
 
 
+def test_decoding_from_fragment_ordered_copies(tmp_path, monkeypatch):
+    """With the size from which a weight is kept a second time, in the order of the matrix
+    instruction's fragments, set to zero, the small wide model keeps copies of every matrix whose
+    inner size the kernel takes (output, gate/up, down, the head of 331 rows, which ends inside a
+    block of 16), and steps of up to 64 rows read them: 1, 3 and 20 requests decoding, eagerly and
+    through graphs, and a portion of 40 tokens beside 3 decoded ones, against the plain model.  A
+    weight that is set anew drops its copy."""
+    from from_scratch_inference_engine_amd import load_model, ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+    from from_scratch_inference_engine_amd.parts.linear import Linear
+
+    d = helpers.make_model_dir(tmp_path / "wide", WIDE, seed=11)
+    plain_model = load_model(d, dtype="bfloat16")
+    assert plain_model.spec.lm_head.linear.streamed is None  # 0.7 MB: far below the size that is copied
+    monkeypatch.setattr(Linear, "streamed_copy_from", 0)
+    model = load_model(d, dtype="bfloat16")
+    block = model.spec.layers[0]
+    copies = [model.spec.lm_head.linear, block.mixer.o, block.ffn.gate_up, block.ffn.down]
+    assert all(isinstance(c.streamed, ops.FragmentOrdered) and c.streamed.shape == tuple(c.weight.shape) for c in copies)
+    assert block.mixer.qkv.streamed is None  # its product has the position encoding in its epilogue and reads rows
+    seen = []
+    real, real_swiglu = ops.gemm_mfma_wide, ops.gemm_mfma_wide_swiglu
+
+    def counted(x, w, **kw):
+        seen.append(("plain", x.shape[0], isinstance(w, ops.FragmentOrdered)))
+        return real(x, w, **kw)
+
+    def counted_swiglu(x, w, **kw):
+        seen.append(("swiglu", x.shape[0], isinstance(w, ops.FragmentOrdered)))
+        return real_swiglu(x, w, **kw)
+
+    monkeypatch.setattr(ops, "gemm_mfma_wide", counted)
+    monkeypatch.setattr(ops, "gemm_mfma_wide_swiglu", counted_swiglu)
+    seqs = [helpers.token_ids(331, 9 + i, 400 + i) for i in range(20)]
+    long = helpers.token_ids(331, 60, 450)
+    ref = [plain.forward_dir(d, ids).numpy() for ids in seqs[:4]]
+    ref_long = plain.forward_dir(d, long).numpy()
+    for graphs in (False, True):
+        for live in (1, 3, 20):
+            runner = Runner(model, page_size=16, num_pages=64, max_requests=24, use_graphs=graphs)
+            caches = [runner.manager.open(i) for i in range(live)]
+            n_pre = [len(ids) - 5 for ids in seqs[:live]]  # four tokens decoded here, the fifth beside the portion
+            runner.step([StepEntry(c, ids[:n], []) for c, ids, n in zip(caches, seqs, n_pre)])
+            for t in range(4):
+                out = runner.step([StepEntry(c, [ids[n + t]], [0]) for c, ids, n in zip(caches, seqs, n_pre)]).float().cpu()
+                for i in range(min(live, 4)):
+                    helpers.assert_close_to_plain(out[i:i + 1].numpy(), ref[i][n_pre[i] + t:n_pre[i] + t + 1], "bfloat16",
+                                                  f"graphs={graphs} {live} live, request {i} token {t}")
+        for c in caches[3:]:
+            runner.manager.close(c)
+        lc = runner.manager.open("long")
+        runner.step([StepEntry(lc, long[:20], [])])
+        entries = [StepEntry(lc, long[20:], list(range(40)))]
+        entries += [StepEntry(c, [ids[n + 4]], [0]) for c, ids, n in zip(caches[:3], seqs, n_pre)]
+        out = runner.step(entries).float().cpu()
+        helpers.assert_close_to_plain(out[:40].numpy(), ref_long[20:], "bfloat16", f"graphs={graphs} portion of 40")
+        for i in range(3):
+            helpers.assert_close_to_plain(out[40 + i:41 + i].numpy(), ref[i][n_pre[i] + 4:n_pre[i] + 5], "bfloat16",
+                                          f"graphs={graphs} request {i} beside the portion")
+    assert seen and all(frag for _, _, frag in seen), seen
+    assert {m for kind, m, _ in seen if kind == "swiglu"} >= {1, 3, 20, 43}
+    assert {m for kind, m, _ in seen if kind == "plain"} >= {1, 3, 20, 43}
+    lin = model.spec.lm_head.linear
+    lin.weight = lin.weight.clone()
+    assert lin.streamed is None
+
+
 def test_prefill_with_the_library_kernel_selection(model_dirs):
     """With tuning on, a prompt portion of a multiple of 256 rows, and a decode batch of a multiple
     of 16, let torch time the library's candidates for their products; whatever it picks, the

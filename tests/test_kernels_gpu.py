@@ -449,6 +449,49 @@ def test_gemm_mfma_wide_with_swiglu_epilogue(ops, m, n, k):
         ops.gemm_mfma_wide_swiglu(x.cuda(), w[:n - 2].contiguous().cuda())
 
 
+@pytest.mark.parametrize("n,k", [(331, 1024), (3072, 1024), (1000, 1536), (48, 128), (17, 256), (18944 * 2, 3584)])
+def test_products_on_fragment_ordered_weights(ops, n, k):
+    """The copy of a weight in the order of the matrix instruction's fragments: the layout itself
+    (against the same permutation written with tensor views), and the products on it, which add the
+    same numbers in the same order as on rows and so give the same bits: every number of 16-row tiles,
+    an N that ends inside a block of 16 rows (the copy's last block is filled up with zeros), slices
+    of K, both epilogues, every launch shape."""
+    from from_scratch_inference_engine_amd.ops import KernelError
+
+    w = rnd((n, k), 31, torch.bfloat16, 0.05).cuda()
+    f = ops.fragment_order(w)
+    assert f.shape == (n, k) and f.data.numel() == -(-n // 16) * 16 * k
+    n16 = -(-n // 16) * 16
+    padded = torch.zeros(n16, k, dtype=torch.bfloat16, device="cuda")
+    padded[:n] = w
+    # [block, row, step, k group, 8] -> [block, step, k group, row, 8]: lane = 16 * k group + row
+    want = padded.view(n16 // 16, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).reshape(-1)
+    assert torch.equal(f.data, want)
+    big = n * k > 1 << 24
+    for m in ((8, 64) if big else (1, 2, 5, 16, 17, 33, 48, 64)):
+        x = rnd((m, k), 32 + m, torch.bfloat16).cuda()
+        shapes = ((0, 0),) if big else ((0, 0), (2, 1), (2, 2), (4, 1), (4, 2), (8, 1), (8, 2))
+        for splits in (1, 2, 3, 8, 16):
+            if not ops.gemm_mfma_wide_splits_ok(k, splits):
+                continue
+            for waves, blocks in shapes:
+                a = ops.gemm_mfma_wide(x, w, splits=splits, waves=waves, blocks=blocks)
+                b = ops.gemm_mfma_wide(x, f, splits=splits, waves=waves, blocks=blocks)
+                assert torch.equal(a, b), (m, splits, waves, blocks)
+        if n % 4 == 0:
+            for waves, blocks in shapes:
+                a = ops.gemm_mfma_wide_swiglu(x, w, waves=waves, blocks=blocks)
+                b = ops.gemm_mfma_wide_swiglu(x, f, waves=waves, blocks=blocks)
+                assert torch.equal(a, b), (m, waves, blocks)
+    if not big:
+        full = (x.double() @ w.double().t()).float()  # the last x: 64 rows
+        assert (ops.gemm_mfma_wide(x, f) - full).abs().max() <= tol(torch.float32, full.cpu()) * 4
+    with pytest.raises(KernelError, match="multiple of 32"):
+        ops.fragment_order(w[:, :k - 16].contiguous())
+    with pytest.raises(KernelError, match="inner size"):
+        ops.gemm_mfma_wide(x[:, :k // 2].contiguous(), f)
+
+
 def test_refusals(ops):
     from from_scratch_inference_engine_amd.ops import KernelError
 
