@@ -242,6 +242,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-kernels", action="store_true", help="skip the time of each class of kernels of a decode step")
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
+    ap.add_argument("--no-streamed-copies", action="store_true",
+                    help="do not keep the large weights a second time in the order of the matrix instruction's fragments")
     ap.add_argument("--workload", choices=["decode", "mixed", "long-prefill"], default="decode",
                     help="decode: the default run.  mixed: --requests prompts of --min-prompt to --max-prompt tokens, "
                          "--outputs tokens each, through the scheduler (made for --shape 14b).  "
@@ -267,6 +269,10 @@ def main() -> int:
 
     if not args.no_tune and args.dtype == "bf16":
         enable_library_tuning()  # the first prefill times the library's kernels for its shapes
+    if args.no_streamed_copies:
+        from from_scratch_inference_engine_amd.parts.linear import Linear
+
+        Linear.streamed_copy_from = None
 
     shape_name, shape = SHAPES[args.shape]
     raw = dict(shape)
@@ -369,6 +375,7 @@ def main() -> int:
             "global_batch": args.batch, "seq_len": context, "prompt_len": args.prompt_len,
             "mean_decode_context": mean_ctx, "kv_block": page, "parallelism": "single GPU",
             "library_gemm_tuning": bool(not args.no_tune and args.dtype == "bf16"),
+            "streamed_weight_copies": bool(not args.no_streamed_copies and args.dtype == "bf16"),
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",

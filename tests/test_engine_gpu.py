@@ -236,6 +236,7 @@ def test_bench_prints_its_line():
     assert rec["value"] > 0 and abs(rec["value"] - 8 / (rec["ms_per_step"] * 1e-3)) <= 1e-6 * rec["value"]
     assert len(rec["config"]) <= 20 and all(not isinstance(v, (dict, list)) for v in rec["config"].values())
     assert rec["config"]["layers"] == 2 and rec["config"]["layers_of_config"] == 24
+    assert rec["config"]["streamed_weight_copies"] is True and rec["config"]["library_gemm_tuning"] is True
     assert rec["prefill"]["tokens"] == 2048 and 0 < rec["prefill"]["frac"] < 1
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0 and 0 < rec["roofline"]["frac"] < 1
     assert set(rec["points"]) == {"decode_b1", "decode_b64"}
