@@ -61,10 +61,12 @@ int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int32_t* slots
                        const float* bias, void* k_pool, void* v_pool, int n_tokens, int n_heads, int n_kv, int head_dim,
                        int rotary_dim, int page_size, int64_t pool_slots, int dtype, hipStream_t stream);
 
-// the same with the whole head rotated by the cosines and sines of fsie_rope_table (head_dim % 8 == 0)
+// the same with the whole head rotated by the cosines and sines of fsie_rope_table (head_dim % 8 == 0);
+// parts (or null): the projection as n_parts float32 partial sums [n_parts][n_tokens][width], added in
+// order; qkv then only receives the q heads
 int fsie_rope_kv_write_table(void* qkv, const float* cos_sin, const int32_t* slots, const float* bias, void* k_pool,
                              void* v_pool, int n_tokens, int n_heads, int n_kv, int head_dim, int page_size,
-                             int64_t pool_slots, int dtype, hipStream_t stream);
+                             int64_t pool_slots, int dtype, const float* parts, int n_parts, hipStream_t stream);
 
 // table [n_tokens, half, 2] float32: cos and sin of positions[t] * inv_freq[i]
 int fsie_rope_table(const int32_t* positions, const double* inv_freq, int n_tokens, int half, float* table,

@@ -139,11 +139,15 @@ struct Quad<bf16_t> {
 // the tokens of one 32-byte run would come from blocks on different dies, each of which would hand
 // its bytes of the run to memory separately.  Eight tokens whose slots are consecutive and start at
 // a multiple of 8 (a portion of a prompt) write 16 bytes per dimension at once.
-template <typename T, bool HAS_BIAS, int TOK>
+// PARTS: the projection comes as float32 partial sums parts[n_parts][n_tokens][width] of a product
+// whose inner dimension was cut into slices; they are added in the order of the slices, and qkv
+// only receives the q heads (TOK == 1).
+template <typename T, bool HAS_BIAS, int TOK, bool PARTS = false>
 __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
     T* __restrict__ qkv, const float* __restrict__ cos_sin, const int32_t* __restrict__ slots,
     const float* __restrict__ bias, T* __restrict__ k_pool, T* __restrict__ v_pool, int n_tokens, int n_heads,
-    int n_kv, int head_dim, int page_size, int write_kv, int64_t pool_slots) {
+    int n_kv, int head_dim, int page_size, int write_kv, int64_t pool_slots, const float* __restrict__ parts = nullptr,
+    int n_parts = 0) {
     const int t0 = blockIdx.x * TOK;
     const int n_here = min(TOK, n_tokens - t0);
     const int half = head_dim / 2;
@@ -156,9 +160,29 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
         slot[j] = (write_kv && j < n_here) ? slots[t0 + j] : -1;
         if (slot[j] >= pool_slots) slot[j] = -1;
     }
+    // the blocks of a token (gridDim.y of them; more than one only where the partial sums make a token
+    // heavy) share its columns
+    const int first = threadIdx.x + blockIdx.y * kThreads;
+    const int stride = kThreads * gridDim.y;
+    // four consecutive columns of token t
+    auto load4 = [&](int t, int col) -> float4 {
+        if constexpr (PARTS) {
+            const float* p = parts + static_cast<int64_t>(t) * width + col;
+            const int64_t step = static_cast<int64_t>(n_tokens) * width;
+            float4 acc = *reinterpret_cast<const float4*>(p);
+#pragma unroll 4
+            for (int s = 1; s < n_parts; ++s) {
+                const float4 v = *reinterpret_cast<const float4*>(p + s * step);
+                acc = float4{acc.x + v.x, acc.y + v.y, acc.z + v.z, acc.w + v.w};
+            }
+            return acc;
+        } else {
+            return Quad<T>::load(qkv + static_cast<int64_t>(t) * width + col);
+        }
+    };
 
     // ---- values
-    bool run = TOK == 8 && n_here == 8 && slot[0] >= 0 && slot[0] % 8 == 0 && page_size % 8 == 0;
+    bool run = !PARTS && TOK == 8 && n_here == 8 && slot[0] >= 0 && slot[0] % 8 == 0 && page_size % 8 == 0;
 #pragma unroll
     for (int j = 1; j < TOK; ++j) run = run && slot[j] == slot[0] + j;
     if (TOK == 8 && run) {
@@ -182,11 +206,10 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
             if (slot[j] < 0) continue;
             const int64_t page = slot[j] / page_size;
             const int off = slot[j] % page_size;
-            const T* v = qkv + static_cast<int64_t>(t0 + j) * width + q_dim + kv_dim;
-            for (int idx = threadIdx.x * 4; idx < kv_dim; idx += kThreads * 4) {
+            for (int idx = first * 4; idx < kv_dim; idx += stride * 4) {
                 const int kvh = idx / head_dim;
                 const int d = idx - kvh * head_dim;
-                float4 x = Quad<T>::load(v + idx);
+                float4 x = load4(t0 + j, q_dim + kv_dim + idx);
                 if (HAS_BIAS) {
                     const float4 b = *reinterpret_cast<const float4*>(bias + q_dim + kv_dim + idx);
                     x = float4{x.x + b.x, x.y + b.y, x.z + b.z, x.w + b.w};
@@ -203,7 +226,7 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
     // ---- q and k heads: unit u of a token = four pairs of one head; the tokens of the block in turn
     const int quads = half / 4;
     const int n_units = (n_heads + n_kv) * quads;
-    for (int u = threadIdx.x; u < n_units; u += kThreads) {
+    for (int u = first; u < n_units; u += stride) {
         const int h = u / quads;
         const int i = (u - h * quads) * 4;
         float4 b1{0.f, 0.f, 0.f, 0.f}, b2{0.f, 0.f, 0.f, 0.f};
@@ -216,7 +239,7 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
             if (j >= n_here) break;
             const int t = t0 + j;
             T* head = qkv + static_cast<int64_t>(t) * width + h * head_dim;
-            float4 a1 = Quad<T>::load(head + i), a2 = Quad<T>::load(head + i + half);
+            float4 a1 = load4(t, h * head_dim + i), a2 = load4(t, h * head_dim + i + half);
             a1 = float4{a1.x + b1.x, a1.y + b1.y, a1.z + b1.z, a1.w + b1.w};
             a2 = float4{a2.x + b2.x, a2.y + b2.y, a2.z + b2.z, a2.w + b2.w};
             const float4* cs = reinterpret_cast<const float4*>(cos_sin + static_cast<int64_t>(t) * head_dim);
@@ -225,8 +248,10 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
                             a1.w * c23.z - a2.w * c23.w};
             const float4 r2{a2.x * c01.x + a1.x * c01.y, a2.y * c01.z + a1.y * c01.w, a2.z * c23.x + a1.z * c23.y,
                             a2.w * c23.z + a1.w * c23.w};
-            Quad<T>::store(head + i, r1);
-            Quad<T>::store(head + i + half, r2);
+            if (!PARTS || h < n_heads) {
+                Quad<T>::store(head + i, r1);
+                Quad<T>::store(head + i + half, r2);
+            }
             if (h >= n_heads && slot[j] >= 0) {
                 const int64_t page = slot[j] / page_size;
                 const int off = slot[j] % page_size;
@@ -295,9 +320,14 @@ extern "C" int fsie_rope_kv_write(void* qkv, const int32_t* positions, const int
 
 // The rotation with cosines and sines from `cos_sin` ([n_tokens, head_dim / 2, 2] float32, made by
 // fsie_rope_table): the whole head is rotated, head_dim a multiple of 8.
+// parts (or null): float32 [n_parts][n_tokens][width], the projection as partial sums of a product cut
+// along its inner dimension; qkv then only receives the rotated q heads (k and v go to the pools).
 extern "C" int fsie_rope_kv_write_table(void* qkv, const float* cos_sin, const int32_t* slots, const float* bias,
                                         void* k_pool, void* v_pool, int n_tokens, int n_heads, int n_kv, int head_dim,
-                                        int page_size, int64_t pool_slots, int dtype, hipStream_t stream) {
+                                        int page_size, int64_t pool_slots, int dtype, const float* parts, int n_parts,
+                                        hipStream_t stream) {
+    FSIE_REQUIRE(!parts || (n_parts >= 1 && n_parts <= FSIE_GEMM_MAX_SPLITS && reinterpret_cast<uintptr_t>(parts) % 16 == 0),
+                 "rope_kv_write_table: 1 to %d aligned partial sums, got %d", FSIE_GEMM_MAX_SPLITS, n_parts);
     FSIE_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv > 0, "rope_kv_write_table: bad sizes");
     FSIE_REQUIRE(head_dim > 0 && head_dim % 8 == 0, "rope_kv_write_table: head_dim %d must be a multiple of 8", head_dim);
     FSIE_REQUIRE(cos_sin && reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0, "rope_kv_write_table: no aligned table");
@@ -309,6 +339,25 @@ extern "C" int fsie_rope_kv_write_table(void* qkv, const float* cos_sin, const i
     FSIE_REQUIRE(!write_kv || (page_size > 0 && pool_slots > 0), "rope_kv_write_table: bad page geometry");
     if (n_tokens == 0) return 0;
     // eight tokens a block where there are enough blocks left to fill the device
+    // blocks a token: so many that the device's units all have one (64 tokens of 4,608 columns in 7 partial
+    // sums on MI355X: 9.0 us with one block a token)
+    const int units = fsie_compute_units();
+    const int per_token = n_tokens > 0 && units > n_tokens ? (units / n_tokens > 8 ? 8 : units / n_tokens) : 1;
+    const dim3 parts_grid(static_cast<unsigned>(n_tokens), static_cast<unsigned>(per_token));
+#define FSIE_ROPE_PARTS(T, B)                                                                                     \
+    rope_kv_write_table_kernel<T, B, 1, true><<<parts_grid, kThreads, 0, stream>>>(                               \
+        static_cast<T*>(qkv), cos_sin, slots, bias, static_cast<T*>(k_pool), static_cast<T*>(v_pool), n_tokens,   \
+        n_heads, n_kv, head_dim, page_size, write_kv, pool_slots, parts, n_parts)
+    if (parts) {
+        if (dtype == FSIE_F32) {
+            if (bias) FSIE_ROPE_PARTS(float, true); else FSIE_ROPE_PARTS(float, false);
+        } else {
+            if (bias) FSIE_ROPE_PARTS(bf16_t, true); else FSIE_ROPE_PARTS(bf16_t, false);
+        }
+        FSIE_CHECK_LAUNCH("rope_kv_write_table");
+        return 0;
+    }
+#undef FSIE_ROPE_PARTS
 #define FSIE_ROPE_LAUNCH(T, B)                                                                                    \
     do {                                                                                                          \
         if (n_tokens >= 1024)                                                                                     \

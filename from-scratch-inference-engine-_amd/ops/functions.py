@@ -185,13 +185,16 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
                   inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor] = None,
                   k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None,
                   page_size: int = 0, bias: Optional[torch.Tensor] = None,
-                  cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  cos_sin: Optional[torch.Tensor] = None, parts: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rotate the q and k heads of ``qkv`` [T, (n_heads + 2 n_kv) head_dim] in place by the angles
     ``positions * inv_freq`` (float64 table of rotary_dim/2 entries; ``None`` = no rotation) and
     copy k and v to the cache slots ``slots`` (int32 [T], negative = not stored) of the pools: keys
     [pages, n_kv, page_size, head_dim], values [pages, n_kv, head_dim, page_size].  ``cos_sin``
     (``rope_table`` of these positions and frequencies): where the whole head is rotated and
-    head_dim is a multiple of 8, the kernel reads the angles' cosines and sines there."""
+    head_dim is a multiple of 8, the kernel reads the angles' cosines and sines there.
+    ``parts`` (float32 [S, T, width], only with ``cos_sin``): the projection as the partial sums of a
+    product cut along its inner dimension; they are added in order, ``qkv`` is then only written: its
+    q columns get the rotated q heads, k and v go to the pools alone."""
     _need(qkv, "qkv", ndim=2)
     t = qkv.shape[0]
     if qkv.shape[1] != (n_heads + 2 * n_kv) * head_dim:
@@ -213,11 +216,20 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
         if tuple(k_pool.shape[1:]) != (n_kv, page_size, head_dim):
             raise KernelError(f"k_pool: shape {tuple(k_pool.shape)} is not [pages, {n_kv}, {page_size}, {head_dim}]")
         pool_slots = k_pool.shape[0] * page_size
+    n_parts = 0
+    if parts is not None:
+        if cos_sin is None or rotary_dim != head_dim or head_dim % 8:
+            raise KernelError("rope_kv_write: partial sums need the table of cosines and sines and a whole head "
+                              "of a multiple of 8 dimensions rotated")
+        n_parts = parts.shape[0] if parts.dim() == 3 else 0
+        _need(parts, "qkv partial sums", dtype=torch.float32, shape=(n_parts, t, qkv.shape[1]))
+        if not 1 <= n_parts <= GEMM_MAX_SPLITS:
+            raise KernelError(f"rope_kv_write: {n_parts} partial sums; 1 to {GEMM_MAX_SPLITS} are taken")
     if cos_sin is not None and rotary_dim == head_dim and head_dim % 8 == 0:
         _need(cos_sin, "cos_sin", dtype=torch.float32, shape=(t, head_dim // 2, 2))
         check(load().fsie_rope_kv_write_table(qkv.data_ptr(), cos_sin.data_ptr(), _ptr(slots), _ptr(bias),
                                               _ptr(k_pool), _ptr(v_pool), t, n_heads, n_kv, head_dim, page_size,
-                                              pool_slots, dtype_code(qkv.dtype), _stream()))
+                                              pool_slots, dtype_code(qkv.dtype), _ptr(parts), n_parts, _stream()))
         return qkv
     check(load().fsie_rope_kv_write(qkv.data_ptr(), positions.data_ptr(), _ptr(slots), _ptr(inv_freq),
                                     _ptr(bias), _ptr(k_pool), _ptr(v_pool), t, n_heads, n_kv, head_dim, rotary_dim,

@@ -37,7 +37,7 @@ _SIGNATURES = {
     "fsie_bias_add": ([_P, _P, c_int, c_int, c_int, _P], c_int),
     "fsie_rope_kv_write": ([_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
                             c_int, _P], c_int),
-    "fsie_rope_kv_write_table": ([_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, _P],
+    "fsie_rope_kv_write_table": ([_P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int64, c_int, _P, c_int, _P],
                                  c_int),
     "fsie_gemm": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_gemm_mfma_fp32": ([_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P], c_int),

@@ -256,6 +256,7 @@ class GQAttention(Mixer):
     def prepare(self, device, compute_dtype) -> None:
         self.position.prepare(device, compute_dtype)
         self.o.prepare()
+        self.qkv.prepare()  # (read by the product of 17 to 64 rows; the few-rows product with the rotation reads rows)
 
     # cache and plan ---------------------------------------------------------------------
     def cache_need(self) -> PagedNeed:
@@ -271,6 +272,12 @@ class GQAttention(Mixer):
         store = KVStore(cache.k_pool, cache.v_pool, cache.slots, cache.page_size) if cache.writes else None
         qkv = self.position.project(x, self.qkv.weight, self.qkv.bias, self.n_heads, self.n_kv, self.head_dim, ctx,
                                     store)
+        if qkv is None:
+            # 17 to 64 rows: the engine's product in slices of K, added up by the kernel that rotates
+            sums = self.qkv.partial_sums(x)
+            if sums is not None:
+                qkv = self.position.apply_sums(sums, self.n_heads, self.n_kv, self.head_dim, ctx, store,
+                                               bias=self.qkv.bias)
         if qkv is None:
             qkv = self.qkv(x, skip_bias=True)
             self.position.apply(qkv, self.n_heads, self.n_kv, self.head_dim, ctx, store, bias=self.qkv.bias)

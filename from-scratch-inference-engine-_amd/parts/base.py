@@ -124,6 +124,14 @@ class PositionEncoding(Part):
         by itself and calls ``apply``."""
         return None
 
+    def apply_sums(self, parts: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, ctx, store,
+                   bias: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """Optional: ``apply`` on a projection that comes as float32 partial sums [S, T, width] of a
+        product cut along its inner dimension (added in order).  Returns [T, width] in the compute
+        dtype, of which the mixer reads only the q columns, or None if this encoding cannot: the
+        mixer then projects whole and calls ``apply``."""
+        return None
+
 
 class Block(Part):
     kind = "block"

@@ -61,6 +61,15 @@ class RotaryEncoding(PositionEncoding):
                               k_pool=store.k_pool, v_pool=store.v_pool, page_size=store.page_size, bias=bias,
                               cos_sin=cos_sin)
 
+    def apply_sums(self, parts, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore], bias=None):
+        if self.rotary_dim != head_dim or head_dim % 8:
+            return None
+        qkv = torch.empty(parts.shape[1:], dtype=ctx.compute_dtype, device=parts.device)
+        kw = {} if store is None else dict(slots=store.slots, k_pool=store.k_pool, v_pool=store.v_pool,
+                                           page_size=store.page_size)
+        return ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, bias=bias,
+                                 cos_sin=self.table(ctx), parts=parts, **kw)
+
     def project(self, x, weight, bias, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore]):
         """For a few rows of bfloat16 (decoding) the projection's own epilogue rotates and stores."""
         if (x.dtype != torch.bfloat16 or not 0 < x.shape[0] <= GEMM_MFMA_SKINNY_BEST_M or x.shape[1] % 8

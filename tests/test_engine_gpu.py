@@ -417,6 +417,13 @@ def test_batches_of_17_to_64_rows_share_x_through_lds(tmp_path):
         return real(x, w, splits=splits, **kw)
 
     ops.gemm_mfma_wide = counted
+    real_rope, summed = ops.rope_kv_write, []
+
+    def rope_counted(qkv, *a, parts=None, **kw):
+        summed.append((qkv.shape[0], parts is not None))
+        return real_rope(qkv, *a, parts=parts, **kw)
+
+    ops.rope_kv_write = rope_counted
     try:
         seqs = [helpers.token_ids(331, 9 + i, 900 + i) for i in range(20)]
         long = helpers.token_ids(331, 60, 950)
@@ -441,6 +448,9 @@ def test_batches_of_17_to_64_rows_share_x_through_lds(tmp_path):
             helpers.assert_close_to_plain(out.numpy(), ref_long[20:], "bfloat16", f"graphs={graphs} portion of 40")
     finally:
         ops.gemm_mfma_wide = real
+        ops.rope_kv_write = real_rope
+    # q/k/v of 17 to 64 rows come as partial sums that the rotation adds up; longer steps whole
+    assert {m for m, parts in summed if parts} >= {20, 40} and all(parts == (16 < m <= 64) for m, parts in summed), summed
     rows = {m for m, _ in calls}
     assert 20 in rows and 40 in rows, rows                      # decode batch and the portion
     used = {s for _, s in calls}
@@ -450,8 +460,9 @@ def test_batches_of_17_to_64_rows_share_x_through_lds(tmp_path):
 def test_decoding_from_fragment_ordered_copies(tmp_path, monkeypatch):
     """With the size from which a weight is kept a second time, in the order of the matrix
     instruction's fragments, set to zero, the small wide model keeps copies of every matrix whose
-    inner size the kernel takes (output, gate/up, down, the head of 331 rows, which ends inside a
-    block of 16), and steps of up to 64 rows read them: 1, 3 and 20 requests decoding, eagerly and
+    inner size the kernel takes (q/k/v, output, gate/up, down, the head of 331 rows, which ends inside
+    a block of 16), and steps of up to 64 rows read them (q/k/v from 17 rows on; with fewer its product
+    has the rotation in its epilogue and reads rows): 1, 3 and 20 requests decoding, eagerly and
     through graphs, and a portion of 40 tokens beside 3 decoded ones, against the plain model.  A
     weight that is set anew drops its copy."""
     from from_scratch_inference_engine_amd import load_model, ops
@@ -465,9 +476,8 @@ def test_decoding_from_fragment_ordered_copies(tmp_path, monkeypatch):
     monkeypatch.setattr(Linear, "streamed_copy_from", 0)
     model = load_model(d, dtype="bfloat16")
     block = model.spec.layers[0]
-    copies = [model.spec.lm_head.linear, block.mixer.o, block.ffn.gate_up, block.ffn.down]
+    copies = [model.spec.lm_head.linear, block.mixer.o, block.mixer.qkv, block.ffn.gate_up, block.ffn.down]
     assert all(isinstance(c.streamed, ops.FragmentOrdered) and c.streamed.shape == tuple(c.weight.shape) for c in copies)
-    assert block.mixer.qkv.streamed is None  # its product has the position encoding in its epilogue and reads rows
     seen = []
     real, real_swiglu = ops.gemm_mfma_wide, ops.gemm_mfma_wide_swiglu
 

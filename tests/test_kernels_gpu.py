@@ -111,6 +111,23 @@ def test_rope_and_cache_write(ops, dtype, from_table, heads, kv, hd, theta):
         assert (vp[s // page, :, :, s % page].reshape(-1) - v_ref[i]).abs().max() <= tol(dtype, v_ref, f32=2e-6)
     untouched = ~written.reshape(pages, 1, page, 1).expand_as(kp)
     assert kp[untouched].abs().max() == 0 and vp.transpose(2, 3)[untouched].abs().max() == 0
+    if from_table:
+        # the projection as three partial sums (what a product cut along its inner dimension leaves):
+        # the same q heads and pools; the k and v columns of the result are not written
+        g = torch.Generator().manual_seed(5)
+        p1, p2 = torch.randn(t, width, generator=g), torch.randn(t, width, generator=g)
+        parts = torch.stack([p1, p2, qkv.float() - p1 - p2]).cuda()
+        out = torch.full((t, width), 7.0, dtype=dtype).cuda()
+        dk2, dv2 = k_pool.cuda(), v_pool.cuda()
+        ops.rope_kv_write(out, pos.cuda(), heads, kv, hd, inv.cuda(), slots=slots.cuda(), k_pool=dk2, v_pool=dv2,
+                          page_size=page, bias=bias.cuda(), cos_sin=table, parts=parts)
+        out = out.float().cpu()
+        assert (out[:, :heads * hd] - q_ref).abs().max() <= tol(dtype, q_ref, f32=4e-6)
+        assert (out[:, heads * hd:] == 7.0).all()
+        assert (dk2.float().cpu() - kp).abs().max() <= tol(dtype, k_ref, f32=4e-6)
+        assert (dv2.float().cpu() - vp).abs().max() <= tol(dtype, v_ref, f32=4e-6)
+        with pytest.raises(Exception, match="partial sums"):
+            ops.rope_kv_write(out.to(dtype).cuda(), pos.cuda(), heads, kv, hd, inv.cuda(), parts=parts)
     # no rotation, no cache: only the bias on q and k
     dq = qkv.clone().cuda()
     ops.rope_kv_write(dq, pos.cuda(), heads, kv, hd, None, bias=bias.cuda())
