@@ -230,6 +230,12 @@ int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, 
 template <bool SWIGLU, bool FRAGS>
 int launch_shape_of(int mt, int waves, int blocks, const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K,
                     int splits, int k_slice, hipStream_t stream) {
+    if constexpr (SWIGLU && FRAGS) {  // gate/up of 17 rows and more: any number of waves that deals the rows evenly
+        if (blocks == 2 && waves == 3) return launch_mt<3, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+        if (blocks == 2 && waves == 5) return launch_mt<5, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+        if (blocks == 2 && waves == 6) return launch_mt<6, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+        if (blocks == 2 && waves == 7) return launch_mt<7, FSIE_WIDE_STEPS, 2, true, true>(mt, x, w, y, M, N, K, splits, k_slice, stream);
+    }
     if (blocks == 2) {
         if (waves == 8) return launch_mt<8, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
         if (waves == 2) return launch_mt<2, FSIE_WIDE_STEPS, 2, SWIGLU, FRAGS>(mt, x, w, y, M, N, K, splits, k_slice, stream);
@@ -258,22 +264,23 @@ __global__ __launch_bounds__(256) void fragment_order_kernel(const u32x4* __rest
 }
 
 // Waves a workgroup and row blocks a wave where the caller leaves them open (0).
-void launch_shape(int mt, int N, int splits, int& waves, int& blocks, bool gate_up = false) {
+void launch_shape(int mt, int N, int splits, int& waves, int& blocks, bool gate_up = false, bool frags = false) {
     if (gate_up && mt >= 2 && waves == 0 && blocks == 0) {
         // 17 rows and more, one slice: the products and the reads of x from LDS bound a workgroup, so
-        // a compute unit with two workgroups takes twice as long as one with one.  The largest
-        // workgroups (they lay x into LDS least often) that still occupy more than half of the units,
-        // one each (MI355X, 256 units, 64 rows, fragment-ordered W: N = 37888, K = 3584 in 148
-        // workgroups of 256 rows 52.5 us, in 296 of 128 rows 62.1; N = 27648, K = 5120 in 216 of 128
-        // rows 48.8, in 108 of 256 rows 69.3; N = 55296, K = 5120 in 216 of 256 rows 86.6, in 432 of
-        // 128 rows 96.1)
+        // a compute unit with two workgroups takes twice as long as one with one, and a unit draws
+        // only so much from memory, so every unit should have one.  Two blocks a wave, and the fewest
+        // waves a workgroup that still give at most one workgroup a unit (MI355X, 256 units, 64 rows,
+        // fragment-ordered W: N = 37888, K = 3584 in 237 workgroups of five waves 48.9 us, in 148 of eight
+        // 52.7, in 296 of four 62.3; N = 27648, K = 5120 in 216 of four waves 48.9, in 288 of three 70.8,
+        // in 173 of five 61.0; N = 55296, K = 5120 in 247 of seven 87.5, in 216 of eight 86.8, in 288 of six
+        // 129.9; N = 19456, K = 2048 in 203 of three 18.7, in 152 of four 20.6, in 304 of two 22.2).
+        // Five, six and seven waves exist only for fragment-ordered weights.
         const int units = fsie_compute_units();
-        static const int shapes[4][2] = {{8, 2}, {4, 2}, {2, 2}, {2, 1}};
-        for (const auto& shape : shapes) {
-            const int rows = 16 * shape[0] * shape[1];
-            waves = shape[0], blocks = shape[1];
-            if (static_cast<int64_t>((N + rows - 1) / rows) * 20 >= static_cast<int64_t>(units) * 11) break;
-        }
+        blocks = 2;
+        for (waves = 2; waves < 8; ++waves)
+            if ((N + 32 * waves - 1) / (32 * waves) <= units) break;
+        if (!frags && waves != 2 && waves != 4) waves = waves < 4 ? 4 : 8;
+        if (waves == 2 && (N + 31) / 32 * 2 <= units) blocks = 1;  // a small N: twice the workgroups of one block a wave
         return;
     }
     if (blocks == 0) {
@@ -399,11 +406,12 @@ extern "C" int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y,
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(y) % 4 == 0,
                  "gemm_mfma_wide_swiglu: operands must be 16-byte aligned, the result 4-byte");
-    FSIE_REQUIRE(waves == 0 || waves == 2 || waves == 4 || waves == 8, "gemm_mfma_wide_swiglu: waves must be 0, 2, 4 or 8");
+    FSIE_REQUIRE(waves == 0 || waves == 2 || waves == 4 || waves == 8 || (frags && blocks == 2 && waves >= 2 && waves <= 8),
+                 "gemm_mfma_wide_swiglu: waves must be 0, 2, 4 or 8 (2 to 8 with two blocks a wave on a fragment-ordered weight)");
     FSIE_REQUIRE(blocks == 0 || blocks == 1 || blocks == 2, "gemm_mfma_wide_swiglu: blocks must be 0, 1 or 2");
     if (M == 0) return 0;
     const int mt = (M + 15) / 16;
-    launch_shape(mt, N, 1, waves, blocks, true);
+    launch_shape(mt, N, 1, waves, blocks, true, frags != 0);
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
     float* yp = static_cast<float*>(y);

@@ -496,10 +496,12 @@ def test_products_on_fragment_ordered_weights(ops, n, k):
                 b = ops.gemm_mfma_wide(x, f, splits=splits, waves=waves, blocks=blocks)
                 assert torch.equal(a, b), (m, splits, waves, blocks)
         if n % 4 == 0:
-            for waves, blocks in shapes:
-                a = ops.gemm_mfma_wide_swiglu(x, w, waves=waves, blocks=blocks)
+            a = ops.gemm_mfma_wide_swiglu(x, w)
+            for waves, blocks in shapes + (() if big else ((3, 2), (5, 2), (6, 2), (7, 2))):  # odd numbers of waves: this copy only
                 b = ops.gemm_mfma_wide_swiglu(x, f, waves=waves, blocks=blocks)
                 assert torch.equal(a, b), (m, waves, blocks)
+            with pytest.raises(KernelError, match="waves must be"):
+                ops.gemm_mfma_wide_swiglu(x, w, waves=5, blocks=2)
     if not big:
         full = (x.double() @ w.double().t()).float()  # the last x: 64 rows
         assert (ops.gemm_mfma_wide(x, f) - full).abs().max() <= tol(torch.float32, full.cpu()) * 4
