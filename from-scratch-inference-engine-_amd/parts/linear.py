@@ -30,8 +30,11 @@ class Linear:
     # K = 3584, 272 MB, 43.7 against 49.3 us; N = 3584, K = 18944, 136 MB, 23.2 against 27.2; N = 152064,
     # K = 3584 179 against 194; N = K = 3584, 26 MB, 7.0 against 6.6, so small ones are not copied).  The
     # rows stay for the library's products of many rows (prefill).  The device has 288 GB: twice the
-    # large matrices of a 32B model are 120.  None: no copies.
+    # large matrices of a 32B model are 120.  None: no copies.  A copy is not made where it would leave
+    # less than ``streamed_copy_reserve`` of the device's memory free (for the cache and the steps'
+    # own tensors): a model that large keeps copies of its first layers only and runs the rest from rows.
     streamed_copy_from = 64 << 20
+    streamed_copy_reserve = 0.25
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False):
         self.in_features = in_features
@@ -57,7 +60,9 @@ class Linear:
         self.streamed = None
         if (self.streamed_copy_from is not None and w is not None and w.dtype == torch.bfloat16 and w.is_cuda
                 and w.numel() * 2 >= self.streamed_copy_from and ops.gemm_mfma_wide_splits_ok(self.in_features, 1)):
-            self.streamed = ops.fragment_order(w)
+            free, total = torch.cuda.mem_get_info(w.device)
+            if free - w.numel() * 2 >= self.streamed_copy_reserve * total:
+                self.streamed = ops.fragment_order(w)
 
     @property
     def wide_weight(self):

@@ -523,6 +523,11 @@ def test_decoding_from_fragment_ordered_copies(tmp_path, monkeypatch):
     lin = model.spec.lm_head.linear
     lin.weight = lin.weight.clone()
     assert lin.streamed is None
+    lin.prepare()
+    assert lin.streamed is not None
+    monkeypatch.setattr(Linear, "streamed_copy_reserve", 1.0)  # no copy may leave that much of the device free
+    lin.prepare()
+    assert lin.streamed is None
 
 
 def test_prefill_with_the_library_kernel_selection(model_dirs):
