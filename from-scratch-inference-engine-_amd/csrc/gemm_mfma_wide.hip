@@ -301,6 +301,10 @@ void launch_shape(int mt, int N, int splits, int& waves, int& blocks, bool gate_
         // slices 39.6 against 38.1); with two blocks a wave, four waves (N = 152064: 236 against 260)
         const int64_t groups4 = static_cast<int64_t>((N + 63) / 64) * splits;
         waves = (groups4 >= 1024 && blocks == 1) ? 8 : 4;
+        // one tile of X at a large N of a fragment-ordered W: nothing to share, and two waves a workgroup stream best (N = 152064,
+        // K = 3584, fragment-ordered: 8 rows 168 us with two waves, 171 with four, 179 with eight; one row
+        // 164 / 168 / 177; N = 152064, K = 5120, 8 rows: 247 / 249 / 259)
+        if (frags && mt == 1 && groups4 >= 1024 && blocks == 1) waves = 2;  // (on rows: 215 / 195 / 194)
         // two waves a workgroup where that deals the waves more evenly to the compute units (N =
         // 5120 in 8 slices: 640 workgroups of four waves put 12 waves on the fullest of 256 units,
         // 1280 of two put 10; K = 13824, 8 rows: 26.7 against 29.8 us)
@@ -386,7 +390,7 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
     FSIE_REQUIRE(blocks == 0 || blocks == 1 || blocks == 2, "gemm_mfma_wide: blocks must be 0, 1 or 2");
     if (M == 0) return 0;
     const int mt = (M + 15) / 16;
-    launch_shape(mt, N, splits, waves, blocks);
+    launch_shape(mt, N, splits, waves, blocks, false, frags != 0);
     const bf16_t* xp = static_cast<const bf16_t*>(x);
     const bf16_t* wq = static_cast<const bf16_t*>(w);
     if (frags) return launch_shape_of<false, true>(mt, waves, blocks, xp, wq, y, M, N, K, splits, k_slice, stream);

@@ -82,11 +82,11 @@ class Linear:
                 return ops.gemm_mfma_fp32(x, w, bias)
             return ops.gemm(x, w, bias, out_dtype=out_dtype)
         wants_f32 = out_dtype is not None and out_dtype != x.dtype
-        if (wants_f32 and bias is None and (8 if self.streamed is None else 2) <= m <= GEMM_MFMA_SKINNY_MAX_M
+        if (wants_f32 and bias is None and (8 if self.streamed is None else 1) <= m <= GEMM_MFMA_SKINNY_MAX_M
                 and ops.gemm_mfma_wide_splits_ok(self.in_features, 1)):
             # logits of 8 to 64 rows: x shared through LDS (N = 152064, K = 3584 on MI355X: 200
-            # against 215 us at 8 rows, 242 against 486 at 64); from the fragment-ordered copy from
-            # two rows on (174 against 179 us; one row 182 against 176)
+            # against 215 us at 8 rows, 242 against 486 at 64); from the fragment-ordered copy at any
+            # number of rows (one row 164 us, the few-rows kernel on rows 176 to 198)
             return ops.gemm_mfma_wide(x, self.wide_weight)
         if (wants_f32 and bias is None and m > GEMM_MFMA_SKINNY_MAX_M and out_dtype == torch.float32
                 and self.in_features % 8 == 0 and self.out_features % 8 == 0):
