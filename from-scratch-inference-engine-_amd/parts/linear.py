@@ -28,12 +28,13 @@ class Linear:
     # instruction's fragments, for the products of up to 64 rows (decoding): a wave then loads 1 KB in
     # one piece with streaming loads, where rows give it 16 pieces of 64 bytes (MI355X, 8 rows: N = 37888,
     # K = 3584, 272 MB, 43.7 against 49.3 us; N = 3584, K = 18944, 136 MB, 23.2 against 27.2; N = 152064,
-    # K = 3584 179 against 194; N = K = 3584, 26 MB, 7.0 against 6.6, so small ones are not copied).  The
+    # K = 3584 179 against 194; N = K = 5120, 52 MB, 10.3 against 12.7; N = K = 4096, 34 MB, 9.3 against 7.5,
+    # and N = K = 3584, 26 MB, 6.7 against 6.5, so small ones are not copied).  The
     # rows stay for the library's products of many rows (prefill).  The device has 288 GB: twice the
     # large matrices of a 32B model are 120.  None: no copies.  A copy is not made where it would leave
     # less than ``streamed_copy_reserve`` of the device's memory free (for the cache and the steps'
     # own tensors): a model that large keeps copies of its first layers only and runs the rest from rows.
-    streamed_copy_from = 64 << 20
+    streamed_copy_from = 48 << 20
     streamed_copy_reserve = 0.25
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False):
