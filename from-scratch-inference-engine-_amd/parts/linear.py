@@ -17,11 +17,14 @@ class Linear:
     float32: the engine's own kernels only (true 32-bit products and sums): vector FMA kernels,
     and for 3 to 64 rows (decoding) the matrix cores' float32 instruction, which rounds nothing.
     bfloat16: up to 16 rows (decoding) the engine's matrix-core kernel that streams the weight
-    once; its sibling that shares x through LDS for float32 results of 8 to 64 rows (the logits; beyond 64 rows the library with a float32 result)
-    and for the residual projections (``for_residual``: 17 to 64 rows, and any number where K is
-    long); everything else the library product
+    once; its sibling that shares x through LDS for float32 results of 8 to 64 rows (the logits;
+    beyond 64 rows the library with a float32 result), for the residual projections
+    (``for_residual``: 17 to 64 rows, and any number where K is long) and for the partial sums of
+    other projections of 17 to 64 rows (``partial_sums``); everything else the library product
     (hipBLASLt through torch, where the reference's engine calls cuBLAS) with float32
-    accumulation, the bias added by a kernel of the engine."""
+    accumulation, the bias added by a kernel of the engine.  A large weight has a second copy in
+    the order of the matrix instruction's fragments (``prepare``, ``streamed``), from which the
+    sibling takes every product of up to 64 rows."""
 
     float32_on_matrix_cores = True  # up to 64 rows of float32: v_mfma_f32_16x16x4_f32 instead of vector FMAs
     # A bfloat16 weight of at least this many bytes is kept a second time, in the order of the matrix
