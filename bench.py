@@ -269,10 +269,6 @@ def main() -> int:
 
     if not args.no_tune and args.dtype == "bf16":
         enable_library_tuning()  # the first prefill times the library's kernels for its shapes
-    if args.no_streamed_copies:
-        from from_scratch_inference_engine_amd.parts.linear import Linear
-
-        Linear.streamed_copy_from = None
 
     shape_name, shape = SHAPES[args.shape]
     raw = dict(shape)
@@ -283,7 +279,7 @@ def main() -> int:
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     itemsize = 2 if args.dtype == "bf16" else 4
     t0 = time.perf_counter()
-    model = Model.from_random(cfg, seed=0, dtype=dtype)
+    model = Model.from_random(cfg, seed=0, dtype=dtype, weight_copies=not args.no_streamed_copies)
     torch.cuda.synchronize()
     print(f"[bench] {layers}-layer model with random weights on the GPU: {model.weight_bytes / 1e9:.2f} GB "
           f"in {time.perf_counter() - t0:.1f} s", file=sys.stderr, flush=True)

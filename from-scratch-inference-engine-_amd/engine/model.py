@@ -100,17 +100,20 @@ class Model:
 
     # ---------------------------------------------------------------- construction
     @classmethod
-    def from_pretrained(cls, model_dir, dtype="bfloat16", device="cuda:0") -> "Model":
+    def from_pretrained(cls, model_dir, dtype="bfloat16", device="cuda:0", weight_copies: bool = True) -> "Model":
+        """``weight_copies=False``: no second, fragment-ordered copy of the large matrices (half
+        the memory; decode steps then read rows and are some 8 % slower)."""
         device = _require_gpu(device)
         config = parse_config(read_config_json(model_dir))
         model = cls(build_model_spec(config), dtype, device)
         model.weight_bytes = load_weights(Path(model_dir), model.spec.bindings, model.dtype, device,
                                           model.spec.ignore_unexpected)
-        model._prepare()
+        model._prepare(weight_copies)
         return model
 
     @classmethod
-    def from_random(cls, config: ModelConfig, seed: int = 0, dtype="bfloat16", device="cuda:0") -> "Model":
+    def from_random(cls, config: ModelConfig, seed: int = 0, dtype="bfloat16", device="cuda:0",
+                    weight_copies: bool = True) -> "Model":
         """Random weights without a folder, drawn on the device (gigabytes in a fraction of a
         second): the very values that ``write_random_model`` writes for this configuration and
         seed (the generator is a function of seed, tensor name and element index)."""
@@ -120,13 +123,21 @@ class Model:
         model.weight_bytes = fill_parts(
             model.spec.bindings, lambda name: random_tensor(specs[name], seed, torch.float32, device=device),
             model.dtype, device)
-        model._prepare()
+        model._prepare(weight_copies)
         return model
 
-    def _prepare(self) -> None:
+    def _prepare(self, weight_copies: bool = True) -> None:
         from ..parts.base import Norm
-        for part in self.spec.all_parts():
-            part.prepare(self.device, self.dtype)
+        from ..parts.linear import Linear
+
+        copy_from = Linear.streamed_copy_from
+        if not weight_copies:
+            Linear.streamed_copy_from = None  # while this model's parts are prepared
+        try:
+            for part in self.spec.all_parts():
+                part.prepare(self.device, self.dtype)
+        finally:
+            Linear.streamed_copy_from = copy_from
         self.partial_sums_ok = all(p.adds_partial_sums for p in self.spec.all_parts() if isinstance(p, Norm))
 
     # ---------------------------------------------------------------- cache

@@ -474,6 +474,10 @@ def test_decoding_from_fragment_ordered_copies(tmp_path, monkeypatch):
     plain_model = load_model(d, dtype="bfloat16")
     assert plain_model.spec.lm_head.linear.streamed is None  # 0.7 MB: far below the size that is copied
     monkeypatch.setattr(Linear, "streamed_copy_from", 0)
+    from from_scratch_inference_engine_amd.engine.model import Model
+    without = Model.from_pretrained(d, dtype="bfloat16", weight_copies=False)
+    assert without.spec.lm_head.linear.streamed is None and Linear.streamed_copy_from == 0
+    del without
     model = load_model(d, dtype="bfloat16")
     block = model.spec.layers[0]
     copies = [model.spec.lm_head.linear, block.mixer.o, block.mixer.qkv, block.ffn.gate_up, block.ffn.down]
