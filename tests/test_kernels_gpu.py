@@ -466,7 +466,8 @@ def test_gemm_mfma_wide_with_swiglu_epilogue(ops, m, n, k):
         ops.gemm_mfma_wide_swiglu(x.cuda(), w[:n - 2].contiguous().cuda())
 
 
-@pytest.mark.parametrize("n,k", [(331, 1024), (3072, 1024), (1000, 1536), (48, 128), (17, 256), (18944 * 2, 3584)])
+@pytest.mark.parametrize("n,k", [(331, 1024), (3072, 1024), (1000, 1536), (48, 128), (17, 256), (18944 * 2, 3584),
+                                 (3584, 18944), (5120, 13824), (152064, 3584)])
 def test_products_on_fragment_ordered_weights(ops, n, k):
     """The copy of a weight in the order of the matrix instruction's fragments: the layout itself
     (against the same permutation written with tensor views), and the products on it, which add the
