@@ -101,7 +101,16 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     const int total_pairs = N / 2;
     const int units = fsie_compute_units();
     int pairs_per_wg = 8;
-    if (mt == 1 && M > 4 && units > 0 && total_pairs > 8 * units && total_pairs <= 16 * units) {  // (no gain at 1 row)
+    // Up to 6 rows of x, a product large enough for it: two workgroups of four waves a unit, each with
+    // 4 to 8 pairs (two waves a SIMD hide each other's waits; MI355X, 256 units, N = 4608, K = 3584: 5
+    // pairs, 461 workgroups: 10.0 us at one row, 11.0 at four, where 8 pairs take 11.8 and 13.0 and 9
+    // pairs 11.6 and 11.7; N = 7168, K = 5120: 7 pairs, 512 workgroups: 15.8 and 16.8 against 17.1 and
+    // 18.6 for 8 pairs; at 8 rows 12.1 against 12.0 and 19.0 against 19.5, at 16 rows 15.6 against 12.9)
+    const int two_each = units > 0 ? (total_pairs + 2 * units - 1) / (2 * units) : 0;
+    const bool two_a_unit = mt == 1 && M <= 6 && units > 0 && total_pairs >= 8 * units && two_each <= 8;
+    if (two_a_unit) {
+        pairs_per_wg = two_each;
+    } else if (mt == 1 && M > 4 && units > 0 && total_pairs > 8 * units && total_pairs <= 16 * units) {
         pairs_per_wg = (total_pairs + units - 1) / units;
     }
     const int blocks = pairs_per_wg > 8 ? 2 : 1;
@@ -110,6 +119,7 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     // (more waves than this only add to the reduction: 12.6 us with four against 14.1 with eight
     // at N = 4608, K = 3584 and one row)
     while (waves < 16 && groups * waves < 1024) waves *= 2;
+    if (two_a_unit) waves = 4;
     while (waves > 1 && pairs < 2 * waves) waves /= 2;
     if (mt * blocks > 4 && waves > 8) waves = 8;  // LDS of the reduction
     const fsie_mm::Call call{x, w, bias, y, M, N, K, 1, stream,

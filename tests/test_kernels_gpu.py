@@ -388,7 +388,11 @@ def test_rmsnorm_adds_partial_sums_at_odd_sizes(ops):
     # on 256 compute units these deal 10 and 14 rotary pairs a workgroup; with a head size of 160 a block's pairs span two heads
     (8, 24, 4, 160, 256, 1e4, True), (16, 40, 8, 128, 128, 1e6, False),
     # the q/k/v projection of the 14B and 32B shapes (7,168 rows of 5,120)
-    (1, 40, 8, 128, 5120, 1e6, True), (8, 40, 8, 128, 5120, 1e6, True), (16, 40, 8, 128, 5120, 1e6, True)])
+    (1, 40, 8, 128, 5120, 1e6, True), (8, 40, 8, 128, 5120, 1e6, True), (16, 40, 8, 128, 5120, 1e6, True),
+    # up to 6 rows of a large projection: two workgroups a compute unit, 5 pairs each on 256 units (the last
+    # one has 4; with a head size of 160 a workgroup's pairs span two heads), 7 pairs at 7,168 rows
+    (1, 28, 4, 128, 3584, 1e6, True), (4, 28, 4, 128, 3584, 1e6, True), (6, 28, 4, 128, 3584, 1e6, False),
+    (3, 24, 4, 160, 256, 1e4, True), (5, 40, 8, 128, 5120, 1e6, True)])
 def test_projection_with_rotary_epilogue(ops, m, heads, kv, hd, k, theta, use_bias):
     """q/k/v projection, bias, rotation and cache write in one kernel, against the plain formulas
     on the float32 product (one rounding to bfloat16, after the rotation)."""
