@@ -11,6 +11,7 @@
 
 #define FSIE_GEMM_SKINNY_MAX_M 8
 #define FSIE_GEMM_MFMA_SKINNY_MAX_M 64
+#define FSIE_GEMM_MFMA_WIDE_MAX_M 112  // the product that shares x through LDS, on a fragment-ordered weight: seven tiles of 16 rows
 #define FSIE_GEMM_MFMA_SKINNY_BEST_M 16  // above this the library product is faster on MI355X
 #define FSIE_GEMM_MAX_SPLITS 16          // most slices of K a product may leave as partial sums
 
@@ -100,6 +101,9 @@ int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int
 // A bfloat16 matrix [N, K] (K a multiple of 32) copied so that the 64 16-byte units of a block of 16
 // rows and 32 values of K lie together in the order of the lanes that hold them: a wave's load of W
 // is then one piece of 1 KB.  The copy has fsie_fragment_order_size values (N rounded up to 16 rows).
+// whether they take M rows of this shape (65 to FSIE_GEMM_MFMA_WIDE_MAX_M rows: only some launch shapes on a
+// fragment-ordered weight)
+int fsie_gemm_mfma_wide_takes(int M, int N, int K, int splits, int gate_up, int frags);
 int64_t fsie_fragment_order_size(int N, int K);
 int fsie_fragment_order(const void* w, void* out, int N, int K, hipStream_t stream);
 

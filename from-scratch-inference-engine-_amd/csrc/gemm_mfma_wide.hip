@@ -220,7 +220,18 @@ int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, 
         case 2: return launch<2, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
 #if FSIE_WIDE_STEPS <= 4
         case 3: return launch<3, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
-        default: return launch<4, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+        case 4: return launch<4, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+        default:
+            // five to seven tiles of X (65 to 112 rows; the x tile still fits the 64 KB of static LDS): on a
+            // fragment-ordered weight, two row blocks a wave, four waves and more
+            if constexpr (FRAGS && NB == 2 && WAVES >= 4) {
+                if (mt == 5) return launch<5, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+                if (mt == 6) return launch<6, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+                if (mt == 7) return launch<7, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
+            }
+            fsie_set_error("gemm_mfma_wide: %d rows only on a fragment-ordered weight with two row blocks a wave and "
+                           "at least four waves (N = %d in %d slices gives %d blocks, %d waves)", M, N, splits, NB, WAVES);
+            return 1;
 #else
         default: fsie_set_error("gemm_mfma_wide: stages of %d steps hold at most 32 rows", STEPS); return 1;
 #endif
@@ -380,8 +391,9 @@ extern "C" int fsie_gemm_mfma_wide_best_splits(int M, int N, int K) {
 extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M, int N, int K, int splits,
                                    int waves, int blocks, int frags, hipStream_t stream) {
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide: bad sizes M=%d N=%d K=%d", M, N, K);
-    FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide: at most %d rows, got %d",
-                 FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
+    FSIE_REQUIRE(M <= (frags ? FSIE_GEMM_MFMA_WIDE_MAX_M : FSIE_GEMM_MFMA_SKINNY_MAX_M),
+                 "gemm_mfma_wide: at most %d rows (%d on a fragment-ordered weight), got %d", FSIE_GEMM_MFMA_SKINNY_MAX_M,
+                 FSIE_GEMM_MFMA_WIDE_MAX_M, M);
     const int k_slice = fsie_gemm_mfma_wide_slice(K, splits);
     FSIE_REQUIRE(k_slice > 0, "gemm_mfma_wide: K=%d cannot be cut into %d slices of whole stages of 128", K, splits);
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
@@ -402,8 +414,9 @@ extern "C" int fsie_gemm_mfma_wide(const void* x, const void* w, float* y, int M
 extern "C" int fsie_gemm_mfma_wide_swiglu(const void* x, const void* w, void* y, int M, int N, int K, int waves,
                                           int blocks, int frags, hipStream_t stream) {
     FSIE_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_mfma_wide_swiglu: bad sizes M=%d N=%d K=%d", M, N, K);
-    FSIE_REQUIRE(M <= FSIE_GEMM_MFMA_SKINNY_MAX_M, "gemm_mfma_wide_swiglu: at most %d rows, got %d",
-                 FSIE_GEMM_MFMA_SKINNY_MAX_M, M);
+    FSIE_REQUIRE(M <= (frags ? FSIE_GEMM_MFMA_WIDE_MAX_M : FSIE_GEMM_MFMA_SKINNY_MAX_M),
+                 "gemm_mfma_wide_swiglu: at most %d rows (%d on a fragment-ordered weight), got %d",
+                 FSIE_GEMM_MFMA_SKINNY_MAX_M, FSIE_GEMM_MFMA_WIDE_MAX_M, M);
     FSIE_REQUIRE(N % 4 == 0, "gemm_mfma_wide_swiglu: N=%d must be a multiple of 4 (gate and up rows in turn)", N);
     const int k_slice = fsie_gemm_mfma_wide_slice(K, 1);
     FSIE_REQUIRE(k_slice > 0, "gemm_mfma_wide_swiglu: K=%d must be a multiple of the stage of %d", K, 32 * FSIE_WIDE_STEPS);
@@ -441,4 +454,18 @@ extern "C" int fsie_fragment_order(const void* w, void* out, int N, int K, hipSt
         static_cast<const u32x4*>(w), static_cast<u32x4*>(out), N, K, units);
     FSIE_CHECK_LAUNCH("fragment_order");
     return 0;
+}
+
+// Whether the products above take M rows of this shape: up to 64 always; 65 to FSIE_GEMM_MFMA_WIDE_MAX_M only
+// on a fragment-ordered weight and where the launch shape they would choose has two row blocks a wave
+// and at least four waves a workgroup (the kernels of five to seven tiles exist for those only).
+// gate_up: the SiLU*up product (one slice).
+extern "C" int fsie_gemm_mfma_wide_takes(int M, int N, int K, int splits, int gate_up, int frags) {
+    if (M <= 0 || N <= 0 || fsie_gemm_mfma_wide_slice(K, gate_up ? 1 : splits) <= 0) return 0;
+    if (gate_up && N % 4) return 0;
+    if (M <= FSIE_GEMM_MFMA_SKINNY_MAX_M) return 1;
+    if (!frags || M > FSIE_GEMM_MFMA_WIDE_MAX_M || FSIE_WIDE_STEPS > 4) return 0;
+    int waves = 0, blocks = 0;
+    launch_shape((M + 15) / 16, N, gate_up ? 1 : splits, waves, blocks, gate_up != 0, true);
+    return blocks == 2 && waves >= 4;
 }

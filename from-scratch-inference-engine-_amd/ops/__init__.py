@@ -9,7 +9,7 @@ from .functions import (FragmentOrdered, attention_merge, attention_mfma, attent
                         attention_mfma_max_waves, attention_mfma_rows, attention_scalar,
                         attention_tile_tokens, bias_add, compute_units, dtype_code, embedding, fragment_order, gemm, gemm_mfma_fp32, gemm_mfma_skinny,
                         gemm_mfma_skinny_rope, gemm_mfma_wide, gemm_mfma_wide_best_splits, gemm_mfma_wide_splits_ok,
-                        gemm_mfma_wide_swiglu, random_fill,
+                        gemm_mfma_wide_swiglu, gemm_mfma_wide_takes, random_fill,
                         residual_add,
                         rmsnorm, rmsnorm_plain, rope_kv_write, rope_table, sample, swiglu, zero_pages, zero_rows)
 from .library import KernelError, KernelLibraryMissing, load
@@ -19,5 +19,5 @@ __all__ = ["FragmentOrdered", "KernelError", "KernelLibraryMissing", "attention_
            "attention_mfma_lds_ok", "attention_mfma_max_waves", "attention_mfma_rows", "attention_scalar",
            "attention_tile_tokens", "bias_add", "compute_units", "disable_library_tuning", "dtype_code", "embedding",
            "enable_library_tuning", "fragment_order", "gemm", "gemm_mfma_fp32", "gemm_mfma_skinny", "gemm_mfma_skinny_rope", "gemm_mfma_wide",
-           "gemm_mfma_wide_best_splits", "gemm_mfma_wide_splits_ok", "gemm_mfma_wide_swiglu", "library_mm", "library_tuning_enabled", "load", "random_fill", "residual_add",
+           "gemm_mfma_wide_best_splits", "gemm_mfma_wide_splits_ok", "gemm_mfma_wide_swiglu", "gemm_mfma_wide_takes", "library_mm", "library_tuning_enabled", "load", "random_fill", "residual_add",
            "rmsnorm", "rmsnorm_plain", "rope_kv_write", "rope_table", "sample", "swiglu", "zero_pages", "zero_rows"]

@@ -49,6 +49,7 @@ _SIGNATURES = {
     "fsie_gemm_mfma_wide_best_splits": ([c_int, c_int, c_int], c_int),
     "fsie_gemm_mfma_wide": ([_P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
     "fsie_gemm_mfma_wide_swiglu": ([_P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P], c_int),
+    "fsie_gemm_mfma_wide_takes": ([c_int, c_int, c_int, c_int, c_int, c_int], c_int),
     "fsie_fragment_order_size": ([c_int, c_int], c_int64),
     "fsie_fragment_order": ([_P, _P, c_int, c_int, _P], c_int),
     "fsie_attention_scalar": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,

@@ -8,7 +8,8 @@ import torch
 
 from .. import ops
 from ..ops.tuning import library_mm
-from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M, GEMM_MFMA_SKINNY_MAX_M, GEMM_SKINNY_MAX_M
+from ..ops.functions import (GEMM_MFMA_SKINNY_BEST_M, GEMM_MFMA_SKINNY_MAX_M, GEMM_MFMA_WIDE_MAX_M,
+                             GEMM_SKINNY_MAX_M)
 
 
 class Linear:
@@ -57,6 +58,7 @@ class Linear:
     def weight(self, t: Optional[torch.Tensor]) -> None:
         self._weight = t
         self.streamed = None  # a copy of the weight that was here says nothing about this one
+        self._wide_splits = {k: v for k, v in getattr(self, "_wide_splits", {}).items() if not isinstance(k, tuple)}
 
     def prepare(self) -> None:
         """Called by the owning part once the weight is set."""
@@ -117,6 +119,14 @@ class Linear:
         partial sums [S, T, N]; the next norm adds them up in order."""
         m = x.shape[0]
         if (getattr(ctx, "partial_sums_ok", False) and x.dtype == torch.bfloat16 and self.bias is None
+                and GEMM_MFMA_SKINNY_MAX_M < m <= GEMM_MFMA_WIDE_MAX_M and self.streamed is not None):
+            # 65 to 112 rows of a fragment-ordered weight: the same kernel with five to seven tiles of x,
+            # where its launch shape has one (N = 3584, K = 18944 on MI355X at 96 rows: 35 us in 9 slices; the
+            # library 95, or some 60 with its kernel chosen by timing)
+            splits = self.wide_splits(m)
+            if splits > 1 and self.wide_takes(m, splits):
+                return ops.gemm_mfma_wide(x, self.streamed, splits=splits)
+        if (getattr(ctx, "partial_sums_ok", False) and x.dtype == torch.bfloat16 and self.bias is None
                 and self.in_features % 8 == 0 and 0 < m <= GEMM_MFMA_SKINNY_MAX_M):
             # the kernel that shares x through LDS: above 16 rows, and at any number of rows where
             # K is long enough for six slices or more (N = 3584, K = 18944 in 8: 26 against 28 us at 8
@@ -130,17 +140,26 @@ class Linear:
         return self(x)
 
     def partial_sums(self, x: torch.Tensor) -> Optional[torch.Tensor]:
-        """x . W^T (no bias) of 17 to 64 rows as float32 partial sums [S, T, N] of slices of K, for a
+        """x . W^T (no bias) of 17 to 64 rows (to 112 from a fragment-ordered copy) as float32 partial sums [S, T, N] of slices of K, for a
         consumer that adds them up itself; None where the engine's kernel for that does not take the
         sizes (N = 4608, K = 3584 on MI355X at 64 rows: 12.4 us, the library's whole product 18.8;
         at 32 rows 9.1 against 13.6)."""
         m = x.shape[0]
-        if x.dtype != torch.bfloat16 or not GEMM_MFMA_SKINNY_BEST_M < m <= GEMM_MFMA_SKINNY_MAX_M:
+        most = GEMM_MFMA_SKINNY_MAX_M if self.streamed is None else GEMM_MFMA_WIDE_MAX_M
+        if x.dtype != torch.bfloat16 or not GEMM_MFMA_SKINNY_BEST_M < m <= most:
             return None
         splits = self.wide_splits(m)
-        if splits < 2:
+        if splits < 2 or not self.wide_takes(m, splits):
             return None
         return ops.gemm_mfma_wide(x, self.wide_weight, splits=splits)
+
+    def wide_takes(self, m: int, splits: int, gate_up: bool = False) -> bool:
+        """Whether the kernel that shares x through LDS takes ``m`` rows of this weight (beyond 64 rows
+        it has kernels for some launch shapes only)."""
+        key = ("takes", -(-m // 16), splits, gate_up, self.streamed is not None)
+        if key not in self._wide_splits:
+            self._wide_splits[key] = ops.gemm_mfma_wide_takes(m, self.wide_weight, splits, gate_up)
+        return self._wide_splits[key]
 
     def wide_splits(self, m: int) -> int:
         """Slices of K for the kernel that shares x through LDS, by the tiles of 16 rows that ``m``

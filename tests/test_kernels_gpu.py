@@ -507,8 +507,35 @@ def test_products_on_fragment_ordered_weights(ops, n, k):
                 assert torch.equal(a, b), (m, waves, blocks)
             with pytest.raises(KernelError, match="waves must be"):
                 ops.gemm_mfma_wide_swiglu(x, w, waves=5, blocks=2)
+    # 65 to 112 rows (five to seven tiles of x): only on this copy and only where the launch shape has two
+    # row blocks a wave and four waves or more, which the real gate/up and down shapes have; a row's sums
+    # are those of the same row in a product of 64 rows
+    for m in (65, 80, 112):
+        x = rnd((m, k), 77 + m, torch.bfloat16).cuda()
+        splits = ops.gemm_mfma_wide_best_splits(m, n, k)
+        takes = ops.gemm_mfma_wide_takes(m, f, splits)
+        assert takes or (n, k) not in ((3584, 18944), (5120, 13824), (152064, 3584)), (m, splits)
+        assert not takes or n >= 2048, (m, splits)  # (few rows of W leave no launch shape with two blocks a wave)
+        assert not ops.gemm_mfma_wide_takes(m, w, splits) and not ops.gemm_mfma_wide_takes(113, f, splits)
+        if takes:
+            got = ops.gemm_mfma_wide(x, f, splits=splits)
+            assert torch.equal(got[..., :64, :], ops.gemm_mfma_wide(x[:64].contiguous(), f, splits=splits))
+            assert torch.equal(got[..., 64:, :], ops.gemm_mfma_wide(x[64:].contiguous(), f, splits=splits))
+        else:
+            with pytest.raises(KernelError, match="rows only on a fragment-ordered weight|at most 64 rows"):
+                ops.gemm_mfma_wide(x, f, splits=splits)
+        if n % 4 == 0:
+            takes = ops.gemm_mfma_wide_takes(m, f, 1, gate_up=True)
+            assert takes == (n >= 24577), m  # four waves of two blocks a workgroup, one workgroup a unit, from there on
+            if takes:
+                got = ops.gemm_mfma_wide_swiglu(x, f)
+                assert torch.equal(got[:64], ops.gemm_mfma_wide_swiglu(x[:64].contiguous(), f))
+                assert torch.equal(got[64:], ops.gemm_mfma_wide_swiglu(x[64:].contiguous(), f))
+        with pytest.raises(KernelError, match="at most 64 rows"):
+            ops.gemm_mfma_wide(x, w, splits=splits)
+    x = rnd((64, k), 32 + 64, torch.bfloat16).cuda()
     if not big:
-        full = (x.double() @ w.double().t()).float()  # the last x: 64 rows
+        full = (x.double() @ w.double().t()).float()  # 64 rows
         assert (ops.gemm_mfma_wide(x, f) - full).abs().max() <= tol(torch.float32, full.cpu()) * 4
     with pytest.raises(KernelError, match="multiple of 32"):
         ops.fragment_order(w[:, :k - 16].contiguous())

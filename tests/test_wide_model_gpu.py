@@ -16,8 +16,9 @@ bound is stated against that: the engine may differ from the plain float32 logit
 twice (largest) and one and a half times (root mean square) what the plain model itself moves
 when its activations are rounded to bfloat16 where the engine rounds them, and it picks the
 plain token wherever that one leads by more than twice the largest difference.  Decode batches
-of 32, 64 and 128 through replayed graphs, with the library's kernels chosen by timing, are checked
-against the plain logits in the same way.
+of 32, 64, 80, 100 and 128 through replayed graphs (rows of 32, 64, 80, 112 and 128: the engine's own
+products up to 112 rows, beyond that the library's, its kernels chosen by timing) are checked against
+the plain logits in the same way.
 """
 
 import json
@@ -197,13 +198,18 @@ def test_bfloat16_families_and_graph_batches_at_7b_widths(wide):
     print(f"bfloat16 at 7B widths: difference / rounding noise, largest {max(r[0] for r in ratios):.2f} (max), "
           f"{max(r[1] for r in ratios):.2f} (rms)")
     del runner
-    # decode batches of 32, 64 and 128 rows: the library's products (chosen by timing) inside replayed
-    # graphs, with other work between the replays; the first eight requests against the plain model
+    # decode batches of 32 to 128 rows: the engine's products up to 112 rows, the library's (chosen by
+    # timing) beyond and for the small matrices, inside replayed graphs, with other work between the replays; the first eight requests against the plain model
     noise = max(n[0] for n in wide["noise"]), max(n[1] for n in wide["noise"])
     short, short_ref = wide["short"], wide["short_ref"]
     ops.enable_library_tuning(max_ms_per_candidate=5, iterations=2)
+    own_rows = set()  # rows of the steps whose feed-forward products are the engine's own kernels
+    real_swiglu, real_wide = ops.gemm_mfma_wide_swiglu, ops.gemm_mfma_wide
+    ops.gemm_mfma_wide_swiglu = lambda x, w, **k: (own_rows.add(("gate/up", x.shape[0])), real_swiglu(x, w, **k))[1]
+    ops.gemm_mfma_wide = lambda x, w, **k: (own_rows.add(("slices", x.shape[0])) if k.get("splits", 1) > 1 else None,
+                                            real_wide(x, w, **k))[1]
     try:
-        for batch in (32, 64, 128):
+        for batch in (32, 64, 80, 100, 128):
             runner = Runner(model, page_size=16, num_pages=batch * 3 + 8, max_requests=batch)
             caches = [runner.manager.open(i) for i in range(batch)]
             runner.step([StepEntry(c, p[:-12], []) for c, p in zip(caches, short)])
@@ -218,3 +224,8 @@ def test_bfloat16_families_and_graph_batches_at_7b_widths(wide):
             del runner, caches
     finally:
         ops.disable_library_tuning()
+        ops.gemm_mfma_wide_swiglu, ops.gemm_mfma_wide = real_swiglu, real_wide
+    # 80 and 100 requests run in graphs of 80 and 112 rows, on the engine's kernels of five and seven tiles
+    # of rows over the fragment-ordered weights; 128 rows are the library's
+    assert {("gate/up", 80), ("gate/up", 112), ("slices", 80), ("slices", 112)} <= own_rows, own_rows
+    assert not any(rows > 112 for _, rows in own_rows), own_rows
