@@ -11,7 +11,7 @@
 
 #define FSIE_GEMM_SKINNY_MAX_M 8
 #define FSIE_GEMM_MFMA_SKINNY_MAX_M 64
-#define FSIE_GEMM_MFMA_WIDE_MAX_M 112  // the product that shares x through LDS, on a fragment-ordered weight: seven tiles of 16 rows
+#define FSIE_GEMM_MFMA_WIDE_MAX_M 128  // the product that shares x through LDS, on a fragment-ordered weight: eight tiles of 16 rows
 #define FSIE_GEMM_MFMA_SKINNY_BEST_M 16  // above this the library product is faster on MI355X
 #define FSIE_GEMM_MAX_SPLITS 16          // most slices of K a product may leave as partial sums
 

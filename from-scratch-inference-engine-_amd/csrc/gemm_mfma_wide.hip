@@ -43,6 +43,11 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+extern __shared__ u32x4 wide_dynamic_lds[];
+constexpr int kStaticLds = 64 * 1024;
+// bytes of the two buffers of a stage of X of `mt` tiles of 16 rows
+constexpr int wide_lds_bytes(int mt, int steps) { return 2 * (4 * steps * (16 * mt + 1) + 1) * 16; }
 typedef const __attribute__((address_space(1))) u32x4* GlobalVec;
 
 union Frag {
@@ -68,7 +73,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_mfma_wide_kernel(const bf16_t
     constexpr int PITCH = ROWS + 1;           // units between consecutive (step, k group) runs: the
                                               // odd pitch spreads a staging wave's writes over the banks
     constexpr int SPARE = 4 * STEPS * PITCH;  // where threads without a unit of their own write
-    __shared__ u32x4 xs[2][4 * STEPS * PITCH + 1];
+    // the two buffers of a stage of X: static up to seven tiles (58 KB); eight tiles (66 KB) take the LDS
+    // that the launch asks for beyond the 64 KB a kernel may declare
+    constexpr int BUF = 4 * STEPS * PITCH + 1;
+    constexpr bool DYNAMIC = wide_lds_bytes(MT, STEPS) > kStaticLds;
+    __shared__ u32x4 xs_static[DYNAMIC ? 1 : 2 * BUF];
+    u32x4* const xs0 = DYNAMIC ? wide_dynamic_lds : xs_static;
+    u32x4* const xs[2] = {xs0, xs0 + BUF};
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -207,7 +218,18 @@ int launch(const bf16_t* x, const bf16_t* w, float* y, int M, int N, int K, int 
            hipStream_t stream) {
     const int rows = 16 * NB * WAVES;
     const dim3 grid(static_cast<unsigned>((N + rows - 1) / rows), static_cast<unsigned>(splits));
-    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB, SWIGLU, FRAGS><<<grid, WAVES * 64, 0, stream>>>(x, w, y, M, N, K, k_slice);
+    constexpr int lds = wide_lds_bytes(MT, STEPS);
+    constexpr int dynamic = lds > kStaticLds ? lds : 0;
+    if constexpr (dynamic > 0) {
+        static const hipError_t allowed = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(&gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB, SWIGLU, FRAGS>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, dynamic);
+        if (allowed != hipSuccess) {
+            fsie_set_error("gemm_mfma_wide: %d bytes of LDS for %d rows: %s", dynamic, M, hipGetErrorString(allowed));
+            return 1;
+        }
+    }
+    gemm_mfma_wide_kernel<MT, WAVES, STEPS, NB, SWIGLU, FRAGS><<<grid, WAVES * 64, dynamic, stream>>>(x, w, y, M, N, K, k_slice);
     FSIE_CHECK_LAUNCH("gemm_mfma_wide");
     return 0;
 }
@@ -222,9 +244,10 @@ int launch_mt(int mt, const bf16_t* x, const bf16_t* w, float* y, int M, int N, 
         case 3: return launch<3, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
         case 4: return launch<4, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
         default:
-            // five to seven tiles of X (65 to 112 rows; the x tile still fits the 64 KB of static LDS): on a
-            // fragment-ordered weight, two row blocks a wave, four waves and more
+            // five to eight tiles of X (65 to 128 rows): on a fragment-ordered weight, two row blocks a
+            // wave, four waves and more
             if constexpr (FRAGS && NB == 2 && WAVES >= 4) {
+                if (mt == 8) return launch<8, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
                 if (mt == 5) return launch<5, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
                 if (mt == 6) return launch<6, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);
                 if (mt == 7) return launch<7, WAVES, STEPS, NB, SWIGLU, FRAGS>(x, w, y, M, N, K, splits, k_slice, stream);

@@ -36,11 +36,11 @@ CAPTURE_AFTER = 3  # a shape is captured the n-th time it is asked for (read whe
 
 def padded_rows(n: int) -> int:
     """Rows of the graph that serves a decode step of ``n`` requests: 1, 2, 4, 8, then multiples
-    of 16 (a tile of rows in the products) up to 112, which is what the engine's own products
+    of 16 (a tile of rows in the products) up to 128, which is what the engine's own products
     take, above that of 32."""
     if n <= 8:
         return 1 << max(0, n - 1).bit_length()
-    step = 16 if n <= 112 else 32
+    step = 16 if n <= 128 else 32
     return -(-n // step) * step
 
 

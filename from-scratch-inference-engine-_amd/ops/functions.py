@@ -13,7 +13,7 @@ ATTN_ITEM_INTS = 8
 ATTN_MERGE_INTS = 4
 GEMM_SKINNY_MAX_M = 8
 GEMM_MFMA_SKINNY_MAX_M = 64
-GEMM_MFMA_WIDE_MAX_M = 112  # the product that shares x through LDS, on a fragment-ordered weight
+GEMM_MFMA_WIDE_MAX_M = 128  # the product that shares x through LDS, on a fragment-ordered weight
 GEMM_MFMA_SKINNY_BEST_M = 16
 GEMM_SPLITS = (2, 4, 8)  # slices of K that the few-rows product may leave as partial sums
 GEMM_MAX_SPLITS = 16     # most slices of the product that shares x through LDS, and most that a norm adds up
@@ -363,8 +363,8 @@ def _wide_weight(weight, k: int):
 
 def gemm_mfma_wide_takes(m: int, weight, splits: int = 1, gate_up: bool = False) -> bool:
     """Whether ``gemm_mfma_wide`` (``gate_up``: ``gemm_mfma_wide_swiglu``) takes ``m`` rows against this
-    weight in ``splits`` slices: up to 64 rows wherever it takes the inner size; 65 to 112 rows only on a
-    ``FragmentOrdered`` copy, for the launch shapes that have kernels of five to seven tiles of rows."""
+    weight in ``splits`` slices: up to 64 rows wherever it takes the inner size; 65 to 128 rows only on a
+    ``FragmentOrdered`` copy, for the launch shapes that have kernels of five to eight tiles of rows."""
     n, k = weight.shape
     return bool(load().fsie_gemm_mfma_wide_takes(int(m), int(n), int(k), int(splits), int(gate_up),
                                                  int(isinstance(weight, FragmentOrdered))))

@@ -7,7 +7,7 @@ other kernels are sometimes a good deal faster (measured on MI355X at 2,048 rows
 torch's TunableOp times the library's candidates the first time a shape is seen and keeps the
 best (in the process, and in a file under the temporary folder for later ones).  Each new shape
 costs seconds (at 16,384 rows, minutes), so only two kinds of row counts are tuned: multiples of 256
-up to 4,096 (a full token budget of prefill), multiples of 16 up to 112 and of 32 up to 256 (decode batches, timed in the eager run that precedes the
+up to 4,096 (a full token budget of prefill), multiples of 16 up to 128 and of 32 up to 256 (decode batches, timed in the eager run that precedes the
 capture of their graph); never inside a graph capture.  Other shapes use what has been found for
 them, or the heuristic.
 """
@@ -23,7 +23,7 @@ from ..csrc.build import private_tmp_dir
 _TUNED_ROWS, _TUNED_MAX_ROWS = 256, 4096
 _TUNED_DECODE_ROWS, _TUNED_DECODE_MAX = 16, 64   # decode batches are padded to these row counts ...
 _TUNED_LARGE_ROWS, _TUNED_LARGE_MAX = 32, 256    # ... and, beyond 64 rows, to these
-_TUNED_TILES_MAX = 112                           # (and to multiples of 16 up to here)
+_TUNED_TILES_MAX = 128                           # (and to multiples of 16 up to here)
 _state = {"on": False}
 
 

@@ -120,7 +120,7 @@ class Linear:
         m = x.shape[0]
         if (getattr(ctx, "partial_sums_ok", False) and x.dtype == torch.bfloat16 and self.bias is None
                 and GEMM_MFMA_SKINNY_MAX_M < m <= GEMM_MFMA_WIDE_MAX_M and self.streamed is not None):
-            # 65 to 112 rows of a fragment-ordered weight: the same kernel with five to seven tiles of x,
+            # 65 to 128 rows of a fragment-ordered weight: the same kernel with five to eight tiles of x,
             # where its launch shape has one (N = 3584, K = 18944 on MI355X at 96 rows: 35 us in 9 slices; the
             # library 95, or some 60 with its kernel chosen by timing)
             splits = self.wide_splits(m)
@@ -140,7 +140,7 @@ class Linear:
         return self(x)
 
     def partial_sums(self, x: torch.Tensor) -> Optional[torch.Tensor]:
-        """x . W^T (no bias) of 17 to 64 rows (to 112 from a fragment-ordered copy) as float32 partial sums [S, T, N] of slices of K, for a
+        """x . W^T (no bias) of 17 to 64 rows (to 128 from a fragment-ordered copy) as float32 partial sums [S, T, N] of slices of K, for a
         consumer that adds them up itself; None where the engine's kernel for that does not take the
         sizes (N = 4608, K = 3584 on MI355X at 64 rows: 12.4 us, the library's whole product 18.8;
         at 32 rows 9.1 against 13.6)."""

@@ -53,13 +53,13 @@ class SwiGLU(FeedForward):
 
     # rows up to which silu(gate) * up comes from the product that shares x through LDS when the weight
     # has a fragment-ordered copy (beyond: the library's product and a kernel for SiLU*up)
-    streamed_swiglu_max_rows = 112
+    streamed_swiglu_max_rows = 128
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         m = x.shape[0]
         if (x.dtype == torch.bfloat16 and self.gate_up.streamed is not None and 0 < m <= self.streamed_swiglu_max_rows
                 and self.gate_up.wide_takes(m, 1, gate_up=True)):
-            # from the fragment-ordered copy at any number of rows up to 64, and up to 112 where the kernel
+            # from the fragment-ordered copy at any number of rows up to 64, and up to 128 where the kernel
             # has the launch shape for it (MI355X, N = 37888, K = 3584: 44 us for 1 to 16 rows, where the
             # few-rows kernel takes 49 to 55 on rows; 49 at 64 rows, 52 at 96, 54 at 112, where the library
             # and a SiLU*up kernel take 66, 69 and 75)

@@ -290,8 +290,8 @@ def test_a_batch_that_shrinks_decodes_through_graphs_of_padded_sizes(model_dirs,
     from from_scratch_inference_engine_amd.engine.graphs import padded_rows
     from from_scratch_inference_engine_amd.engine.model import Runner
 
-    assert [padded_rows(n) for n in (1, 2, 3, 4, 5, 8, 9, 16, 17, 33, 64, 65, 100, 113, 130)] == \
-        [1, 2, 4, 4, 8, 8, 16, 16, 32, 48, 64, 80, 112, 128, 160]
+    assert [padded_rows(n) for n in (1, 2, 3, 4, 5, 8, 9, 16, 17, 33, 64, 65, 100, 113, 129, 130)] == \
+        [1, 2, 4, 4, 8, 8, 16, 16, 32, 48, 64, 80, 112, 128, 160, 160]
     model = load_model(model_dirs["A"], dtype=dtype)
     vocab = plain.read_config(model_dirs["A"])["vocab_size"]
     seqs = [helpers.token_ids(vocab, 30 + 3 * i, 900 + i) for i in range(7)]

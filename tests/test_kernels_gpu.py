@@ -507,16 +507,16 @@ def test_products_on_fragment_ordered_weights(ops, n, k):
                 assert torch.equal(a, b), (m, waves, blocks)
             with pytest.raises(KernelError, match="waves must be"):
                 ops.gemm_mfma_wide_swiglu(x, w, waves=5, blocks=2)
-    # 65 to 112 rows (five to seven tiles of x): only on this copy and only where the launch shape has two
+    # 65 to 128 rows (five to eight tiles of x, the eighth with LDS that the launch asks for): only on this copy and only where the launch shape has two
     # row blocks a wave and four waves or more, which the real gate/up and down shapes have; a row's sums
     # are those of the same row in a product of 64 rows
-    for m in (65, 80, 112):
+    for m in (65, 80, 112, 128):
         x = rnd((m, k), 77 + m, torch.bfloat16).cuda()
         splits = ops.gemm_mfma_wide_best_splits(m, n, k)
         takes = ops.gemm_mfma_wide_takes(m, f, splits)
         assert takes or (n, k) not in ((3584, 18944), (5120, 13824), (152064, 3584)), (m, splits)
         assert not takes or n >= 2048, (m, splits)  # (few rows of W leave no launch shape with two blocks a wave)
-        assert not ops.gemm_mfma_wide_takes(m, w, splits) and not ops.gemm_mfma_wide_takes(113, f, splits)
+        assert not ops.gemm_mfma_wide_takes(m, w, splits) and not ops.gemm_mfma_wide_takes(129, f, splits)
         if takes:
             got = ops.gemm_mfma_wide(x, f, splits=splits)
             assert torch.equal(got[..., :64, :], ops.gemm_mfma_wide(x[:64].contiguous(), f, splits=splits))
