@@ -48,7 +48,8 @@ class Linear:
         self._weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
         self.streamed = None  # the weight in fragment order (ops.FragmentOrdered), if prepare() made one
-        self._wide_splits: dict = {}
+        self._wide_splits: dict = {}  # tiles of rows -> slices of K (a property of the sizes alone)
+        self._wide_takes: dict = {}   # (tiles, slices, gate/up) -> whether the kernel takes them from this weight
 
     @property
     def weight(self) -> Optional[torch.Tensor]:
@@ -58,7 +59,7 @@ class Linear:
     def weight(self, t: Optional[torch.Tensor]) -> None:
         self._weight = t
         self.streamed = None  # a copy of the weight that was here says nothing about this one
-        self._wide_splits = {k: v for k, v in getattr(self, "_wide_splits", {}).items() if not isinstance(k, tuple)}
+        self._wide_takes = {}
 
     def prepare(self) -> None:
         """Called by the owning part once the weight is set."""
@@ -156,10 +157,10 @@ class Linear:
     def wide_takes(self, m: int, splits: int, gate_up: bool = False) -> bool:
         """Whether the kernel that shares x through LDS takes ``m`` rows of this weight (beyond 64 rows
         it has kernels for some launch shapes only)."""
-        key = ("takes", -(-m // 16), splits, gate_up, self.streamed is not None)
-        if key not in self._wide_splits:
-            self._wide_splits[key] = ops.gemm_mfma_wide_takes(m, self.wide_weight, splits, gate_up)
-        return self._wide_splits[key]
+        key = (-(-m // 16), splits, gate_up, self.streamed is not None)
+        if key not in self._wide_takes:
+            self._wide_takes[key] = ops.gemm_mfma_wide_takes(m, self.wide_weight, splits, gate_up)
+        return self._wide_takes[key]
 
     def wide_splits(self, m: int) -> int:
         """Slices of K for the kernel that shares x through LDS, by the tiles of 16 rows that ``m``
