@@ -93,6 +93,7 @@ def kernel_classes(runner, cfg, batch: int, prompt_len: int, itemsize: int) -> d
     classify = {
         "gemm_mfma_skinny_rope": lambda a, k: "qkv", "rope_kv_write": lambda a, k: "qkv", "bias_add": lambda a, k: "qkv",
         "attention_mfma": lambda a, k: "attention", "attention_mfma_lds": lambda a, k: "attention",
+        "attention_mfma_qkv": lambda a, k: "attention",
         "attention_scalar": lambda a, k: "attention", "attention_merge": lambda a, k: "attention",
         "gemm_mfma_skinny": lambda a, k: matrix_class(a[1]), "gemm_mfma_wide": lambda a, k: matrix_class(a[1]),
         "gemm_mfma_wide_swiglu": lambda a, k: "gate_up",
@@ -128,8 +129,7 @@ def kernel_classes(runner, cfg, batch: int, prompt_len: int, itemsize: int) -> d
         runner.graphs = graphs
     weights = {"qkv": h * (q + 2 * cfg.num_key_value_heads * cfg.head_dim), "o": q * h, "gate_up": 2 * h * inter,
                "down": h * inter}
-    n_layers = sum(1 for c in calls if c[0] == "qkv" and c[1].__name__ in ("gemm_mfma_skinny_rope", "library_mm", "gemm",
-                                                                         "gemm_mfma_fp32"))
+    n_layers = sum(1 for c in calls if c[0] == "down")  # (one product a layer, whichever kernel takes it)
     read = {k: n * itemsize * n_layers for k, n in weights.items()}
     read["lm_head"] = h * v * itemsize
     read["attention"] = batch * (prompt_len + 1) * 2 * cfg.num_key_value_heads * cfg.head_dim * itemsize * n_layers

@@ -119,6 +119,14 @@ int fsie_attention_mfma(const void* q, int64_t q_stride, const void* k_pool, con
                         const int32_t* block_tables, int max_pages, const int32_t* items, int n_items, void* out,
                         float* partials, int n_heads, int n_kv, int head_dim, int page_size, int window, float scale,
                         int large, int waves, hipStream_t stream);
+// the same for a step of one token a request, from the q/k/v product's partial sums: bias, rotation and the
+// write into the pools happen in the kernel
+int fsie_attention_mfma_qkv_ok(int head_dim, int page_size);
+int fsie_attention_mfma_qkv(const float* sums, int n_parts, int n_tokens, const float* bias, const float* cos_sin,
+                            const int32_t* slots, void* k_pool, void* v_pool, int64_t pool_slots,
+                            const int32_t* block_tables, int max_pages, const int32_t* items, int n_items, void* out,
+                            float* partials, int n_heads, int n_kv, int head_dim, int page_size, int window,
+                            float scale, int waves, hipStream_t stream);
 int fsie_attention_mfma_lds_ok(int head_dim, int page_size);
 int fsie_attention_mfma_lds(const void* q, int64_t q_stride, const void* k_pool, const void* v_pool,
                             const int32_t* block_tables, int max_pages, const int32_t* items, const int32_t* groups,

@@ -14,4 +14,12 @@ LaunchFn table_a(int hdt, int large) {
     }
 }
 
+LaunchQkvFn table_a_qkv(int hdt) {
+    switch (hdt) {
+        case 2: return launch_qkv<2>;
+        case 4: return launch_qkv<4>;
+        default: return nullptr;
+    }
+}
+
 }  // namespace fsie_attn

@@ -14,4 +14,12 @@ LaunchFn table_b(int hdt, int large) {
     }
 }
 
+LaunchQkvFn table_b_qkv(int hdt) {
+    switch (hdt) {
+        case 6: return launch_qkv<6>;
+        case 8: return launch_qkv<8>;
+        default: return nullptr;
+    }
+}
+
 }  // namespace fsie_attn

@@ -14,4 +14,12 @@ LaunchFn table_c(int hdt, int large) {
     }
 }
 
+LaunchQkvFn table_c_qkv(int hdt) {
+    switch (hdt) {
+        case 10: return launch_qkv<10>;
+        case 12: return launch_qkv<12>;
+        default: return nullptr;
+    }
+}
+
 }  // namespace fsie_attn

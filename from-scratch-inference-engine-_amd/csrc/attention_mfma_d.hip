@@ -14,4 +14,12 @@ LaunchFn table_d(int hdt, int large) {
     }
 }
 
+LaunchQkvFn table_d_qkv(int hdt) {
+    switch (hdt) {
+        case 14: return launch_qkv<14>;
+        case 16: return launch_qkv<16>;
+        default: return nullptr;
+    }
+}
+
 }  // namespace fsie_attn

@@ -31,6 +31,12 @@
 // maxima and sums through LDS, then the first wave adds the others' rescaled accumulators to its
 // own in the fixed order of the waves.  Decoding against a long context therefore needs neither partial
 // records in memory nor a second kernel, and the result does not depend on timing.
+//
+// QKV: the variant for steps of one token a request takes q, k and v as the float32 partial sums
+// that a product in slices of K leaves, and finishes them itself: every workgroup adds up the
+// heads it needs (its queries, and its kv head's key and value), adds the bias, rotates queries
+// and key, and the workgroup whose keys end with the new one scores it from registers and writes
+// it and its value into the pools.  That spares the launch between the product and attention.
 #pragma once
 
 #include "common.h"
@@ -56,6 +62,48 @@ union F8B {
 __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ uint2 ld8(const bf16_t* p) { return *reinterpret_cast<const uint2*>(p); }
 
+// What the QKV variant reads and writes beside the kernel's other operands.
+struct QkvSums {
+    const float* sums;     // [n_parts][n_tokens][width], width = (n_heads + 2 n_kv) head_dim
+    const float* bias;     // [width], or null
+    const float* cos_sin;  // [n_tokens][head_dim / 2] pairs (cos, sin) of each token's position
+    const int32_t* slots;  // [n_tokens] slot of a token's key and value in the pools (negative: nowhere)
+    bf16_t* k_out;         // the pools again, to write
+    bf16_t* v_out;
+    int64_t part_stride;   // n_tokens * width
+    int64_t pool_slots;
+    int n_parts, width;
+};
+
+// Element d of a head after the rotation of the pairs (i, i + HD / 2) by the angles whose
+// cosines and sines are cs[i].  One fixed sequence of roundings, whoever asks: the key that a
+// step scores from registers and its copy in the cache are the same numbers.
+__device__ __forceinline__ float rotated_by(float a, float b, float cosine, float sine, bool hi) {
+    const float bs = __fmul_rn(b, sine);
+    return __fmaf_rn(a, cosine, hi ? bs : -bs);
+}
+template <int HD>
+__device__ __forceinline__ float rotated(const float* head, const float2* cs, int d) {
+    constexpr int half = HD / 2;
+    const bool hi = d >= half;
+    const float2 t = cs[hi ? d - half : d];
+    return rotated_by(head[d], head[hi ? d - half : d + half], t.x, t.y, hi);
+}
+// The same for the elements d0 .. d0 + 7 (d0 a multiple of 8), as two bfloat16 a register: 16-byte reads.
+template <int HD>
+__device__ __forceinline__ uint4 rotated8(const float* head, const float2* cs, int d0) {
+    constexpr int half = HD / 2;
+    const bool hi = d0 >= half;
+    const float4* a = reinterpret_cast<const float4*>(head + d0);
+    const float4* b = reinterpret_cast<const float4*>(head + (hi ? d0 - half : d0 + half));
+    const float4* t = reinterpret_cast<const float4*>(cs + (hi ? d0 - half : d0));
+    const float4 a0 = a[0], a1 = a[1], b0 = b[0], b1 = b[1], t0 = t[0], t1 = t[1], t2 = t[2], t3 = t[3];
+    return uint4{pack2_bf16(rotated_by(a0.x, b0.x, t0.x, t0.y, hi), rotated_by(a0.y, b0.y, t0.z, t0.w, hi)),
+                 pack2_bf16(rotated_by(a0.z, b0.z, t1.x, t1.y, hi), rotated_by(a0.w, b0.w, t1.z, t1.w, hi)),
+                 pack2_bf16(rotated_by(a1.x, b1.x, t2.x, t2.y, hi), rotated_by(a1.y, b1.y, t2.z, t2.w, hi)),
+                 pack2_bf16(rotated_by(a1.z, b1.z, t3.x, t3.y, hi), rotated_by(a1.w, b1.w, t3.z, t3.w, hi))};
+}
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -64,12 +112,13 @@ constexpr int max_waves() {
     return HDT <= 4 ? 16 : (HDT <= 8 ? 8 : 4);  // registers per wave grow with the head size
 }
 
-template <int HDT, int NT, int MAXW, bool V16>
-__global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW == 1 && NT > 1 ? 2 : 1))) void attention_mfma_kernel(
+template <int HDT, int NT, int MAXW, bool V16, bool QKV = false>
+__global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW == 1 && NT > 1 ? 2 : 1))) void attention_mfma_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_pages,
     const int32_t* __restrict__ items, bf16_t* __restrict__ out, float* __restrict__ partials, int n_heads,
-    int n_kv, int page_size, int window, float scale, int gh, int head_chunks) {
+    int n_kv, int page_size, int window, float scale, int gh, int head_chunks, QkvSums f) {
+    static_assert(!QKV || (NT == 1 && HDT % 2 == 0), "the QKV variant: one query tile, head_dim a multiple of 32");
     constexpr int HD = HDT * 16;
     // scores: 32-wide steps over the head dimension when head_dim is a multiple of 32, else
     // 16-wide steps throughout (the two shapes are never chained on one accumulator)
@@ -85,9 +134,15 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
     const int n_q = item[FSIE_ATTN_ITEM_NQ];
     const int pos0 = item[FSIE_ATTN_ITEM_POS];
     const int key_begin = item[FSIE_ATTN_ITEM_KBEGIN];
-    const int key_end = item[FSIE_ATTN_ITEM_KEND];
+    int key_end = item[FSIE_ATTN_ITEM_KEND];
     const int partial_base = item[FSIE_ATTN_ITEM_PARTIAL];
     if (n_q <= 0) return;  // padding item
+    // QKV: the item whose keys end with the request's new one walks the cache up to it and takes
+    // the new key and value from the sums
+    const bool owner = QKV && pos0 >= key_begin && pos0 < key_end;
+    if (owner) key_end = pos0;
+    int new_slot = -1;
+    if constexpr (QKV) new_slot = f.slots[q_row0];
 
     const int group = n_heads / n_kv;
     const int kvh = blockIdx.y / head_chunks;
@@ -98,11 +153,87 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int n_waves = blockDim.x >> 6;
+    // (the QKV variant of one wave is launched with four: three only help to add up the sums)
+    const int n_waves = QKV && MAXW == 1 ? 1 : blockDim.x >> 6;
     const int c = lane & 15;  // column of S^T and O^T (query row of a tile); row of the A tiles
     const int G = lane >> 4;  // lane group: which 4 (or 8) of the reduction indices this lane holds
     const int32_t* table = block_tables + static_cast<int64_t>(seq) * max_pages;
     const float scale2 = scale * kLog2e;  // scores in units of log2 e: exp() becomes exp2()
+
+    // LDS: the accumulators that the waves after the first hand over at the end; before that, in
+    // the QKV variant, the heads added up from the sums (up to 16 of queries, a key, a value) and
+    // the cosines and sines
+    constexpr int kCombine = MAXW > 1 ? (MAXW - 1) * NT * HDT * 64 : 0;
+    constexpr int RS = HD + 4;  // a head's row in LDS: four floats apart from a multiple of the banks, so that 16 rows read 16 bytes each without conflict
+    constexpr int kHeads = QKV ? (18 * RS + HD) / 4 : 0;
+    constexpr int kLds = kCombine > kHeads ? kCombine : (kHeads > 0 ? kHeads : 1);
+    __shared__ floatx4 s_o[kLds];
+    float* s_row = reinterpret_cast<float*>(s_o);
+    float2* s_cs = reinterpret_cast<float2*>(s_row + 18 * RS);
+    // The heads this workgroup needs, added up over the slices, with the bias, into LDS.  In two
+    // steps, so that the reads of the first slices (straight-line code: a slice past the last reads
+    // the last one again, a thread without a column reads column 0) are under way together with the
+    // first reads of the block table, and one trip to memory serves both.
+    // (the variant of one wave is launched with four: the other three add up the sums, so that the
+    // first has only its keys under way: the hardware counts 63 reads at most, and a wait for one of
+    // 27 reads of sums behind 64 of keys would wait for most of the keys too)
+    constexpr int kThreadsLeast = MAXW == 1 ? 192 : 64 * MAXW;  // threads that add up sums
+    constexpr int NJ = QKV ? (18 * HD / 4 + kThreadsLeast - 1) / kThreadsLeast : 1;  // columns of four a thread
+    constexpr int PC = NJ <= 3 ? 8 : 4;                                              // slices read at once
+    float4 part[NJ][PC], bias_of[NJ];
+    float2 angle = float2{1.f, 0.f};
+    int lds_at[NJ];
+    const float* col_at[NJ];
+    const int sum_thread = MAXW == 1 ? static_cast<int>(threadIdx.x) - 64 : static_cast<int>(threadIdx.x);
+    const int sum_threads = MAXW == 1 ? static_cast<int>(blockDim.x) - 64 : static_cast<int>(blockDim.x);
+    const bool helper = QKV && MAXW == 1 && wave > 0;  // a wave that only adds up sums
+    const bool sums_here = MAXW > 1 || wave > 0;
+    auto issue_sums = [&]() {
+        const int q_dim = n_heads * HD, kv_dim = n_kv * HD;
+        const int n_cols = (gh_here + 2) * HD;
+        const float* row = f.sums + static_cast<int64_t>(q_row0) * f.width;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            if (j * sum_threads * 4 >= n_cols) {  // (the same for the whole workgroup: no thread has such a column)
+                lds_at[j] = -1;
+                continue;
+            }
+            const int i = (sum_thread + j * sum_threads) * 4;
+            const bool has = i >= 0 && i < n_cols;
+            const int ic = has ? i : 0;
+            const int seg = ic / HD, d = ic - seg * HD;
+            lds_at[j] = has ? seg * RS + d : -1;
+            const int col = seg < gh_here ? (h_base + seg) * HD + d : q_dim + (seg - gh_here) * kv_dim + kvh * HD + d;
+            col_at[j] = row + col;
+#pragma unroll
+            for (int u = 0; u < PC; ++u)
+                part[j][u] = *reinterpret_cast<const float4*>(col_at[j] + min(u, f.n_parts - 1) * f.part_stride);
+            bias_of[j] = *reinterpret_cast<const float4*>(f.bias ? f.bias + col : col_at[j]);
+        }
+        const float2* cs = reinterpret_cast<const float2*>(f.cos_sin) + static_cast<int64_t>(q_row0) * (HD / 2);
+        angle = cs[min(max(sum_thread, 0), HD / 2 - 1)];
+    };
+    auto finish_sums = [&]() {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            if (j * sum_threads * 4 >= (gh_here + 2) * HD) continue;
+            float4 a{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < PC; ++u)
+                if (u < f.n_parts)
+                    a = float4{a.x + part[j][u].x, a.y + part[j][u].y, a.z + part[j][u].z, a.w + part[j][u].w};
+            for (int s = PC; s < f.n_parts; ++s) {  // (more slices than are read at once: a trip each)
+                const float4 v = *reinterpret_cast<const float4*>(col_at[j] + s * f.part_stride);
+                a = float4{a.x + v.x, a.y + v.y, a.z + v.z, a.w + v.w};
+            }
+            if (f.bias) a = float4{a.x + bias_of[j].x, a.y + bias_of[j].y, a.z + bias_of[j].z, a.w + bias_of[j].w};
+            if (lds_at[j] >= 0) *reinterpret_cast<float4*>(s_row + lds_at[j]) = a;
+        }
+        for (int i = max(sum_thread, 0); i < HD / 2; i += sum_threads) {
+            if (i == sum_thread) s_cs[i] = angle;
+            else s_cs[i] = (reinterpret_cast<const float2*>(f.cos_sin) + static_cast<int64_t>(q_row0) * (HD / 2))[i];
+        }
+    };
 
     // ---- the item's queries: B operands, kept for the whole item
     bool rvalid[NT];
@@ -117,12 +248,14 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
         rtok[nt] = tq;
         rhead[nt] = h_base + hh;
         rpos[nt] = pos0 + tq;
-        const bf16_t* qp = q + static_cast<int64_t>(q_row0 + (rvalid[nt] ? tq : 0)) * q_stride +
-                           static_cast<int64_t>(rvalid[nt] ? rhead[nt] : h_base) * HD;
+        if constexpr (!QKV) {
+            const bf16_t* qp = q + static_cast<int64_t>(q_row0 + (rvalid[nt] ? tq : 0)) * q_stride +
+                               static_cast<int64_t>(rvalid[nt] ? rhead[nt] : h_base) * HD;
 #pragma unroll
-        for (int s = 0; s < S32; ++s) qf[nt][s].raw = ld16(qp + s * 32 + 8 * G);  // a row that does not exist reads
+            for (int s = 0; s < S32; ++s) qf[nt][s].raw = ld16(qp + s * 32 + 8 * G);  // a row that does not exist reads
 #pragma unroll
-        for (int s = 0; s < S16; ++s) qt[nt][s].raw = ld8(qp + s * 16 + 4 * G);   // the item's first row: masked later
+            for (int s = 0; s < S16; ++s) qt[nt][s].raw = ld8(qp + s * 16 + 4 * G);   // the item's first row: masked later
+        }
     }
 
     float m_run[NT], l_run[NT];
@@ -134,6 +267,13 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
 #pragma unroll
         for (int dt = 0; dt < HDT; ++dt) acc[nt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
+
+    // QKV: the queries (one token: row c of the tile is head c of the group) from the heads in LDS
+    auto build_queries = [&]() {
+        const float* head = s_row + (rvalid[0] ? c : 0) * RS;
+#pragma unroll
+        for (int s = 0; s < S32; ++s) qf[0][s].raw = rotated8<HD>(head, s_cs, s * 32 + 8 * G);
+    };
 
     const int64_t head_stride = static_cast<int64_t>(page_size) * HD;  // one kv head of one page
     // key / page_size as one multiplication (the host has checked that keys * page_size < 2^32): a
@@ -291,25 +431,92 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
     // one for the data, where fetching a block ahead costs a trip per block (8.0 -> 7.3 us a layer for
     // eight requests of 640 keys).
     constexpr bool ALL_AHEAD = PREFETCH && MAXW == 1;
+    // QKV: the new key and value, from the sums: a block of their own whose first key they are (the
+    // mask hides the rest), and into the pools for the steps to come.  The first wave does it before
+    // its walk, while its first keys from the cache are under way.
+    auto score_new_key = [&]() {
+        if (!(owner && wave == 0)) return;
+        key_end = pos0 + 1;
+        const float* kh = s_row + gh_here * RS;
+        const float* vh = kh + RS;
+        Block nb;
+#pragma unroll
+        for (int s = 0; s < S32; ++s) {
+            const uint4 r = rotated8<HD>(kh, s_cs, s * 32 + 8 * G);
+            nb.kf[0][s].raw = c == 0 ? r : uint4{0u, 0u, 0u, 0u};
+            nb.kf[1][s].raw = uint4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int dt = 0; dt < HDT; ++dt)
+            nb.vf[dt].raw = uint4{G == 0 ? pack2_bf16(vh[dt * 16 + c], 0.f) : 0u, 0u, 0u, 0u};
+        compute_block(pos0, nb);
+        key_end = pos0;
+        if (chunk == 0 && new_slot >= 0 && new_slot < f.pool_slots) {
+            const int page = new_slot / page_size;
+            const int off = new_slot - page * page_size;
+            bf16_t* kd = f.k_out + ((static_cast<int64_t>(page) * n_kv + kvh) * page_size + off) * HD;
+            for (int d = 2 * lane; d < HD; d += 128)
+                *reinterpret_cast<uint32_t*>(kd + d) = pack2_bf16(rotated<HD>(kh, s_cs, d), rotated<HD>(kh, s_cs, d + 1));
+            bf16_t* vd = f.v_out + (static_cast<int64_t>(page) * n_kv + kvh) * head_stride + off;
+            for (int d = lane; d < HD; d += 64) vd[static_cast<int64_t>(d) * page_size] = from_float<bf16_t>(vh[d]);
+        }
+    };
+
+    // QKV: the block table (warm in the L2) is read first, then the reads of the sums (which come from
+    // further away) and of the first keys go out together; the queries are built from LDS while the keys
+    // are under way
     if constexpr (ALL_AHEAD) {
-        for (int kb0 = kb_begin; kb0 < kb_end; kb0 += 4 * 32) {
-            Where at[4];
-            Block blk[4];
+        Where at[4];
+        Block blk[4];
+        auto locate4 = [&](int kb0) {
 #pragma unroll
             for (int d = 0; d < 4; ++d) locate(kb0 + 32 * d, at[d]);  // past the end: page 0, masked below
+        };
+        auto load4 = [&]() {
 #pragma unroll
             for (int d = 0; d < 4; ++d) load_block(at[d], blk[d]);
+        };
+        const bool any = !helper && kb_begin < kb_end;
+        if (any) locate4(kb_begin);
+        if (any) load4();
+        if constexpr (QKV) {
+            if (sums_here) {
+                issue_sums();
+                finish_sums();
+            }
+            __syncthreads();
+            if (helper) return;
+            build_queries();
+            score_new_key();
+        }
+        for (int kb0 = kb_begin; kb0 < kb_end; kb0 += 4 * 32) {
+            if (kb0 > kb_begin) {
+                locate4(kb0);
+                load4();
+            }
 #pragma unroll
             for (int d = 0; d < 4; ++d)
                 if (kb0 + 32 * d < kb_end) compute_block(kb0 + 32 * d, blk[d]);
         }
-    } else if (kb_begin < kb_end) {
+    } else {
+        const bool any = !helper && kb_begin < kb_end;
         Where at;
-        locate(kb_begin, at);
-        if (PREFETCH) {
-            Block cur, nxt;
+        Block cur, nxt;
+        if (any) locate(kb_begin, at);
+        if constexpr (QKV)
+            if (sums_here) issue_sums();
+        if (PREFETCH && any) {
             load_block(at, cur);
             locate(kb_begin + 32, at);
+        }
+        if constexpr (QKV) {
+            if (sums_here) finish_sums();
+            __syncthreads();
+            if (helper) return;
+            build_queries();
+            score_new_key();
+        }
+        if (PREFETCH && any) {
             for (int kb = kb_begin; kb < kb_end; kb += 32) {
                 if (kb + 32 < kb_end) {
                     load_block(at, nxt);
@@ -318,12 +525,11 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
                 compute_block(kb, cur);
                 cur = nxt;
             }
-        } else {
+        } else if (any) {
             for (int kb = kb_begin; kb < kb_end; kb += 32) {
-                Block blk;
-                load_block(at, blk);
+                load_block(at, cur);
                 locate(kb + 32, at);
-                compute_block(kb, blk);
+                compute_block(kb, cur);
             }
         }
     }
@@ -342,7 +548,6 @@ __global__ __launch_bounds__(64 * MAXW) __attribute__((amdgpu_waves_per_eu(MAXW 
     }
     if (MAXW > 1 && n_waves > 1) {
         __shared__ float s_m[NT][MAXW][16], s_l[NT][MAXW][16];
-        __shared__ floatx4 s_o[(MAXW > 1 ? MAXW - 1 : 1) * NT * HDT * 64];
         if (G == 0) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -439,7 +644,7 @@ int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_po
     attention_mfma_kernel<HDT, NT, W, V><<<grid, THREADS, 0, stream>>>(                                              \
         static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), \
         block_tables, max_pages, items, static_cast<bf16_t*>(out), partials, n_heads, n_kv, page_size, window, scale, \
-        gh, head_chunks)
+        gh, head_chunks, QkvSums{})
     const bool v16 = page_size % 8 == 0;
     if (waves == 1) {
         if (v16) FSIE_ATTN_LAUNCH(1, 64, true);
@@ -452,6 +657,34 @@ int launch(const void* q, int64_t q_stride, const void* k_pool, const void* v_po
     FSIE_CHECK_LAUNCH("attention_mfma");
     return 0;
 }
+
+// The QKV variant: items of one token, head_dim a multiple of 32, page_size a multiple of 8.
+template <int HDT>
+int launch_qkv(const QkvSums& f, const void* k_pool, const void* v_pool, const int32_t* block_tables, int max_pages,
+               const int32_t* items, int n_items, void* out, float* partials, int n_heads, int n_kv, int page_size,
+               int window, float scale, int waves, hipStream_t stream) {
+    constexpr int MAXW = max_waves<HDT>();
+    const int group = n_heads / n_kv;
+    const int gh = group < 16 ? group : 16;
+    const int head_chunks = (group + gh - 1) / gh;
+    const dim3 grid(n_items, n_kv * head_chunks);
+    if (waves < 1) waves = 1;
+    if (waves > MAXW) waves = MAXW;
+#define FSIE_ATTN_LAUNCH(W, THREADS)                                                                                 \
+    attention_mfma_kernel<HDT, 1, W, true, true><<<grid, THREADS, 0, stream>>>(                                      \
+        nullptr, 0, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), block_tables, max_pages, \
+        items, static_cast<bf16_t*>(out), partials, n_heads, n_kv, page_size, window, scale, gh, head_chunks, f)
+    // one wave and three that only help with the sums; or all the waves the kernel has (those that an
+    // item's keys leave idle help with the sums too)
+    if (waves == 1) FSIE_ATTN_LAUNCH(1, 256);
+    else FSIE_ATTN_LAUNCH(MAXW, 64 * MAXW);
+#undef FSIE_ATTN_LAUNCH
+    FSIE_CHECK_LAUNCH("attention_mfma_qkv");
+    return 0;
+}
+
+typedef int (*LaunchQkvFn)(const QkvSums&, const void*, const void*, const int32_t*, int, const int32_t*, int, void*,
+                           float*, int, int, int, int, float, int, hipStream_t);
 
 typedef int (*LaunchFn)(const void*, int64_t, const void*, const void*, const int32_t*, int, const int32_t*, int, void*,
                         float*, int, int, int, int, float, int, hipStream_t);

@@ -562,6 +562,51 @@ def attention_mfma(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
     return out
 
 
+def attention_mfma_qkv_ok(head_dim: int, page_size: int) -> bool:
+    """Whether the attention kernel that finishes the q/k/v product itself takes this geometry."""
+    return bool(load().fsie_attention_mfma_qkv_ok(head_dim, page_size))
+
+
+def attention_mfma_qkv(sums: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: torch.Tensor, slots: torch.Tensor,
+                       k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor, items: torch.Tensor,
+                       n_items: int, out: torch.Tensor, partials: Optional[torch.Tensor], n_heads: int, n_kv: int,
+                       head_dim: int, window: Optional[int], scale: float, waves: int = 1) -> torch.Tensor:
+    """Attention of a step of one token a request (every item: one query row a head) from the q/k/v
+    product's float32 partial sums [S, T, (heads + 2 kv heads) head_dim]: the kernel adds them up, adds
+    ``bias``, rotates queries and keys by ``cos_sin`` [T, head_dim / 2, 2], scores each request's new key
+    from registers and writes it and the value to ``slots[t]`` of the pools (negative: nowhere)."""
+    width = (n_heads + 2 * n_kv) * head_dim
+    _need(sums, "q/k/v sums", dtype=torch.float32, ndim=3)
+    n_parts, t = sums.shape[0], sums.shape[1]
+    if sums.shape[2] != width or t < 1:
+        raise KernelError(f"q/k/v sums: shape {tuple(sums.shape)} does not hold rows of {width}")
+    if bias is not None:
+        _need(bias, "q/k/v bias", dtype=torch.float32, shape=(width,))
+    _need(cos_sin, "cos_sin", dtype=torch.float32)
+    if cos_sin.numel() != t * head_dim:
+        raise KernelError(f"cos_sin: {cos_sin.numel()} values for {t} tokens of head_dim {head_dim}")
+    _need(slots, "slots", dtype=torch.int32, shape=(t,))
+    _need(k_pool, "k_pool", dtype=torch.bfloat16, ndim=4)
+    _need(v_pool, "v_pool", dtype=torch.bfloat16,
+          shape=(k_pool.shape[0], k_pool.shape[1], k_pool.shape[3], k_pool.shape[2]))
+    _need(block_tables, "block_tables", dtype=torch.int32, ndim=2)
+    _need(items, "attention items", dtype=torch.int32, ndim=2)
+    if items.shape[1] != ATTN_ITEM_INTS or items.shape[0] < n_items:
+        raise KernelError(f"attention items: shape {tuple(items.shape)} does not hold {n_items} items")
+    _need(out, "attention out", dtype=torch.bfloat16, shape=(t, n_heads * head_dim))
+    pages, kvh, page_size, hd = k_pool.shape
+    if kvh != n_kv or hd != head_dim:
+        raise KernelError(f"k_pool: shape {tuple(k_pool.shape)} does not match kv heads {n_kv}, head_dim {head_dim}")
+    if partials is not None:
+        _need(partials, "attention partials", dtype=torch.float32, ndim=1)
+    check(load().fsie_attention_mfma_qkv(sums.data_ptr(), n_parts, t, _ptr(bias), cos_sin.data_ptr(), slots.data_ptr(),
+                                         k_pool.data_ptr(), v_pool.data_ptr(), pages * page_size,
+                                         block_tables.data_ptr(), block_tables.shape[1], items.data_ptr(), n_items,
+                                         out.data_ptr(), _ptr(partials), n_heads, n_kv, head_dim, page_size,
+                                         int(window or 0), float(scale), int(waves), _stream()))
+    return out
+
+
 def attention_mfma_lds_ok(head_dim: int, page_size: int) -> bool:
     """Whether the kernel that shares a block of keys among four waves takes this geometry."""
     return bool(load().fsie_attention_mfma_lds_ok(head_dim, page_size))

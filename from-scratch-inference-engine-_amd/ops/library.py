@@ -56,6 +56,9 @@ _SIGNATURES = {
                                c_int, c_int, c_float, c_int, _P], c_int),
     "fsie_attention_mfma": ([_P, c_int64, _P, _P, _P, c_int, _P, c_int, _P, _P, c_int, c_int, c_int,
                              c_int, c_int, c_float, c_int, c_int, _P], c_int),
+    "fsie_attention_mfma_qkv_ok": ([c_int, c_int], c_int),
+    "fsie_attention_mfma_qkv": ([_P, c_int, c_int, _P, _P, _P, _P, _P, c_int64, _P, c_int, _P, c_int, _P, _P, c_int,
+                                 c_int, c_int, c_int, c_int, c_float, c_int, _P], c_int),
     "fsie_attention_mfma_max_waves": ([c_int], c_int),
     "fsie_attention_mfma_lds_ok": ([c_int, c_int], c_int),
     "fsie_attention_mfma_lds": ([_P, c_int64, _P, _P, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int,

@@ -209,6 +209,7 @@ class AttentionPlanner:
             "groups": np.asarray(groups, dtype=np.int32).reshape(-1, 2), "n_groups": len(groups),
             "n_small": len(small), "n_large": len(large) - n_long, "n_long": n_long, "n_merges": len(merges),
             "n_partial": n_partial, "mfma": mfma, "waves": waves,
+            "single": all(host.q_lens[s] == 1 for s in range(host.n_seqs)),  # one token a request
         }
 
 
@@ -220,6 +221,9 @@ class GQAttention(Mixer):
     positions a query reads (None: all)."""
 
     share_keys = True  # long portions: four tiles of a request share each block of keys through LDS
+    # steps of one token a request: the attention kernel adds up the q/k/v product's partial sums,
+    # rotates and writes the cache itself (one launch fewer a layer)
+    finish_qkv_in_attention = True
 
     @property
     def graph_safe(self) -> bool:
@@ -268,7 +272,36 @@ class GQAttention(Mixer):
         return self._planner
 
     # compute ----------------------------------------------------------------------------
+    def _from_sums(self, x: torch.Tensor, ctx, cache, plan) -> Optional[torch.Tensor]:
+        """Attention of a step of one token a request straight from the q/k/v product's partial sums
+        (None: not such a step, or the kernels do not take the sizes)."""
+        if not (self.finish_qkv_in_attention and cache.writes and plan.mfma and plan.single and plan.n_small
+                and not plan.n_large and not plan.n_long and x.dtype == torch.bfloat16
+                and ops.attention_mfma_qkv_ok(self.head_dim, cache.page_size)):
+            return None
+        table = self.position.rotation_table(self.head_dim, ctx)
+        if table is None:
+            return None
+        sums = self.qkv.partial_sums(x, few_rows=True)
+        if sums is None:
+            return None
+        out = torch.empty((x.shape[0], self.q_dim), dtype=x.dtype, device=x.device)
+        partials = None
+        if plan.n_partial:
+            partials = torch.empty((plan.n_partial * self.n_heads * (self.head_dim + 2),), dtype=torch.float32,
+                                   device=x.device)
+        ops.attention_mfma_qkv(sums, self.qkv.bias, table, cache.slots, cache.k_pool, cache.v_pool,
+                               cache.block_tables, plan.items, plan.n_small, out, partials, self.n_heads, self.n_kv,
+                               self.head_dim, self.window, self.scale, waves=plan.waves)
+        if plan.n_merges:
+            ops.attention_merge(partials, plan.merges, plan.n_merges, out, self.n_heads, self.head_dim)
+        return out
+
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        plan = ctx.plan(self.planner())
+        out = self._from_sums(x, ctx, cache, plan)
+        if out is not None:
+            return self.o.for_residual(out, ctx)
         store = KVStore(cache.k_pool, cache.v_pool, cache.slots, cache.page_size) if cache.writes else None
         qkv = self.position.project(x, self.qkv.weight, self.qkv.bias, self.n_heads, self.n_kv, self.head_dim, ctx,
                                     store)
@@ -281,7 +314,6 @@ class GQAttention(Mixer):
         if qkv is None:
             qkv = self.qkv(x, skip_bias=True)
             self.position.apply(qkv, self.n_heads, self.n_kv, self.head_dim, ctx, store, bias=self.qkv.bias)
-        plan = ctx.plan(self.planner())
         t = x.shape[0]
         out = torch.empty((t, self.q_dim), dtype=x.dtype, device=x.device)
         partials = None

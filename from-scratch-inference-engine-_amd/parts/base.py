@@ -132,6 +132,12 @@ class PositionEncoding(Part):
         mixer then projects whole and calls ``apply``."""
         return None
 
+    def rotation_table(self, head_dim: int, ctx) -> Optional[torch.Tensor]:
+        """Optional: if this encoding is the rotation of the pairs (i, i + head_dim / 2) of every
+        q and k head by an angle per token and pair, the step's float32 table [T, head_dim / 2, 2]
+        of their cosines and sines, for a mixer whose own kernel rotates; else None."""
+        return None
+
 
 class Block(Part):
     kind = "block"

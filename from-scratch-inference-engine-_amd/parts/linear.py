@@ -140,14 +140,15 @@ class Linear:
                 return ops.gemm_mfma_skinny(x, self.weight, splits=splits)
         return self(x)
 
-    def partial_sums(self, x: torch.Tensor) -> Optional[torch.Tensor]:
+    def partial_sums(self, x: torch.Tensor, few_rows: bool = False) -> Optional[torch.Tensor]:
         """x . W^T (no bias) of 17 to 64 rows (to 128 from a fragment-ordered copy) as float32 partial sums [S, T, N] of slices of K, for a
         consumer that adds them up itself; None where the engine's kernel for that does not take the
         sizes (N = 4608, K = 3584 on MI355X at 64 rows: 12.4 us, the library's whole product 18.8;
         at 32 rows 9.1 against 13.6)."""
         m = x.shape[0]
         most = GEMM_MFMA_SKINNY_MAX_M if self.streamed is None else GEMM_MFMA_WIDE_MAX_M
-        if x.dtype != torch.bfloat16 or not GEMM_MFMA_SKINNY_BEST_M < m <= most:
+        least = 0 if few_rows else GEMM_MFMA_SKINNY_BEST_M  # (fewer rows: for a consumer that spares a launch by it)
+        if x.dtype != torch.bfloat16 or not least < m <= most:
             return None
         splits = self.wide_splits(m)
         if splits < 2 or not self.wide_takes(m, splits):

@@ -52,6 +52,9 @@ class RotaryEncoding(PositionEncoding):
             table = ctx.memo[key] = ops.rope_table(ctx.positions, self.inv_freq)
         return table
 
+    def rotation_table(self, head_dim, ctx):
+        return self.table(ctx) if self.rotary_dim == head_dim else None
+
     def apply(self, qkv, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore], bias=None) -> None:
         cos_sin = self.table(ctx) if self.rotary_dim == head_dim and head_dim % 8 == 0 else None
         if store is None:

@@ -457,6 +457,55 @@ def test_batches_of_17_to_64_rows_share_x_through_lds(tmp_path):
     assert 1 in used and len(used) > 1 and all(1 <= s <= 16 for s in used), calls  # logits whole, projections in slices
 
 
+def test_steps_of_one_token_a_request_finish_qkv_inside_attention(tmp_path, monkeypatch):
+    """Steps in which every request has one token hand the q/k/v product's partial sums to the
+    attention kernel, which adds them up, rotates, scores the new key and writes the cache itself:
+    1, 3 and 20 requests decoding, eagerly and through graphs, against the plain model; the tokens
+    such steps wrote are then read by a portion of several tokens; and with the switch off the same
+    steps give the same logits up to rounding through the kernels that do these one after the other."""
+    from from_scratch_inference_engine_amd import load_model, ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+    from from_scratch_inference_engine_amd.parts.attention import GQAttention
+
+    d = helpers.make_model_dir(tmp_path / "wide", WIDE, seed=13)
+    model = load_model(d, dtype="bfloat16")
+    fused, apart = [], []
+    real_qkv, real_rope, real_project = ops.attention_mfma_qkv, ops.rope_kv_write, ops.gemm_mfma_skinny_rope
+    monkeypatch.setattr(ops, "attention_mfma_qkv", lambda sums, *a, **k: (fused.append(sums.shape[:2]), real_qkv(sums, *a, **k))[1])
+    monkeypatch.setattr(ops, "rope_kv_write", lambda qkv, *a, **k: (apart.append(qkv.shape[0]), real_rope(qkv, *a, **k))[1])
+    monkeypatch.setattr(ops, "gemm_mfma_skinny_rope", lambda x, *a, **k: (apart.append(x.shape[0]), real_project(x, *a, **k))[1])
+    seqs = [helpers.token_ids(331, 40 + 3 * i, 700 + i) for i in range(20)]
+    ref = [plain.forward_dir(d, ids).numpy() for ids in seqs[:4]]
+    logits = {}
+    for on in (True, False):
+        monkeypatch.setattr(GQAttention, "finish_qkv_in_attention", on)
+        for graphs in (False, True):
+            for live in (1, 3, 20):
+                runner = Runner(model, page_size=16, num_pages=160, max_requests=24, use_graphs=graphs)
+                caches = [runner.manager.open(i) for i in range(live)]
+                n_pre = [len(ids) - 9 for ids in seqs[:live]]
+                runner.step([StepEntry(c, ids[:n], []) for c, ids, n in zip(caches, seqs, n_pre)])
+                fused.clear(), apart.clear()
+                for t in range(5):  # five tokens one by one ...
+                    out = runner.step([StepEntry(c, [ids[n + t]], [0]) for c, ids, n in zip(caches, seqs, n_pre)]).float().cpu()
+                    logits[(on, graphs, live, t)] = out
+                    for i in range(min(live, 4)):
+                        helpers.assert_close_to_plain(out[i:i + 1].numpy(), ref[i][n_pre[i] + t:n_pre[i] + t + 1], "bfloat16",
+                                                      f"in attention={on} graphs={graphs} {live} live, request {i} token {t}")
+                if not graphs:
+                    assert (len(fused) == 5 * 2 and not apart) if on else (len(apart) == 5 * 2 and not fused), (on, fused, apart)
+                    assert all(shape[1] == live and shape[0] >= 2 for shape in fused), fused
+                # ... then the last four of the first request together: they read what those steps wrote
+                out = runner.step([StepEntry(caches[0], seqs[0][n_pre[0] + 5:], [0, 1, 2, 3])]).float().cpu()
+                helpers.assert_close_to_plain(out.numpy(), ref[0][n_pre[0] + 5:], "bfloat16",
+                                              f"in attention={on} graphs={graphs} {live} live: four tokens after the decoded ones")
+    for (on, graphs, live, t), out in logits.items():
+        if on:
+            other = logits[(False, graphs, live, t)]
+            assert (out - other).abs().max() <= 2.0 ** -6 * other.abs().max(), (graphs, live, t)
+
+
 def test_decoding_from_fragment_ordered_copies(tmp_path, monkeypatch):
     """With the size from which a weight is kept a second time, in the order of the matrix
     instruction's fragments, set to zero, the small wide model keeps copies of every matrix whose

@@ -713,6 +713,88 @@ def test_attention_over_pages_at_the_lengths_that_are_timed(ops, heads, kv, seqs
         assert max(m[2] for m in plan["merges"]) > (64 if heads == 28 else 40)  # splits of the long decode
 
 
+@pytest.mark.parametrize("units", [4096, 8])  # items of 128 keys, one wave each, and a merge; whole requests, up to 8 waves
+@pytest.mark.parametrize("heads, kv, hd, page, window, n_parts, bias", [
+    (28, 4, 128, 16, None, 8, True),   # a large model's geometry
+    (40, 8, 128, 16, None, 4, True),
+    (14, 2, 64, 8, None, 3, True),
+    (20, 1, 32, 8, None, 1, False),    # more heads per kv head than rows of a block: two workgroups a kv head, one of them writes
+    (6, 3, 96, 24, None, 2, True),     # head size and page size no powers of two
+    (3, 1, 256, 64, None, 5, False),
+    (6, 2, 128, 16, 37, 7, True),      # a window
+])
+def test_attention_from_the_projections_partial_sums(ops, units, heads, kv, hd, page, window, n_parts, bias):
+    """A step of one token a request: the kernel that takes q/k/v as the partial sums of a product cut
+    along K (adds them up, adds the bias, rotates, scores the new key from registers, writes it and the
+    value into the pools) against the kernels that do these one after the other.  Positions at the
+    edges of pages, of the blocks of 32 keys and of the items of 128."""
+    from from_scratch_inference_engine_amd.parts.attention import AttentionPlanner
+
+    pasts = [0, 19, 31, 32, 600, 127, 128, 2500, 1023, 1024, 7, 255]
+    seqs = [(p, 1) for p in pasts]
+    t, width = len(seqs), (heads + 2 * kv) * hd
+    AttentionPlanner.compute_units = units
+    try:
+        case = paged_case(seqs, heads, kv, hd, page, torch.bfloat16, seed=heads + hd, window=window)
+    finally:
+        AttentionPlanner.compute_units = None
+    plan = case["plan"]
+    assert plan["mfma"] and plan["single"] and not plan["n_large"]
+    if window is None:
+        assert plan["n_merges"] > 0 if units == 4096 else plan["waves"] > 1
+    g = torch.Generator().manual_seed(5)
+    parts = torch.randn(n_parts, t, width, generator=g).cuda()
+    b = torch.randn(width, generator=g).cuda() if bias else None
+    positions = torch.tensor(pasts, dtype=torch.int32).cuda()
+    inv_freq = torch.pow(torch.tensor(1e4, dtype=torch.float64), -torch.arange(0, hd, 2, dtype=torch.float64) / hd).cuda()
+    table = ops.rope_table(positions, inv_freq)
+    tables = case["tables"]
+    slots = torch.tensor([int(tables[s, p // page]) * page + p % page for s, p in enumerate(pasts)], dtype=torch.int32).cuda()
+    items = torch.from_numpy(plan["items"]).cuda()
+    merges = torch.from_numpy(plan["merges"]).cuda()
+    scale = 1.0 / math.sqrt(hd)
+
+    def pools():
+        return case["k_pool"].cuda().clone(), case["v_pool"].cuda().clone(), tables.cuda()
+
+    # one after the other: the sums added and rotated into q and the pools, then attention over the pools
+    k1, v1, bt = pools()
+    qkv = torch.empty(t, width, dtype=torch.bfloat16).cuda()
+    ops.rope_kv_write(qkv, positions, heads, kv, hd, inv_freq, slots=slots, k_pool=k1, v_pool=v1, page_size=page, bias=b,
+                      cos_sin=table, parts=parts)
+    out1 = torch.zeros(t, heads * hd, dtype=torch.bfloat16).cuda()
+    partials1 = torch.zeros(max(plan["n_partial"], 1) * heads * (hd + 2)).cuda()
+    ops.attention_mfma(qkv, width, k1, v1, bt, items, plan["n_small"], out1, partials1, heads, kv, hd, window, scale, t,
+                       large=False, waves=plan["waves"])
+    # in one kernel
+    k2, v2, bt = pools()
+    out2 = torch.zeros(t, heads * hd, dtype=torch.bfloat16).cuda()
+    partials2 = torch.zeros_like(partials1)
+    assert ops.attention_mfma_qkv_ok(hd, page)
+    ops.attention_mfma_qkv(parts, b, table, slots, k2, v2, bt, items, plan["n_small"], out2, partials2, heads, kv, hd,
+                           window, scale, waves=plan["waves"])
+    if plan["n_merges"]:
+        ops.attention_merge(partials1, merges, plan["n_merges"], out1, heads, hd)
+        ops.attention_merge(partials2, merges, plan["n_merges"], out2, heads, hd)
+    torch.cuda.synchronize()
+    # the pools: the new keys and values are there (the rotation's roundings may differ in the last
+    # bit), and nothing else has changed
+    for new, old, start in ((k2, k1, case["k_pool"].cuda()), (v2, v1, case["v_pool"].cuda())):
+        assert (old != start).sum() >= t * kv * hd * 0.9
+        assert (new.float() - old.float()).abs().max() <= 2.0 ** -7 * old.float().abs().max()
+        assert torch.equal(new != start, old != start) or ((new != start) ^ (old != start)).sum() <= 4  # (a value that rounds to the stale one)
+    ref, got = out1.float(), out2.float()
+    assert ref.abs().max() > 0.1
+    for row in range(t):
+        err = (got[row] - ref[row]).abs().max().item()
+        assert err <= 2.0 ** -6 * ref[row].abs().max().item(), f"request of {pasts[row]} past keys: {err}"
+    with pytest.raises(ops.KernelError, match="multiple of 32"):
+        ops.attention_mfma_qkv(torch.zeros(1, 1, 3 * 48).cuda(), None, torch.zeros(1, 24, 2).cuda(), slots[:1],
+                               torch.zeros(2, 1, 8, 48, dtype=torch.bfloat16).cuda(),
+                               torch.zeros(2, 1, 48, 8, dtype=torch.bfloat16).cuda(), bt[:1], items, 1,
+                               torch.zeros(1, 48, dtype=torch.bfloat16).cuda(), None, 1, 1, 48, None, 1.0)
+
+
 @pytest.mark.parametrize("dtype, scalar", [(torch.float32, True), (torch.bfloat16, False)])
 def test_attention_finds_one_far_key_and_respects_edges(ops, dtype, scalar):
     """Inputs that random data would hide a fault behind: for every query one key far back (or
