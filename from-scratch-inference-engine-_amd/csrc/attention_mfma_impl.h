@@ -289,6 +289,10 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     constexpr int kBlocksPerWave = NT == 1 ? 4 : 16;
     const int n_active = min(n_waves, max(1, (n_blocks + kBlocksPerWave - 1) / kBlocksPerWave));
     const int per_wave = (n_blocks + n_active - 1) / n_active;
+    // QKV: the request's new key is a run of its own, for a wave that the keys of the cache leave
+    // idle if there is one (else for the first); n_runs = waves whose results are combined
+    const int new_key_wave = owner && n_active < n_waves ? n_active : 0;
+    const int n_runs = owner && n_active < n_waves ? n_active + 1 : n_active;
     const int kb_begin = kb_first + wave * per_wave * 32;
     const int kb_end = min(key_end, kb_begin + per_wave * 32);
     // the keys (A operand of the scores) and values (A operand of the second product) of a block
@@ -306,26 +310,35 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     struct Where {
         int64_t k[2], v[2];  // element offsets into the pools
     };
-    auto locate = [&](int kb, Where& at) {
+    struct Asked {
         int page[4], idx[4], key[4];
+    };
+    auto ask_pages = [&](int kb, Asked& p) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            key[t] = kb + 8 * (c >> 2) + 4 * t + (c & 3);
-            key[2 + t] = kb + 8 * G + 4 * t;
+            p.key[t] = kb + 8 * (c >> 2) + 4 * t + (c & 3);
+            p.key[2 + t] = kb + 8 * G + 4 * t;
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {  // the four table reads go out together
-            idx[i] = static_cast<int>(__umulhi(static_cast<uint32_t>(key[i]), page_magic));
-            page[i] = table[min(idx[i], max_pages - 1)];
+            p.idx[i] = static_cast<int>(__umulhi(static_cast<uint32_t>(p.key[i]), page_magic));
+            p.page[i] = table[min(p.idx[i], max_pages - 1)];
         }
+    };
+    auto place = [&](const Asked& p, Where& at) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const bool ok = key[i] < key_end && idx[i] < max_pages && page[i] >= 0;
-            const int64_t head = (static_cast<int64_t>(ok ? page[i] : 0) * n_kv + kvh) * head_stride;
-            const int off = ok ? key[i] - idx[i] * page_size : 0;
+            const bool ok = p.key[i] < key_end && p.idx[i] < max_pages && p.page[i] >= 0;
+            const int64_t head = (static_cast<int64_t>(ok ? p.page[i] : 0) * n_kv + kvh) * head_stride;
+            const int off = ok ? p.key[i] - p.idx[i] * page_size : 0;
             if (i < 2) at.k[i] = head + static_cast<int64_t>(off) * HD + (X32 ? 8 : 4) * G;
             else at.v[i - 2] = head + off + static_cast<int64_t>(c) * page_size;
         }
+    };
+    auto locate = [&](int kb, Where& at) {
+        Asked p;
+        ask_pages(kb, p);
+        place(p, at);
     };
     auto load_block = [&](const Where& at, Block& blk) {
 #pragma unroll
@@ -432,10 +445,10 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     // eight requests of 640 keys).
     constexpr bool ALL_AHEAD = PREFETCH && MAXW == 1;
     // QKV: the new key and value, from the sums: a block of their own whose first key they are (the
-    // mask hides the rest), and into the pools for the steps to come.  The first wave does it before
-    // its walk, while its first keys from the cache are under way.
+    // mask hides the rest), and into the pools for the steps to come.  An idle wave does it, or the
+    // first one before its walk, while its first keys from the cache are under way.
     auto score_new_key = [&]() {
-        if (!(owner && wave == 0)) return;
+        if (!(owner && wave == new_key_wave)) return;
         key_end = pos0 + 1;
         const float* kh = s_row + gh_here * RS;
         const float* vh = kh + RS;
@@ -502,9 +515,13 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
         const bool any = !helper && kb_begin < kb_end;
         Where at;
         Block cur, nxt;
-        if (any) locate(kb_begin, at);
+        // (QKV: the reads of the sums, which come from further away than the table, go out before the
+        // wait for the table)
+        Asked first;
+        if (any) ask_pages(kb_begin, first);
         if constexpr (QKV)
             if (sums_here) issue_sums();
+        if (any) place(first, at);
         if (PREFETCH && any) {
             load_block(at, cur);
             locate(kb_begin + 32, at);
@@ -559,9 +576,9 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             float m_all = -INFINITY;
-            for (int w = 0; w < n_active; ++w) m_all = fmaxf(m_all, s_m[nt][w][c]);
+            for (int w = 0; w < n_runs; ++w) m_all = fmaxf(m_all, s_m[nt][w][c]);
             float denom = 0.f;
-            for (int w = 0; w < n_active; ++w) {
+            for (int w = 0; w < n_runs; ++w) {
                 const float mw = s_m[nt][w][c];
                 if (mw != -INFINITY) denom += s_l[nt][w][c] * __builtin_amdgcn_exp2f(mw - m_all);
             }
@@ -573,7 +590,7 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
                 acc[nt][dt][2] *= mine;
                 acc[nt][dt][3] *= mine;
             }
-            if (wave > 0 && wave < n_active) {
+            if (wave > 0 && wave < n_runs) {
 #pragma unroll
                 for (int dt = 0; dt < HDT; ++dt) s_o[(((wave - 1) * NT + nt) * HDT + dt) * 64 + lane] = acc[nt][dt];
             }
@@ -582,7 +599,7 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
         }
         __syncthreads();
         if (wave > 0) return;
-        for (int w = 1; w < n_active; ++w) {
+        for (int w = 1; w < n_runs; ++w) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll

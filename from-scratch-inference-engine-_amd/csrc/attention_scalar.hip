@@ -255,44 +255,72 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __rest
     const int64_t rec_size = hd + 2;
     const float* rec0 = partials + (static_cast<int64_t>(first) * n_heads + hq) * rec_size;
     const int64_t rec_step = static_cast<int64_t>(stride) * n_heads * rec_size;
-    float m = -INFINITY;
-    for (int base = 0; base < n_splits; base += 64) {
-        const int s = base + lane;
-        m = fmaxf(m, s < n_splits ? rec0[s * rec_step + hd] : -INFINITY);
-    }
-    m = wave_max(m);
+    constexpr int AHEAD = 8;
     float denom = 0.f;  // summed in the order of the splits, as the accumulators are
     float a[DIMS];
 #pragma unroll
     for (int i = 0; i < DIMS; ++i) a[i] = 0.f;
-    for (int base = 0; base < n_splits; base += 64) {
-        const int s = base + lane;
-        float w = 0.f, l = 0.f;
-        if (s < n_splits) {
-            const float ms = rec0[s * rec_step + hd];
-            l = rec0[s * rec_step + hd + 1];
-            w = ms == -INFINITY ? 0.f : expf(ms - m);
+    if (n_splits <= AHEAD) {
+        // few splits (a decode step's usual case): maxima, denominators and sums are all asked for
+        // at once, one trip to memory instead of two; the arithmetic and its order are those of
+        // the general case below
+        const int s = min(lane, n_splits - 1);
+        const float ms = rec0[s * rec_step + hd];
+        const float l = rec0[s * rec_step + hd + 1];
+        float v[AHEAD][DIMS];
+#pragma unroll
+        for (int j = 0; j < AHEAD; ++j) {
+            const float* r = rec0 + min(j, n_splits - 1) * rec_step;
+#pragma unroll
+            for (int i = 0; i < DIMS; ++i) v[j][i] = r[min(lane + 64 * i, hd - 1)];
         }
-        const int here = min(64, n_splits - base);
-        const float* rec = rec0 + base * rec_step;
-        constexpr int AHEAD = 8;
-        for (int j0 = 0; j0 < here; j0 += AHEAD) {
-            float v[AHEAD][DIMS];
+        const float m = wave_max(lane < n_splits ? ms : -INFINITY);
+        const float w = (lane >= n_splits || ms == -INFINITY) ? 0.f : expf(ms - m);
 #pragma unroll
-            for (int j = 0; j < AHEAD; ++j) {  // a split past the end reads the last one again, with weight 0
-                const float* r = rec + min(j0 + j, here - 1) * rec_step;
+        for (int j = 0; j < AHEAD; ++j) {
+            const float wj = j < n_splits ? __shfl(w, j) : 0.f;
+            const float lj = __shfl(l, j);
+            if (wj != 0.f) {  // the same for the whole wave
+                denom += lj * wj;
 #pragma unroll
-                for (int i = 0; i < DIMS; ++i) v[j][i] = r[min(lane + 64 * i, hd - 1)];
+                for (int i = 0; i < DIMS; ++i) a[i] += v[j][i] * wj;
             }
+        }
+    } else {
+        float m = -INFINITY;
+        for (int base = 0; base < n_splits; base += 64) {
+            const int s = base + lane;
+            m = fmaxf(m, s < n_splits ? rec0[s * rec_step + hd] : -INFINITY);
+        }
+        m = wave_max(m);
+        for (int base = 0; base < n_splits; base += 64) {
+            const int s = base + lane;
+            float w = 0.f, l = 0.f;
+            if (s < n_splits) {
+                const float ms = rec0[s * rec_step + hd];
+                l = rec0[s * rec_step + hd + 1];
+                w = ms == -INFINITY ? 0.f : expf(ms - m);
+            }
+            const int here = min(64, n_splits - base);
+            const float* rec = rec0 + base * rec_step;
+            for (int j0 = 0; j0 < here; j0 += AHEAD) {
+                float v[AHEAD][DIMS];
 #pragma unroll
-            for (int j = 0; j < AHEAD; ++j) {
-                const int src = min(j0 + j, 63);
-                const float wj = j0 + j < here ? __shfl(w, src) : 0.f;
-                const float lj = __shfl(l, src);
-                if (wj != 0.f) {  // the same for the whole wave
-                    denom += lj * wj;
+                for (int j = 0; j < AHEAD; ++j) {  // a split past the end reads the last one again, with weight 0
+                    const float* r = rec + min(j0 + j, here - 1) * rec_step;
 #pragma unroll
-                    for (int i = 0; i < DIMS; ++i) a[i] += v[j][i] * wj;
+                    for (int i = 0; i < DIMS; ++i) v[j][i] = r[min(lane + 64 * i, hd - 1)];
+                }
+#pragma unroll
+                for (int j = 0; j < AHEAD; ++j) {
+                    const int src = min(j0 + j, 63);
+                    const float wj = j0 + j < here ? __shfl(w, src) : 0.f;
+                    const float lj = __shfl(l, src);
+                    if (wj != 0.f) {  // the same for the whole wave
+                        denom += lj * wj;
+#pragma unroll
+                        for (int i = 0; i < DIMS; ++i) a[i] += v[j][i] * wj;
+                    }
                 }
             }
         }
