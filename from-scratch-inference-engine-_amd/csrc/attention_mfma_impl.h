@@ -164,19 +164,23 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     // the QKV variant, the heads added up from the sums (up to 16 of queries, a key, a value) and
     // the cosines and sines
     constexpr int kCombine = MAXW > 1 ? (MAXW - 1) * NT * HDT * 64 : 0;
-    constexpr int RS = HD + 4;  // a head's row in LDS: four floats apart from a multiple of the banks, so that 16 rows read 16 bytes each without conflict
+    // a head's row in LDS is four floats longer than the head, so that the 16 rows that a wave reads
+    // at once, 16 bytes each, fall into different banks
+    constexpr int RS = HD + 4;
     constexpr int kHeads = QKV ? (18 * RS + HD) / 4 : 0;
     constexpr int kLds = kCombine > kHeads ? kCombine : (kHeads > 0 ? kHeads : 1);
     __shared__ floatx4 s_o[kLds];
     float* s_row = reinterpret_cast<float*>(s_o);
     float2* s_cs = reinterpret_cast<float2*>(s_row + 18 * RS);
     // The heads this workgroup needs, added up over the slices, with the bias, into LDS.  In two
-    // steps, so that the reads of the first slices (straight-line code: a slice past the last reads
-    // the last one again, a thread without a column reads column 0) are under way together with the
-    // first reads of the block table, and one trip to memory serves both.
-    // (the variant of one wave is launched with four: the other three add up the sums, so that the
-    // first has only its keys under way: the hardware counts 63 reads at most, and a wait for one of
-    // 27 reads of sums behind 64 of keys would wait for most of the keys too)
+    // steps: first all the reads of up to eight slices, in straight-line code (a slice past the last
+    // reads the last one again, a thread without a column reads column 0), so that they are under
+    // way together, and with the reads of the first keys where the same wave walks keys; then the
+    // additions.  A loop of one read and one addition a slice would be a trip to memory a slice.
+    // The variant of one wave is launched with four: the other three add up the sums and leave
+    // after the barrier, so that the first has only its keys under way.  The hardware counts 63
+    // reads of a wave at most, and a wait for one of 27 reads of sums behind 64 of keys would wait
+    // for most of the keys too.
     constexpr int kThreadsLeast = MAXW == 1 ? 192 : 64 * MAXW;  // threads that add up sums
     constexpr int NJ = QKV ? (18 * HD / 4 + kThreadsLeast - 1) / kThreadsLeast : 1;  // columns of four a thread
     constexpr int PC = NJ <= 3 ? 8 : 4;                                              // slices read at once
