@@ -60,6 +60,12 @@ union F8B {
 };
 
 __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+// the same as a streaming load: for data that is read once and whose whole lines one load of a wave covers
+__device__ __forceinline__ uint4 ld16_once(const bf16_t* p) {
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const u4 v = __builtin_nontemporal_load(reinterpret_cast<const u4*>(p));
+    return uint4{v[0], v[1], v[2], v[3]};
+}
 __device__ __forceinline__ uint2 ld8(const bf16_t* p) { return *reinterpret_cast<const uint2*>(p); }
 
 // What the QKV variant reads and writes beside the kernel's other operands.
@@ -356,7 +362,7 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
         const bf16_t* v0 = v_pool + at.v[0];
         if (V16) {
 #pragma unroll
-            for (int dt = 0; dt < HDT; ++dt) blk.vf[dt].raw = ld16(v0 + static_cast<int64_t>(dt * 16) * page_size);
+            for (int dt = 0; dt < HDT; ++dt) blk.vf[dt].raw = ld16_once(v0 + static_cast<int64_t>(dt * 16) * page_size);
         } else {
             const bf16_t* v1 = v_pool + at.v[1];
 #pragma unroll
