@@ -543,7 +543,8 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
             build_queries();
             score_new_key();
         }
-        if (PREFETCH && any) {
+        constexpr bool IN_TURN = QKV && MAXW <= 8;  // (16 waves a workgroup have 128 registers each: not enough)
+        if (PREFETCH && any && !IN_TURN) {
             for (int kb = kb_begin; kb < kb_end; kb += 32) {
                 if (kb + 32 < kb_end) {
                     load_block(at, nxt);
@@ -551,6 +552,27 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
                 }
                 compute_block(kb, cur);
                 cur = nxt;
+            }
+        } else if (PREFETCH && any) {
+            // two blocks in turn, each in registers of its own: while one is computed the other's
+            // data is under way (with one name for "this block" the copy from the next one's
+            // registers at the end of a pass waits for that data).  A per cent of a step with long
+            // contexts; the variants that would spill registers this way keep the loop above
+            for (int kb = kb_begin;;) {
+                if (kb + 32 < kb_end) {
+                    load_block(at, nxt);
+                    locate(kb + 64, at);
+                }
+                compute_block(kb, cur);
+                kb += 32;
+                if (kb >= kb_end) break;
+                if (kb + 32 < kb_end) {
+                    load_block(at, cur);
+                    locate(kb + 64, at);
+                }
+                compute_block(kb, nxt);
+                kb += 32;
+                if (kb >= kb_end) break;
             }
         } else if (any) {
             for (int kb = kb_begin; kb < kb_end; kb += 32) {
