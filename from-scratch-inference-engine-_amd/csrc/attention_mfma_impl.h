@@ -362,7 +362,11 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
         const bf16_t* v0 = v_pool + at.v[0];
         if (V16) {
 #pragma unroll
-            for (int dt = 0; dt < HDT; ++dt) blk.vf[dt].raw = ld16_once(v0 + static_cast<int64_t>(dt * 16) * page_size);
+            for (int dt = 0; dt < HDT; ++dt) {
+                // (streaming loads where several waves walk long runs of keys; the short items of one wave are slower with them)
+                const bf16_t* vp = v0 + static_cast<int64_t>(dt * 16) * page_size;
+                blk.vf[dt].raw = MAXW > 1 ? ld16_once(vp) : ld16(vp);
+            }
         } else {
             const bf16_t* v1 = v_pool + at.v[1];
 #pragma unroll
