@@ -717,6 +717,7 @@ def test_attention_over_pages_at_the_lengths_that_are_timed(ops, heads, kv, seqs
 @pytest.mark.parametrize("heads, kv, hd, page, window, n_parts, bias", [
     (28, 4, 128, 16, None, 8, True),   # a large model's geometry
     (40, 8, 128, 16, None, 4, True),
+    (12, 4, 128, 16, None, 11, True),  # more slices than the kernel reads at once
     (14, 2, 64, 8, None, 3, True),
     (20, 1, 32, 8, None, 1, False),    # more heads per kv head than rows of a block: two workgroups a kv head, one of them writes
     (6, 3, 96, 24, None, 2, True),     # head size and page size no powers of two
