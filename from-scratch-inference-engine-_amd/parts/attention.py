@@ -114,7 +114,31 @@ class AttentionPlanner:
         # 4.17 against 4.27), in three or more it is (8 requests in five: 3.55 against 3.60)
         if keys and split < longest and max(keys) <= longest and -(-max(keys) // split) <= 2:
             return longest
+        # Items of the matrix-core kernel may be longer: the waves of a workgroup deal an item's keys
+        # among themselves, and an item more for a request costs the work before the walk again and
+        # a merge.  Where the requests alone give every compute unit a workgroup they stay whole,
+        # however long (MI355X, a step of 64 requests at 28/4 heads of 128: 2,000 keys each 4.92 ms
+        # whole against 5.52 in items of 1,024, 3,500 keys 5.76 against 6.34; 64 requests of 1,040
+        # keys at 40/8 heads 15.8 against 17.6, where the second item had 16 keys).  Fewer requests
+        # take the longest items of which the full ones still number the units (8 requests of 16,000
+        # keys at 40/8 heads: 16.4 ms in items of 4,096 against 17.2); fewer workgroups than units lose
+        # (48 requests of 2,000 keys whole: 6.1 ms against 4.8).
+        if self.long_items and mfma and keys and split == longest and units > 0 and max(keys) > longest:
+            long = longest
+            while long < max(keys):
+                long *= 2
+            if len(keys) * per_item < units:
+                while long > longest and sum(max(1, k // long) for k in keys) * per_item < units:
+                    long //= 2
+            split = long
         return split
+
+    long_items = True  # items beyond the longest of `geometry` where they still fill the device
+
+    @staticmethod
+    def _items_of(keys: int, split_keys: int, longest: int) -> int:
+        """Items that the ``keys`` keys of a small portion are cut into: runs of ``split_keys``."""
+        return max(1, -(-keys // split_keys))
 
     def graph_bucket(self, host):
         """What a captured graph of this step's shape must fix: the number of (small) work items,
@@ -123,14 +147,18 @@ class AttentionPlanner:
         mfma = self.uses_mfma(host.compute_dtype, host.page_size)
         small_tokens = self.geometry(mfma)[0]
         split_keys = self.split_keys(host, mfma)
+        most = self.geometry(mfma)[2]
         n, longest = 0, 1
         for s in range(host.n_seqs):
             if host.q_lens[s] > small_tokens:
                 return None
             first_key = max(0, host.past_lens[s] - self.window + 1) if self.window else 0
             keys = host.past_lens[s] + host.q_lens[s] - first_key
-            longest = max(longest, min(keys, split_keys))
-            n += max(1, -(-keys // split_keys))
+            mine = self._items_of(keys, split_keys, most)
+            longest = max(longest, keys - (mine - 1) * split_keys)  # (the last item; the others have split_keys, if any)
+            if mine > 1:
+                longest = max(longest, split_keys)
+            n += mine
         if mfma:
             # items: a multiple of the number of requests, and of what 1,024 keys of each need, so
             # that a graph serves as many steps with short items as with long ones (the captured
@@ -143,7 +171,7 @@ class AttentionPlanner:
 
     def plan(self, host) -> Dict[str, object]:
         mfma = self.uses_mfma(host.compute_dtype, host.page_size)
-        small_tokens, large_tokens, _ = self.geometry(mfma)
+        small_tokens, large_tokens, most = self.geometry(mfma)
         padded = getattr(host, "pad", None) is not None
         split_keys = host.pad[self.key][2] if padded else self.split_keys(host, mfma)
         small, large, merges = [], [], []
@@ -152,12 +180,12 @@ class AttentionPlanner:
             n, p, row0 = host.q_lens[s], host.past_lens[s], host.q_starts[s]
             first_key = max(0, p - self.window + 1) if self.window else 0
             total = p + n
-            if n <= small_tokens and split_keys is not None and total - first_key > split_keys:
-                n_splits = -(-(total - first_key) // split_keys)
+            n_splits = self._items_of(total - first_key, split_keys, most) if split_keys is not None else 1
+            if n <= small_tokens and n_splits > 1:
                 base = n_partial
                 for i in range(n_splits):
                     kb = first_key + i * split_keys
-                    small.append((s, row0, n, p, kb, min(total, kb + split_keys), base + i * n, 0))
+                    small.append((s, row0, n, p, kb, total if i == n_splits - 1 else kb + split_keys, base + i * n, 0))
                 for t in range(n):
                     merges.append((row0 + t, base + t, n_splits, n))
                 n_partial += n_splits * n

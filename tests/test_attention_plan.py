@@ -133,6 +133,26 @@ def test_decode_items_shorten_while_compute_units_are_idle():
         assert plan["n_small"] == n_requests * -(-keys // split)
         assert plan["waves"] == {128: 1, 256: 2, 512: 4, 1024: 8}[split]  # one wave per 128 keys
         assert plan["n_merges"] == (n_requests if keys > split else 0)
+    # requests that by themselves give every unit a workgroup stay whole, however long: no item of 16 keys and no
+    # merge for requests that have just passed 1,024; fewer long requests take the longest items of which the
+    # full ones still number the units
+    for n_requests, keys, split, items in ((64, 1040, 2048, 1), (64, 3500, 4096, 1), (80, 2000, 2048, 1), (64, 16000, 16384, 1),
+                                           (48, 2000, 1024, 2), (48, 4100, 2048, 3), (32, 3500, 1024, 4), (16, 9000, 2048, 5)):
+        host = Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16)
+        assert planner.split_keys(host, True) == split
+        plan = planner.plan(host)
+        check_plan(planner, host, plan)
+        assert plan["n_small"] == n_requests * items and plan["waves"] == 8
+        assert plan["n_merges"] == (n_requests if items > 1 else 0)
+        bucket = planner.graph_bucket(host)
+        assert bucket[0] >= plan["n_small"] and bucket[1] == 8 and bucket[2] == split
+    wide = AttentionPlanner(40, 8, 128, None)
+    wide.compute_units = 256
+    for n_requests, keys, split in ((8, 16000, 2048), (8, 16500, 4096), (32, 2300, 4096), (16, 4000, 1024), (8, 640, 256)):
+        assert wide.split_keys(Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16), True) == split
+    planner.long_items = False
+    assert planner.split_keys(Host([(3499, 1)] * 64, 16, torch.bfloat16), True) == 1024
+    planner.long_items = True
     # the float32-arithmetic kernel: 256 keys an item on a full device, down to 64 (two passes of 32) on an idle one
     for n_requests, keys, split in ((1, 5000, 64), (8, 640, 64), (64, 640, 256), (4, 2000, 128), (16, 2000, 256)):
         host = Host([(keys - 1, 1)] * n_requests, 16, torch.float32)
