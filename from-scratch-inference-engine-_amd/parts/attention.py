@@ -127,6 +127,14 @@ class AttentionPlanner:
             long = longest
             while long < max(keys):
                 long *= 2
+            # (no item longer than the keys a unit gets when they are dealt evenly, as a power of two:
+            # one request of 100,000 keys among 63 short ones is cut, or its workgroups would run long
+            # after the others)
+            even = sum(keys) * per_item / units
+            most = longest
+            while most < even:
+                most *= 2
+            long = min(long, most)
             if len(keys) * per_item < units:
                 while long > longest and sum(max(1, k // long) for k in keys) * per_item < units:
                     long //= 2

@@ -146,6 +146,12 @@ def test_decode_items_shorten_while_compute_units_are_idle():
         assert plan["n_merges"] == (n_requests if items > 1 else 0)
         bucket = planner.graph_bucket(host)
         assert bucket[0] >= plan["n_small"] and bucket[1] == 8 and bucket[2] == split
+    # one very long request among short ones is cut, the short ones stay whole
+    host = Host([(599, 1)] * 63 + [(99999, 1)], 16, torch.bfloat16)
+    assert planner.split_keys(host, True) == 4096
+    plan = planner.plan(host)
+    check_plan(planner, host, plan)
+    assert plan["n_small"] == 63 + 25 and plan["n_merges"] == 1
     wide = AttentionPlanner(40, 8, 128, None)
     wide.compute_units = 256
     for n_requests, keys, split in ((8, 16000, 2048), (8, 16500, 4096), (32, 2300, 4096), (16, 4000, 1024), (8, 640, 256)):
