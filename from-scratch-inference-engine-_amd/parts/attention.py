@@ -121,7 +121,7 @@ class AttentionPlanner:
         # whole against 5.52 in items of 1,024, 3,500 keys 5.76 against 6.34; 64 requests of 1,040
         # keys at 40/8 heads 15.8 against 17.6, where the second item had 16 keys).  Fewer requests
         # take the longest items of which the full ones still number the units (8 requests of 16,000
-        # keys at 40/8 heads: 16.4 ms in items of 4,096 against 17.2); fewer workgroups than units lose
+        # keys at 40/8 heads: 16.6 ms in items of 2,048 against 17.2 in items of 1,024); fewer workgroups than units lose
         # (48 requests of 2,000 keys whole: 6.1 ms against 4.8).
         if self.long_items and mfma and keys and split == longest and units > 0 and max(keys) > longest:
             long = longest
