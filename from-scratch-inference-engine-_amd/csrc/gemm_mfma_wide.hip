@@ -403,6 +403,21 @@ extern "C" int fsie_gemm_mfma_wide_best_splits(int M, int N, int K) {
         const bool better = best == 1 || (fits && !best_fits) || (fits == best_fits && (fits ? groups >= best_groups : groups < best_groups));
         if (better) best = s, best_groups = groups, best_fits = fits;
     }
+    // The partial sums are bytes too: S * rows * N * 4, written and read again.  At four tiles of X
+    // they can weigh a quarter of the weights (N = 4608, K = 3584 in seven slices: 8.3 MB beside
+    // 33 MB): beyond a fifth, the fewest slices whose workgroups still number four fifths of the
+    // units (there three: a decode step of 64 requests at that shape 4.01 ms against 4.04; at two
+    // and three tiles seven slices stay faster, 3.51 against 3.58 ms at 32 rows, and at N = 7168,
+    // K = 5120 the sums of the rule's four slices are a tenth and the rule's choice the fastest).
+    if (mt == 4 && best > 2 && 4.0 * best * 64 * N > 0.2 * 2.0 * N * K) {
+        for (int s = 2; s < best; ++s) {
+            if (K / s < 512 || fsie_gemm_mfma_wide_slice(K, s) <= 0) continue;
+            int waves = 0, blocks = 0;
+            launch_shape(mt, N, s, waves, blocks);
+            const int rows = 16 * blocks * waves;
+            if (static_cast<int64_t>((N + rows - 1) / rows) * s * 5 >= static_cast<int64_t>(units) * 4) return s;
+        }
+    }
     return best;
 }
 
