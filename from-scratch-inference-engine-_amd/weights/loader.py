@@ -2,8 +2,9 @@
 
 An architecture describes what it expects as a list of ``ParamBinding``: "this parameter of
 this part is made of these checkpoint tensors (concatenated along dim 0), stored this way".
-The loader compares the expectation with the file, reports *all* missing and unexpected tensors
-and wrong shapes in one error, then fills the parts.
+The loader compares the expectation with the file, reports *all* missing and unexpected tensors,
+wrong shapes and wrong stored dtypes (a weight or vector stored as anything but 32- or 16-bit
+floating point, an integer table stored as floating point) in one error, then fills the parts.
 
 Storage on the device:
   * ``matrix``  - the run's compute dtype (bfloat16, or float32 in the 32-bit path);
@@ -25,11 +26,12 @@ from .safetensors_file import SafetensorsFile
 class WeightsError(RuntimeError):
     """The checkpoint does not hold what the architecture expects."""
 
-    def __init__(self, message: str, missing=(), unexpected=(), wrong_shape=()):
+    def __init__(self, message: str, missing=(), unexpected=(), wrong_shape=(), wrong_dtype=()):
         super().__init__(message)
         self.missing = list(missing)
         self.unexpected = list(unexpected)
         self.wrong_shape = list(wrong_shape)
+        self.wrong_dtype = list(wrong_dtype)
 
 
 @dataclass(frozen=True)
@@ -64,15 +66,42 @@ def expected_tensors(bindings: Sequence[ParamBinding]) -> Dict[str, TensorSpec]:
     return out
 
 
+# What a stored tensor may be for each kind of parameter.  Weights and vectors are numbers the
+# model computes with: 32-bit or 16-bit floating point, as the reference's container accepts
+# (include/engine/dtype.hpp:68-79 refuses every other dtype, tests/cpp/test_safetensors.cpp:100);
+# an integer, boolean or 64-bit tensor under a weight's name is a wrong file, not a value to cast.
+_STORED_AS = {
+    "matrix": (torch.float32, torch.float16, torch.bfloat16),
+    "vector": (torch.float32, torch.float16, torch.bfloat16),
+    "int_table": (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8),
+}
+
+
+def _dtype_name(dtype: torch.dtype) -> str:
+    return str(dtype).replace("torch.", "")
+
+
+def storage_of(bindings: Sequence[ParamBinding]) -> Dict[str, str]:
+    """Checkpoint tensor name -> storage kind of the parameter it goes into."""
+    return {s.name: b.storage for b in bindings for s in b.sources}
+
+
 def check_against(bindings: Sequence[ParamBinding], found: Dict[str, Tuple[int, ...]],
-                  ignore_unexpected: Sequence[str] = ()) -> None:
-    """Raise one ``WeightsError`` that lists everything wrong."""
+                  ignore_unexpected: Sequence[str] = (),
+                  found_dtypes: Optional[Dict[str, torch.dtype]] = None) -> None:
+    """Raise one ``WeightsError`` that lists everything wrong: missing and unexpected tensors,
+    wrong shapes and (where ``found_dtypes`` gives them) tensors stored in a dtype that their
+    parameter cannot mean."""
     expect = expected_tensors(bindings)
     missing = sorted(n for n in expect if n not in found)
     unexpected = sorted(n for n in found if n not in expect and n not in ignore_unexpected)
     wrong = sorted((n, expect[n].shape, tuple(found[n])) for n in expect
                    if n in found and tuple(found[n]) != tuple(expect[n].shape))
-    if not (missing or unexpected or wrong):
+    kinds = storage_of(bindings)
+    wrong_dtype = sorted((n, kinds[n], found_dtypes[n]) for n in expect
+                         if found_dtypes is not None and n in found_dtypes
+                         and found_dtypes[n] not in _STORED_AS[kinds[n]])
+    if not (missing or unexpected or wrong or wrong_dtype):
         return
     lines = ["checkpoint does not match the model:"]
     if missing:
@@ -84,7 +113,11 @@ def check_against(bindings: Sequence[ParamBinding], found: Dict[str, Tuple[int, 
     if wrong:
         lines.append(f"  wrong shapes ({len(wrong)}):")
         lines += [f"    {n}  expected {list(e)}, found {list(f)}" for n, e, f in wrong]
-    raise WeightsError("\n".join(lines), missing, unexpected, wrong)
+    if wrong_dtype:
+        lines.append(f"  wrong dtypes ({len(wrong_dtype)}):")
+        lines += [f"    {n}  stored as {_dtype_name(d)}, a {k.replace('_', ' ')} must be one of "
+                  f"{', '.join(_dtype_name(a) for a in _STORED_AS[k])}" for n, k, d in wrong_dtype]
+    raise WeightsError("\n".join(lines), missing, unexpected, wrong, wrong_dtype)
 
 
 def _to_storage(t: torch.Tensor, storage: str, compute_dtype: torch.dtype) -> torch.dtype:
@@ -110,8 +143,11 @@ def fill_parts(bindings: Sequence[ParamBinding], get_tensor, compute_dtype: torc
             pieces = []
             for s in b.sources:
                 t = get_tensor(s.name)
-                if b.storage == "int_table" and t.dtype.is_floating_point:
-                    raise WeightsError(f"tensor {s.name} must hold integers, found {t.dtype}")
+                if t.dtype not in _STORED_AS[b.storage]:
+                    # (a caller that did not go through check_against: the same refusal, one tensor)
+                    what = "must hold integers" if b.storage == "int_table" else "must hold 32- or 16-bit floating point"
+                    raise WeightsError(f"tensor {s.name} {what}, found {_dtype_name(t.dtype)}",
+                                       wrong_dtype=[(s.name, b.storage, t.dtype)])
                 pieces.append(t.to(device=device, dtype=target, non_blocking=False))
             if len(pieces) == 1:
                 value = pieces[0]
@@ -177,6 +213,9 @@ class CheckpointFiles:
     def shape(self, name: str):
         return self._where[name].shape(name)
 
+    def dtype(self, name: str) -> torch.dtype:
+        return self._where[name].dtype(name)
+
     def get(self, name: str) -> torch.Tensor:
         return self._where[name].get(name)
 
@@ -188,5 +227,6 @@ def load_weights(path, bindings: Sequence[ParamBinding], compute_dtype: torch.dt
     import os
 
     f = CheckpointFiles(path) if os.path.isdir(path) else SafetensorsFile(path)
-    check_against(bindings, {n: f.shape(n) for n in f.names()}, ignore_unexpected)
+    check_against(bindings, {n: f.shape(n) for n in f.names()}, ignore_unexpected,
+                  {n: f.dtype(n) for n in f.names()})
     return fill_parts(bindings, f.get, compute_dtype, device)

@@ -105,6 +105,42 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert piece in text
 
 
+def test_a_weight_stored_in_a_dtype_it_cannot_mean_is_refused(tmp_path):
+    """An integer, boolean or 64-bit tensor under a weight's name is a wrong file, not a value to
+    cast: the reference's container accepts F32, F16 and BF16 only (include/engine/dtype.hpp:68-79,
+    tests/cpp/test_safetensors.cpp:100).  The refusal comes with the other problems, in one error,
+    and before any parameter is set."""
+    cfg = helpers.TINY_A
+    tensors = helpers.random_tensors(cfg, 2)
+    tensors["model.layers.0.self_attn.q_proj.weight"] = torch.ones(64, 64, dtype=torch.int32)
+    tensors["model.layers.1.input_layernorm.weight"] = torch.ones(64, dtype=torch.bool)
+    tensors["model.layers.1.mlp.down_proj.weight"] = torch.zeros(64, 176, dtype=torch.float64)
+    tensors["model.layers.1.self_attn.v_proj.bias"] = torch.zeros(32, dtype=torch.float16)  # fine
+    del tensors["model.norm.weight"]
+    d = helpers.make_model_dir(tmp_path / "m", cfg, 2, tensors=tensors)
+    spec = _spec(cfg)
+    with pytest.raises(WeightsError) as err:
+        load_weights(d, spec.bindings, torch.bfloat16, "cpu", spec.ignore_unexpected)
+    e = err.value
+    assert e.missing == ["model.norm.weight"]
+    assert [(n, str(t)) for n, _, t in e.wrong_dtype] == [
+        ("model.layers.0.self_attn.q_proj.weight", "torch.int32"),
+        ("model.layers.1.input_layernorm.weight", "torch.bool"),
+        ("model.layers.1.mlp.down_proj.weight", "torch.float64")]
+    for piece in ("wrong dtypes (3)", "q_proj.weight  stored as int32", "input_layernorm.weight  stored as bool",
+                  "missing tensors (1)"):
+        assert piece in str(e), piece
+    assert all(getattr(p, a, None) is None for p in spec.all_parts() for a in p.param_decls()), "nothing was set"
+    # the same file with those three as they should be loads
+    good = helpers.random_tensors(cfg, 2)
+    good["model.layers.1.self_attn.v_proj.bias"] = torch.zeros(32, dtype=torch.float16)
+    load_weights(helpers.make_model_dir(tmp_path / "g", cfg, 2, tensors=good), spec.bindings, torch.bfloat16, "cpu",
+                 spec.ignore_unexpected)
+    # and a caller that fills parts without the check meets the same refusal, tensor by tensor
+    with pytest.raises(WeightsError, match="q_proj.weight must hold 32- or 16-bit floating point, found int32"):
+        fill_parts(_spec(cfg).bindings, lambda n: tensors.get(n, good[n]), torch.bfloat16, "cpu")
+
+
 def test_a_checkpoint_in_several_files_is_read_through_its_index(tmp_path):
     """Large checkpoints come as several safetensors files and model.safetensors.index.json; the
     folder loads to the same parameters as the single file, and an index that does not fit its
