@@ -345,12 +345,14 @@ def main() -> int:
     step_bytes = decode_bytes(cfg, layers, args.batch, mean_ctx, itemsize)
     achieved = step_bytes / (dt / args.steps) / 1e9
     print(f"[bench] decode batch {args.batch}: {dt / args.steps * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
-    points = {}
+    points, points_frac = {}, {}
     if not args.no_points:
         for b in (1, 64):
             k = min(args.steps, 64)
-            d, _ = decode(b, k, min(args.warmup, 16))
+            d, ctx_b = decode(b, k, min(args.warmup, 16))
             points[f"decode_b{b}"] = b * k / d
+            # the same roofline fraction as for the timed batch: bytes of a step / its time / the peak
+            points_frac[f"decode_b{b}"] = decode_bytes(cfg, layers, b, ctx_b, itemsize) / (d / k) / HBM_BYTES_PER_S
             print(f"[bench] decode batch {b}: {d / k * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
 
     kernels = {}
@@ -377,6 +379,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
                      "frac": achieved / (HBM_BYTES_PER_S / 1e9)},
         "points": points,
+        "points_roofline_frac": points_frac,
         "kernels": kernels,
     }
     print(json.dumps(line))

@@ -145,7 +145,11 @@ int fsie_attention_mfma_max_waves(int head_dim);
 // allocated or freed, here or in any routine called from here).  The caller passes the inputs, the
 // tables and the output as for those entry points; `n_partial_slots` is one more than the largest
 // partial slot that `items` and `merges` name (slot = one query token of one split); a step that
-// needs more than the buffer holds is refused with an error, never computed.  `mfma` != 0: the
+// needs more than the buffer holds is refused with an error, never computed.  The two tables lie in
+// device memory, which this call does not wait for: it runs the kernels on copies of them (kept in
+// the same buffer, behind the records, and counted against its size) in which an item or merge that
+// names a slot at or beyond `n_partial_slots` does nothing, so a wrong table leaves rows of `out`
+// unwritten and never reaches memory outside the buffer.  `mfma` != 0: the
 // matrix-core kernel (bfloat16), else the float32-arithmetic kernel.  Every call on a GPU uses
 // that GPU's one buffer, which keeps the last call's contents: calls that overlap on one GPU
 // (different streams, or threads) race; calls on one stream are ordered and safe.  Nothing needs

@@ -170,12 +170,13 @@ def mlp_block(x, w: dict, prefix: str) -> torch.Tensor:
     return linear(silu_mul(gate, up), w[f"{prefix}mlp.down_proj.weight"])
 
 
-def forward(cfg: dict, w: dict, ids) -> torch.Tensor:
+def forward(cfg: dict, w: dict, ids, rows=None) -> torch.Tensor:
     """Logits [S, vocab] of one whole sequence  (src/model/model.cpp:90-149).
 
     Per layer: x += attn(norm1(x)); x += mlp(norm2(x)).  Then the final norm and the LM head,
     which is lm_head.weight if that tensor exists and the embedding table otherwise
-    (src/model/model.cpp:144-148).
+    (src/model/model.cpp:144-148).  ``rows``: the positions whose logits are wanted (all by
+    default; a long sequence at a large vocabulary is asked for a few).
     """
     ids = list(ids)
     positions = list(range(len(ids)))
@@ -186,6 +187,8 @@ def forward(cfg: dict, w: dict, ids) -> torch.Tensor:
         x = x + attention_block(normed, w, p, cfg, positions)
         normed2 = rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg["rms_norm_eps"])
         x = x + mlp_block(normed2, w, p)
+    if rows is not None:
+        x = x[torch.as_tensor(list(rows), dtype=torch.int64)]
     normed = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
     head = w["lm_head.weight"] if "lm_head.weight" in w else w["model.embed_tokens.weight"]
     return linear(normed, head)

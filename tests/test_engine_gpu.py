@@ -157,6 +157,38 @@ def test_small_pool_preempts_and_still_matches(model_dirs):
         engine.add_request([1, 256], max_tokens=2)
 
 
+def test_a_preempted_request_draws_the_same_samples_again(model_dirs):
+    """Temperature 0.7 in a pool so small that requests are preempted and recomputed: every
+    request's tokens are those of a pool that never preempts.  A draw belongs to (seed, request,
+    token index), so the recomputed request meets the same uniform numbers at the same places; a
+    generator shared by the batch, or one that counts draws, would give other tokens here."""
+    from from_scratch_inference_engine_amd import Engine, SamplingParams, SeqStatus, load_model
+
+    model = load_model(model_dirs["A"], dtype="float32")
+    prompts = [helpers.token_ids(256, n, 70 + n) for n in (4, 4, 7, 3)]
+    params = SamplingParams(temperature=0.7)
+
+    def run(num_blocks, seed=3):
+        engine = Engine(model, block_size=4, num_blocks=num_blocks, seed=seed, max_batch=4, max_tokens_per_step=8)
+        ids = [engine.add_request(p, params, max_tokens=9) for p in prompts]
+        steps = 0
+        while engine.has_work():
+            engine.step()
+            steps += 1
+            assert steps < 400
+        assert all(engine.status(i) == SeqStatus.Finished for i in ids)
+        assert engine.free_blocks() == num_blocks
+        return [engine.output(i) for i in ids], engine.preemptions()
+
+    roomy, none = run(64)
+    tight, some = run(6)
+    assert none == 0 and some > 0
+    assert tight == roomy
+    assert run(64, seed=4)[0] != roomy                      # the draws do depend on the seed
+    greedy = Engine(model, block_size=4, num_blocks=64, max_batch=4, max_tokens_per_step=8)
+    assert greedy.generate_batch(prompts, SamplingParams(temperature=0.0), max_tokens=9) != roomy  # and are draws
+
+
 def test_temperature_sampling_is_reproducible_and_independent_of_the_batch(llms):
     """Two engines with the same seed: all requests at once in one, one at a time in the other.
     Draws belong to (seed, request, token index), so the outputs are the same."""
@@ -239,7 +271,8 @@ def test_bench_prints_its_line():
     assert rec["config"]["streamed_weight_copies"] is True and rec["config"]["library_gemm_tuning"] is True
     assert rec["prefill"]["tokens"] == 2048 and 0 < rec["prefill"]["frac"] < 1
     assert rec["roofline"]["bound"] == "hbm" and rec["roofline"]["peak"] == 8000.0 and 0 < rec["roofline"]["frac"] < 1
-    assert set(rec["points"]) == {"decode_b1", "decode_b64"}
+    assert set(rec["points"]) == {"decode_b1", "decode_b64"} == set(rec["points_roofline_frac"])
+    assert all(0 < f < 1 for f in rec["points_roofline_frac"].values())
     assert {"attention", "qkv", "gate_up", "down", "o", "norms", "lm_head"} <= set(rec["kernels"])
     assert all(v["ms"] > 0 and v["launches"] > 0 for v in rec["kernels"].values())
     two = subprocess.run(cmd[:2] + ["--gpus", "2"], capture_output=True, text=True, timeout=120, cwd=str(helpers.ROOT))

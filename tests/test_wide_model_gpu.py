@@ -18,7 +18,14 @@ when its activations are rounded to bfloat16 where the engine rounds them, and i
 plain token wherever that one leads by more than twice the largest difference.  Decode batches
 of 32, 64, 80, 100, 128 and 140 through replayed graphs (rows of 32, 64, 80, 112, 128 and 160: the engine's
 own products up to 128 rows, beyond that the library's, its kernels chosen by timing) are checked against
-the plain logits in the same way.
+the plain logits in the same way.  One step of 2,048 tokens with the library's kernels chosen by
+timing (what the prefill measurement runs) is held to the same bound at 24 of its rows, and
+``Engine.generate_batch`` (scheduler, one step ahead, graphs, sampling on the device) must give the
+plain greedy tokens in float32 up to the first place where the plain choice is not clear.
+
+The same at the layer sizes of Qwen2.5-14B and -32B (hidden 5120, 40 query and 8 key/value heads of
+128, so five heads a group, intermediate 13824, eps 1e-5; two layers, named here): the families
+that decode and mix, in both precisions.
 """
 
 import json
@@ -39,11 +46,14 @@ WIDE = {
     "intermediate_size": 18944, "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
     "tie_word_embeddings": False, "max_position_embeddings": 4096, "use_sliding_window": False,
 }
+LAYERS_14B = 2  # of the 48 that the 14B shape has
+WIDE_14B = dict(WIDE, hidden_size=5120, num_hidden_layers=LAYERS_14B, num_attention_heads=40, num_key_value_heads=8,
+                intermediate_size=13824, rms_norm_eps=1e-5, max_position_embeddings=8192)
 LENGTHS = [330, 301, 77]
 PORTIONS = [7, 2, 16, 3, 2, 33, 5, 2, 64, 9, 130]
 
 
-def _rounded_plain(cfg, w, ids):
+def _rounded_plain(cfg, w, ids, rows=None):
     """The plain model with its activations rounded to bfloat16 where the bfloat16 engine rounds
     them: the inputs of every product, q and k after the rotation, the gated activation."""
     r16 = lambda t: t.to(torch.bfloat16).float()
@@ -52,41 +62,81 @@ def _rounded_plain(cfg, w, ids):
     plain.rope = lambda *a, **k: r16(rope(*a, **k))
     plain.silu_mul = lambda g, u: r16(silu(r16(g), r16(u)))
     try:
-        return plain.forward(cfg, w, ids)
+        return plain.forward(cfg, w, ids, rows=rows)
     finally:
         plain.linear, plain.rope, plain.silu_mul = lin, rope, silu
 
 
-@pytest.fixture(scope="module")
-def wide(tmp_path_factory):
-    """The model folder (bfloat16 values, drawn on the device by the test's own generator, so
-    that both precisions and the plain side read the same numbers) and the plain logits."""
+def _write_model(folder, raw, seed):
+    """bfloat16 values, drawn on the device by the test's own generator, so that both precisions
+    and the plain side read the same numbers."""
     from safetensors.torch import save_file
 
-    d = tmp_path_factory.mktemp("wide7b")
-    (d / "config.json").write_text(json.dumps(WIDE))
-    g = torch.Generator(device="cuda").manual_seed(11)
+    (folder / "config.json").write_text(json.dumps(raw))
+    g = torch.Generator(device="cuda").manual_seed(seed)
     tensors = {}
-    for name, shape in sorted(helpers.expected_tensor_shapes(WIDE).items()):
+    for name, shape in sorted(helpers.expected_tensor_shapes(raw).items()):
         t = torch.randn(shape, generator=g, device="cuda") * 0.02
         if name.endswith("norm.weight") or name.endswith("layernorm.weight"):
             t = t + 1.0
         tensors[name] = t.to(torch.bfloat16).cpu()
-    save_file(tensors, str(d / "model.safetensors"))
-    del tensors
-    print("wide model written", flush=True)
+    save_file(tensors, str(folder / "model.safetensors"))
+
+
+def _plain_side(d, raw):
     cfg, w = plain.read_config(d), plain.read_weights(d)
-    prompts = [helpers.token_ids(WIDE["vocab_size"], n, 4000 + n) for n in LENGTHS]
+    prompts = [helpers.token_ids(raw["vocab_size"], n, 4000 + n) for n in LENGTHS]
     ref = [plain.forward(cfg, w, p) for p in prompts]
     print("plain logits done", flush=True)
     moved = [(_rounded_plain(cfg, w, p) - r) for p, r in zip(prompts, ref)]
     noise = [(m.abs().max().item(), m.pow(2).mean().sqrt().item()) for m in moved]
-    # short prompts of the decode batches (graphs): the first eight are compared with the plain model
-    short = [helpers.token_ids(WIDE["vocab_size"], 20 + i % 7 + 12, 5000 + i) for i in range(140)]
-    short_ref = [plain.forward(cfg, w, p) for p in short[:8]]
-    del w, moved
     print("rounded plain logits done", flush=True)
-    return {"dir": d, "prompts": prompts, "ref": ref, "noise": noise, "short": short, "short_ref": short_ref}
+    return cfg, w, {"dir": d, "prompts": prompts, "ref": ref, "noise": noise}
+
+
+@pytest.fixture(scope="module")
+def wide(tmp_path_factory):
+    """The model folder at 7B widths and the plain logits."""
+    d = tmp_path_factory.mktemp("wide7b")
+    _write_model(d, WIDE, 11)
+    print("wide model written", flush=True)
+    cfg, w, out = _plain_side(d, WIDE)
+    # short prompts of the decode batches (graphs): the first eight are compared with the plain model
+    out["short"] = [helpers.token_ids(WIDE["vocab_size"], 20 + i % 7 + 12, 5000 + i) for i in range(140)]
+    out["short_ref"] = [plain.forward(cfg, w, p) for p in out["short"][:8]]
+    # one prompt of 2,048 tokens, its plain logits at 24 places and what rounding alone moves there
+    long_ids = helpers.token_ids(WIDE["vocab_size"], 2048, 6000)
+    rows = sorted({0, 1, 15, 16, 17, 255, 256, 1023, 1024, 2046, 2047} | set(range(100, 2048, 150)))
+    long_ref = plain.forward(cfg, w, long_ids, rows=rows)
+    moved = _rounded_plain(cfg, w, long_ids, rows=rows) - long_ref
+    out["long"] = {"ids": long_ids, "rows": rows, "ref": long_ref,
+                   "noise": (moved.abs().max().item(), moved.pow(2).mean().sqrt().item())}
+    print("plain logits of the 2,048-token prompt done", flush=True)
+    # greedy continuations of three short prompts, with the lead of every chosen token
+    greedy = []
+    for p in out["short"][:3]:
+        ids, toks, leads = list(p), [], []
+        for _ in range(12):
+            last = plain.forward(cfg, w, ids, rows=[len(ids) - 1])[0]
+            top2 = last.topk(2)
+            toks.append(int(top2.indices[0]))
+            leads.append(float(top2.values[0] - top2.values[1]))
+            ids.append(toks[-1])
+        greedy.append((toks, leads))
+    out["greedy"] = greedy
+    print("plain greedy continuations done", flush=True)
+    del w
+    return out
+
+
+@pytest.fixture(scope="module")
+def wide_14b(tmp_path_factory):
+    d = tmp_path_factory.mktemp("wide14b")
+    _write_model(d, WIDE_14B, 12)
+    print("14B-geometry model written", flush=True)
+    _, w, out = _plain_side(d, WIDE_14B)
+    del w
+    return out
 
 
 def _plans():
@@ -229,3 +279,89 @@ def test_bfloat16_families_and_graph_batches_at_7b_widths(wide):
     # and eight tiles of rows over the fragment-ordered weights; 160 rows are the library's
     assert {("gate/up", r) for r in (80, 112, 128)} | {("slices", r) for r in (80, 112, 128)} <= own_rows, own_rows
     assert not any(rows > 128 for _, rows in own_rows), own_rows
+
+
+def test_a_2048_token_step_with_the_librarys_timed_kernels_at_7b_widths(wide):
+    """What the prefill measurement runs: one step of 2,048 tokens in bfloat16 with the library's
+    kernels chosen by timing, against the plain logits at 24 places (the first and last tokens, the
+    edges of pages and of the kernels' tiles, and places in between)."""
+    from from_scratch_inference_engine_amd import ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Model, Runner
+
+    long = wide["long"]
+    model = Model.from_pretrained(wide["dir"], dtype="bfloat16")
+    runner = Runner(model, page_size=16, num_pages=2048 // 16 + 40, max_requests=4)
+    ops.enable_library_tuning(max_ms_per_candidate=5, iterations=2)
+    try:
+        for attempt in ("first (the library times its kernels)", "second (the kernels it kept)"):
+            rc = runner.manager.open(attempt)
+            got = runner.step([StepEntry(rc, long["ids"], long["rows"])]).float().cpu()
+            runner.manager.close(rc)
+            ratio = _assert_within_rounding(got, long["ref"], long["noise"], f"2,048-token step, {attempt}")
+            print(f"2,048-token step, {attempt}: difference / rounding noise {ratio[0]:.2f} (max), {ratio[1]:.2f} (rms)")
+    finally:
+        ops.disable_library_tuning()
+    # the same prompt in two portions of 1,024 beside a decoding request, without timing: same bound
+    rc, other = runner.manager.open("portions"), runner.manager.open("other")
+    short = wide["short"][0]
+    runner.step([StepEntry(other, short[:-1], [])])
+    rows = long["rows"]
+    first = runner.step([StepEntry(rc, long["ids"][:1024], [r for r in rows if r < 1024])]).float().cpu()
+    both = runner.step([StepEntry(other, short[-1:], [0]),
+                        StepEntry(rc, long["ids"][1024:], [r - 1024 for r in rows if r >= 1024])]).float().cpu()
+    _assert_within_rounding(torch.cat([first, both[1:]]), long["ref"], long["noise"], "2,048 tokens in two portions")
+    _assert_within_rounding(both[:1], wide["short_ref"][0][-1:], long["noise"], "the token decoded beside a portion")
+
+
+def test_engine_generates_the_plain_greedy_tokens_at_7b_widths(wide, monkeypatch):
+    """tests/cpp/test_cuda_engine.cpp:45-79 at real widths: the engine (scheduler, one step ahead,
+    graphs from the third step of a shape on, argmax over 152,064 logits on the device) in float32
+    against greedy decoding by repeated whole forwards of the plain model.  A request is compared up
+    to the first token whose plain lead over the runner-up is not clear."""
+    from from_scratch_inference_engine_amd import Engine, SamplingParams
+    from from_scratch_inference_engine_amd.engine import graphs
+    from from_scratch_inference_engine_amd.engine.model import Model
+
+    monkeypatch.setattr(graphs, "CAPTURE_AFTER", 3)  # the engine's own: eager steps, a capture, replays
+    model = Model.from_pretrained(wide["dir"], dtype="float32")
+    prompts = wide["short"][:3]
+    for run_ahead in (True, False):
+        engine = Engine(model, block_size=16, num_blocks=24, max_batch=4, max_tokens_per_step=64)
+        engine.run_ahead = run_ahead
+        got = engine.generate_batch(prompts, SamplingParams(temperature=0.0), max_tokens=12)
+        compared = 0
+        for out, (toks, leads) in zip(got, wide["greedy"]):
+            assert len(out) == 12
+            clear = next((i for i, lead in enumerate(leads) if lead <= 4 * helpers.F32_ATOL), len(leads))
+            assert out[:clear] == toks[:clear], f"run_ahead={run_ahead}: {out} against plain {toks} (clear up to {clear})"
+            compared += clear
+        assert compared >= 24, f"only {compared} of 36 tokens had a clear plain choice"
+        if run_ahead:
+            assert engine.runner.graphs.replays > 0, "the decode steps were replayed from a graph"
+        assert engine.free_blocks() == 24
+    print(f"engine at 7B widths, float32: {compared} of 36 greedy tokens compared with plain")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_and_mixed_families_at_14b_widths(wide_14b, dtype):
+    from from_scratch_inference_engine_amd.engine.model import Model, Runner
+
+    model = Model.from_pretrained(wide_14b["dir"], dtype=dtype)
+    runner = Runner(model, page_size=16, num_pages=46, max_requests=4)
+    plans = _plans()
+    worst = 0.0
+    for family in ("decode", "mixed"):
+        for key, (i, logits) in _run(runner, wide_14b["prompts"], plans[family]).items():
+            ref = wide_14b["ref"][i]
+            assert logits.shape[0] == LENGTHS[i]
+            if dtype == "float32":
+                helpers.assert_close_to_plain(logits.numpy(), ref.numpy(), "float32", f"14B widths float32 {family} {key}")
+                worst = max(worst, float((logits - ref).abs().max()))
+            else:
+                r = _assert_within_rounding(logits, ref, wide_14b["noise"][i], f"14B widths bfloat16 {family} {key}")
+                worst = max(worst, r[0])
+    alloc = runner.manager.allocators[0]
+    assert len(alloc.pages_issued_again()) > alloc.num_pages // 2 and alloc.num_free == alloc.num_pages
+    print(f"{dtype} at 14B widths, {LAYERS_14B} layers: " +
+          (f"largest difference {worst:.3e}" if dtype == "float32" else f"difference / rounding noise {worst:.2f}"))
