@@ -166,7 +166,7 @@ def kernel_classes(runner, cfg, batch: int, prompt_len: int, itemsize: int) -> d
     return out
 
 
-def other_workload(args, cfg, model, shape_name, layers, full_layers, page) -> int:
+def other_workload(args, cfg, model, shape_name, layers, full_layers, page, fill_rows) -> int:
     """The two workloads beside the default run (many requests of mixed lengths through the
     scheduler; one long prompt in portions); one JSON line each."""
     import torch
@@ -182,7 +182,7 @@ def other_workload(args, cfg, model, shape_name, layers, full_layers, page) -> i
     if args.workload == "mixed":
         longest = args.max_prompt + args.outputs
         engine = Engine(model, block_size=page, num_blocks=args.requests * -(-longest // page) + 64,
-                        max_batch=args.requests, max_tokens_per_step=budget)
+                        max_batch=args.requests, max_tokens_per_step=budget, fill_rows=fill_rows)
         record = None
         # the same lengths in both passes: the first pays the graph captures and the library's kernel
         # selection for every step size they lead to, the second is measured
@@ -212,7 +212,7 @@ def other_workload(args, cfg, model, shape_name, layers, full_layers, page) -> i
         return 0
     n = args.prefill_tokens
     engine = Engine(model, block_size=page, num_blocks=-(-(n + 1) // page) + 64, max_batch=1,
-                    max_tokens_per_step=budget)
+                    max_tokens_per_step=budget, fill_rows=fill_rows)
     times = []
     for rep in range(3):
         prompt = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
@@ -267,8 +267,12 @@ def main() -> int:
     from from_scratch_inference_engine_amd.models import parse_config
     from from_scratch_inference_engine_amd.ops import enable_library_tuning
 
+    fill_rows = None
     if not args.no_tune and args.dtype == "bf16":
+        from from_scratch_inference_engine_amd.engine.context import padded_tokens
+
         enable_library_tuning()  # the first prefill times the library's kernels for its shapes
+        fill_rows = padded_tokens  # and steps that are not decode steps are filled up to the timed row counts
 
     shape_name, shape = SHAPES[args.shape]
     raw = dict(shape)
@@ -287,7 +291,7 @@ def main() -> int:
     page = 16
     context = raw["max_position_embeddings"]
     if args.workload != "decode":
-        return other_workload(args, cfg, model, shape_name, layers, full_layers, page)
+        return other_workload(args, cfg, model, shape_name, layers, full_layers, page, fill_rows)
     biggest = max(args.batch, 1 if args.no_points else 64)
     budget = 2048  # tokens a step may hold: the prompts of a large batch enter over several steps
     # requests whose prompt went in first decode while the others' prompts still enter: they get
@@ -295,7 +299,8 @@ def main() -> int:
     head_start = -(-biggest * args.prompt_len // budget) + 1
     per_req = args.prompt_len + args.steps + args.warmup + head_start + 2 * page
     num_blocks = max(biggest * -(-per_req // page), -(-2048 // page) * 2) + 64
-    engine = Engine(model, block_size=page, num_blocks=num_blocks, max_batch=biggest, max_tokens_per_step=budget)
+    engine = Engine(model, block_size=page, num_blocks=num_blocks, max_batch=biggest, max_tokens_per_step=budget,
+                    fill_rows=fill_rows)
     gen = torch.Generator().manual_seed(0)
 
     def prompts(n, length):

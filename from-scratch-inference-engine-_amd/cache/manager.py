@@ -48,6 +48,11 @@ class CacheManager:
             raise ValueError("CacheManager: max_requests must be positive")
         self.page_size = int(page_size)
         self.groups: List[CacheNeed] = list(paged_groups)
+        # per group: entries in a page and positions in an entry (a need may state its own)
+        self.entries_per_page = [int(getattr(n, "page_entries", None) or self.page_size) for n in self.groups]
+        self.tokens_per_entry = [int(getattr(n, "tokens_per_entry", 1) or 1) for n in self.groups]
+        if any(e < 1 for e in self.entries_per_page) or any(t < 1 for t in self.tokens_per_entry):
+            raise ValueError("CacheManager: a group's page_entries and tokens_per_entry must be positive")
         if isinstance(num_pages, int):
             num_pages = [num_pages] * len(self.groups)
         if len(num_pages) != len(self.groups):
@@ -95,8 +100,20 @@ class CacheManager:
         del self._live[rc.request_id]
 
     # ------------------------------------------------------------------ pages
-    def pages_for(self, tokens: int) -> int:
-        return -(-tokens // self.page_size)
+    def tokens_per_page(self, group: int = 0) -> int:
+        """Positions that one page of ``group`` holds."""
+        if not self.groups:
+            return self.page_size
+        return self.entries_per_page[group] * self.tokens_per_entry[group]
+
+    @property
+    def smallest_page_tokens(self) -> int:
+        """The positions of the smallest page of any group: between two multiples of it no group
+        needs a new page."""
+        return min([self.tokens_per_page(g) for g in range(len(self.groups))] or [self.page_size])
+
+    def pages_for(self, tokens: int, group: int = 0) -> int:
+        return -(-tokens // self.tokens_per_page(group))
 
     def free_pages(self, group: int = 0) -> int:
         return self.allocators[group].num_free
@@ -107,23 +124,22 @@ class CacheManager:
         window = self.groups[group].window
         if window is None:
             return 0
-        return max(0, length - window + 1) // self.page_size
+        return max(0, length - window + 1) // self.tokens_per_page(group)
 
     def new_pages_needed(self, rc: RequestCache, n_tokens: int) -> List[int]:
         """Pages each group must take from its pool to hold ``n_tokens`` more."""
-        target = self.pages_for(rc.length + n_tokens)
-        return [max(0, target - len(t)) for t in rc.tables]
+        return [max(0, self.pages_for(rc.length + n_tokens, g) - len(t)) for g, t in enumerate(rc.tables)]
 
     def max_pages_held(self, total_tokens: int, portion: int) -> List[int]:
         """Upper bound of pages a request of ``total_tokens`` holds at once per group when it is
         fed in portions of at most ``portion`` tokens."""
         out = []
-        for need in self.groups:
+        for g, need in enumerate(self.groups):
             if need.window is None:
-                out.append(self.pages_for(total_tokens))
+                out.append(self.pages_for(total_tokens, g))
             else:
-                span = min(total_tokens, need.window + portion + self.page_size)
-                out.append(min(self.pages_for(total_tokens), self.pages_for(span) + 1))
+                span = min(total_tokens, need.window + portion + self.tokens_per_page(g))
+                out.append(min(self.pages_for(total_tokens, g), self.pages_for(span, g) + 1))
         return out
 
     def can_reserve(self, items: Iterable[Tuple[RequestCache, int]]) -> bool:
@@ -159,7 +175,7 @@ class CacheManager:
         that no later query of a windowed group can read."""
         if rc.closed:
             raise RuntimeError(f"CacheManager: request {rc.request_id!r} is closed")
-        if rc.tables and rc.length + n_tokens > min(len(t) for t in rc.tables) * self.page_size:
+        if rc.tables and rc.length + n_tokens > min(len(t) * self.tokens_per_page(g) for g, t in enumerate(rc.tables)):
             raise RuntimeError("CacheManager: commit beyond the reserved pages")
         rc.length += n_tokens
         for g, table in enumerate(rc.tables):

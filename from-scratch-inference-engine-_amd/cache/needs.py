@@ -22,9 +22,11 @@ page where the rows that pad a batch read and write; the step's tables name unit
 per-request need: the slots + 1, the last one the spare slot):
 
   allocate(n_caches, units, page_size, device, dtype) -> store    anything the need likes
+      (``page_size``: the entries of a page of this need's group)
   view(store, plane, ctx, group, writes) -> what the mixer's ``forward`` gets as ``cache``;
-      ``ctx.block_tables[group]`` [requests, pages] and ``ctx.slots[group]`` [tokens] are the
-      step's tables of a per-token group, ``ctx.seq_slots`` [requests] the slots
+      ``ctx.block_tables[group]`` [requests, pages] and ``ctx.slots[group]`` [tokens] (the slot of
+      the entry that holds each token's position: unit * entries per page + entry in the page) are
+      the step's tables of a per-token group, ``ctx.seq_slots`` [requests] the slots
   bytes_per_token(dtype) -> int       per-token needs: for the measurement of cache traffic
   store_bytes(store) -> int
   reset(store, ctx)                   per-request needs: zero the slots ``ctx.reset_slots`` names
@@ -44,6 +46,13 @@ from typing import Optional, Tuple
 class CacheNeed:
     per_token: bool = True
     window: Optional[int] = None
+    # Per-token needs: how the positions of a request map to the entries of its pages.  One entry
+    # holds ``tokens_per_entry`` consecutive positions (1: an entry a token; k: a mixer that keeps
+    # one record per block of k tokens), and a page of this need's group has ``page_entries``
+    # entries (None: the page size the cache was made with).  The manager counts pages, and the
+    # step's tables name slots, by these numbers; groups with other numbers have pools of their own.
+    tokens_per_entry: int = 1
+    page_entries: Optional[int] = None
 
     def allocate(self, n_caches: int, units: int, page_size: int, device, dtype):
         raise NotImplementedError

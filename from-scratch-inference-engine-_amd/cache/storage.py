@@ -44,8 +44,11 @@ class CacheStorage:
         self.dtype = dtype
         self.spare_pages: List[int] = [manager.allocators[g].num_pages for g in range(len(layout.paged_groups))]
         self.spare_slot = manager.max_requests
-        self.group_stores = [need.allocate(len(layout.group_caches[g]), self.spare_pages[g] + 2, self.page_size,
-                                           device, dtype)
+        # positions that a page of each group holds (the filler rows of a padded batch need as many
+        # entries of the spare page in their tables as their tokens span)
+        self.tokens_per_page: List[int] = [manager.tokens_per_page(g) for g in range(len(layout.paged_groups))]
+        self.group_stores = [need.allocate(len(layout.group_caches[g]), self.spare_pages[g] + 2,
+                                           manager.entries_per_page[g], device, dtype)
                              for g, need in enumerate(layout.paged_groups)]
         self.state_stores = {cid: need.allocate(1, manager.max_requests + 1, self.page_size, device, dtype)
                              for cid, need in layout.state_caches.items()}

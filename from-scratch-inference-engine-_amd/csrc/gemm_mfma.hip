@@ -84,8 +84,8 @@ extern "C" int fsie_gemm_mfma_skinny_rope(const void* x, const void* w, const fl
     FSIE_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
                  "gemm_mfma_skinny_rope: operands must be 16-byte aligned");
     FSIE_REQUIRE(positions, "gemm_mfma_skinny_rope: no positions");
-    FSIE_REQUIRE(!cos_sin || (inv_freq && reinterpret_cast<uintptr_t>(cos_sin) % 8 == 0),
-                 "gemm_mfma_skinny_rope: a table of cosines and sines goes with a frequency table and is 8-byte aligned");
+    FSIE_REQUIRE(!cos_sin || reinterpret_cast<uintptr_t>(cos_sin) % 8 == 0,
+                 "gemm_mfma_skinny_rope: the table of cosines and sines must be 8-byte aligned");
     const bool store = k_pool != nullptr;
     FSIE_REQUIRE(!store || (v_pool && slots && page_size > 0 && pool_slots > 0),
                  "gemm_mfma_skinny_rope: a cache needs both pools, slots and a page geometry");

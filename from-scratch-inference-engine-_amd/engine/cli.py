@@ -46,16 +46,12 @@ def _llm(args):
     if args.config is not None or args.random_weights is not None:
         if args.config is None or args.random_weights is None:
             raise SystemExit("--config FILE and --random-weights SEED go together")
-        if args.tune_gemms:
-            from ..ops import enable_library_tuning
-
-            enable_library_tuning()
         with open(args.config) as f:
             raw = json.load(f)
         return LLM.from_config(raw, args.random_weights, block_size=args.block_size, num_blocks=args.num_blocks,
                                seed=args.seed, max_batch=args.max_batch, dtype=args.dtype,
                                max_tokens_per_step=args.max_tokens_per_step, prefill_chunk=args.prefill_chunk,
-                               weight_copies=not args.no_weight_copies)
+                               weight_copies=not args.no_weight_copies, tune_gemms=args.tune_gemms)
     if not args.model_dir:
         raise SystemExit("--model-dir (or $ENGINE_MODEL_DIR), or --config with --random-weights, is required")
     return LLM(args.model_dir, block_size=args.block_size, num_blocks=args.num_blocks, seed=args.seed,

@@ -28,12 +28,13 @@ class StepEntry:
     fresh: Sequence[Sequence[int]] = ()
 
 
-def filler_entry(storage, n_tokens: int, page_size: int):
+def filler_entry(storage, n_tokens: int):
     """Stands in a batch for a request that does not exist: ``n_tokens`` tokens of id 0 from
     position 0 that want no logits (or, with one token, its own), whose cache is the spare page
     of every pool, over and over, and the spare state slot.  Nothing a request reads is written."""
-    pages = max(1, -(-n_tokens // max(page_size, 1)))
-    spare = SimpleNamespace(length=0, slot=storage.spare_slot, tables=[[p] * pages for p in storage.spare_pages],
+    spare = SimpleNamespace(length=0, slot=storage.spare_slot,
+                            tables=[[p] * max(1, -(-n_tokens // per_page))
+                                    for p, per_page in zip(storage.spare_pages, storage.tokens_per_page)],
                             request_id="(filler)")
     return SimpleNamespace(cache=spare, tokens=(0,) * n_tokens, want=())
 
@@ -196,7 +197,6 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
     i_reset = pk.add(np.asarray(host.reset_slots, dtype=np.int32))
     i_qs = pk.add(np.asarray(host.q_starts, dtype=np.int32))
     i_past = pk.add(np.asarray(host.past_lens, dtype=np.int32))
-    ps = manager.page_size
     group_idx = []
     fresh_idx = []
     for g in range(len(manager.groups)):
@@ -215,14 +215,17 @@ def build_context(entries: Sequence[StepEntry], manager: CacheManager, planners:
             max_pages = pad["pages"]
         table = np.full((len(entries), max_pages), -1, dtype=np.int32)
         slot_map = np.full((host.n_tokens,), -1, dtype=np.int32)
+        # the group's own geometry: a position lies in entry pos // tokens_per_entry, an entry in page
+        # entry // entries_per_page
+        per_entry, ps = manager.tokens_per_entry[g], manager.entries_per_page[g]
         for s, e in enumerate(entries):
             # page ids become units of the pool: unit 0 is the null page, page p is unit p + 1
             pages = np.asarray(e.cache.tables[g], dtype=np.int32)
             pages = np.where(pages >= 0, pages + 1, -1)
             table[s, :pages.size] = pages
-            pos = host.positions[host.q_starts[s]:host.q_starts[s + 1]]
-            page_of = pages[pos // ps]
-            slot_map[host.q_starts[s]:host.q_starts[s + 1]] = np.where(page_of >= 0, page_of * ps + pos % ps, -1)
+            entry = host.positions[host.q_starts[s]:host.q_starts[s + 1]] // per_entry
+            page_of = pages[entry // ps]
+            slot_map[host.q_starts[s]:host.q_starts[s + 1]] = np.where(page_of >= 0, page_of * ps + entry % ps, -1)
         group_idx.append((pk.add(table), pk.add(slot_map)))
     plan_idx = []
     for planner in planners:

@@ -31,15 +31,16 @@ class Engine:
     """``Engine(model, block_size, num_blocks, seed=0, max_batch=256)`` with ``add_request``,
     ``step``, ``has_work``, ``output``, ``status``, ``preemptions`` and ``generate`` as in the
     reference (bindings/module.cpp:103-147, include/engine/engine.hpp:36-89).  Added:
-    ``max_tokens_per_step`` (token budget of a step) and ``prefill_chunk`` (longest portion of a
-    prompt in one step).  ``enable_prefix_cache`` is accepted for compatibility; prefix caching
+    ``max_tokens_per_step`` (token budget of a step), ``prefill_chunk`` (longest portion of a
+    prompt in one step) and ``fill_rows`` (see ``Runner``).  ``enable_prefix_cache`` is accepted for compatibility; prefix caching
     is not part of this engine and the flag changes nothing."""
 
     def __init__(self, model: Model, block_size: int = 16, num_blocks: int = 2048, seed: int = 0,
                  max_batch: int = 256, enable_prefix_cache: bool = False, *, max_tokens_per_step: int = 2048,
-                 prefill_chunk: Optional[int] = None):
+                 prefill_chunk: Optional[int] = None, fill_rows=None):
         self.model = model
-        self.runner = Runner(model, page_size=block_size, num_pages=num_blocks, max_requests=max_batch)
+        self.runner = Runner(model, page_size=block_size, num_pages=num_blocks, max_requests=max_batch,
+                             fill_rows=fill_rows)
         self.scheduler = Scheduler(self.runner.manager, max_batch=max_batch,
                                    max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk,
                                    max_position=self.runner.max_position)

@@ -56,8 +56,9 @@ class DecodeGraphs:
         self._asked: Dict[Tuple, int] = {}
         self._graphs: Dict[Tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor, torch.Tensor]] = {}
         model = runner.model
-        parts = [p for block in model.spec.layers for p in (block, *block.sub_parts().values())]
-        self.enabled = all(p.graph_safe for p in parts) and all(hasattr(p, "graph_bucket") for p in model.planners)
+        # every part of the model: the embedding, the head and the final norm as well as the layers'
+        self.enabled = (all(p.graph_safe for p in model.spec.all_parts())
+                        and all(hasattr(p, "graph_bucket") for p in model.planners))
         self.replays = 0
         self.captures = 0
         self._host = None  # the host view that shape_of made, for the step that follows
@@ -72,7 +73,7 @@ class DecodeGraphs:
     def filled_up(self, entries: Sequence[StepEntry]) -> List:
         """The entries and, behind them, the rows that pad the batch to a graph's size."""
         runner = self.runner
-        filler = filler_entry(runner.storage, 1, runner.manager.page_size)
+        filler = filler_entry(runner.storage, 1)
         filler.want = (0,)
         return list(entries) + [filler] * (padded_rows(len(entries)) - len(entries))
 
@@ -119,7 +120,7 @@ class DecodeGraphs:
             # the library's kernel selection.  It runs on rows that belong to no request (the spare
             # page, the spare slot), so that the step itself is executed once and only once, by the
             # replay below: a part whose cache is a running state would otherwise advance it twice.
-            warm = [filler_entry(runner.storage, 1, runner.manager.page_size) for _ in entries]
+            warm = [filler_entry(runner.storage, 1) for _ in entries]
             for w in warm:
                 w.want = (0,)
             warm_ctx, _ = build_context(warm, runner.manager, runner.model.planners, runner._staging,

@@ -40,16 +40,11 @@ class LLM:
                  weight_copies: bool = True):
         if quantize:
             raise NotImplementedError("LLM: quantized weights are not part of this engine")
-        if tune_gemms:
-            # bfloat16 prefill: let torch time the library's kernels for each new product shape of
-            # a full token budget (seconds, once per shape) instead of trusting its heuristic
-            from ..ops import enable_library_tuning
-
-            enable_library_tuning()
         model_dir = Path(model_dir)
         self.model = Model.from_pretrained(model_dir, dtype=dtype, device=device, weight_copies=weight_copies)
         self.engine = Engine(self.model, block_size, num_blocks, seed, max_batch, enable_prefix_cache,
-                             max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk)
+                             max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk,
+                             fill_rows=self._tuned_rows(tune_gemms, self.model))
         if eos_id is None:
             # the folder's generation_config.json, then the model's typed configuration
             eos_id = generation_end_token(model_dir)
@@ -59,11 +54,26 @@ class LLM:
         self._model_dir = model_dir
         self._tokenizer = None
 
+    @staticmethod
+    def _tuned_rows(tune_gemms: bool, model):
+        """``tune_gemms``: let torch time the library's kernels for the product shapes of a few row
+        counts (seconds, once per shape) instead of trusting its heuristic, and fill the steps that are
+        not decode steps up to those counts.  Only the bfloat16 path calls the library."""
+        import torch
+
+        if not tune_gemms or model.dtype != torch.bfloat16:
+            return None
+        from ..ops import enable_library_tuning
+        from .context import padded_tokens
+
+        enable_library_tuning()
+        return padded_tokens
+
     @classmethod
     def from_config(cls, config, weight_seed: int = 0, *, block_size: int = 16, num_blocks: int = 2048, seed: int = 0,
                     max_batch: int = 256, eos_id: int = -1, dtype: str = "bfloat16", device: str = "cuda:0",
                     max_tokens_per_step: int = 2048, prefill_chunk: Optional[int] = None,
-                    weight_copies: bool = True) -> "LLM":
+                    weight_copies: bool = True, tune_gemms: bool = False) -> "LLM":
         """An engine over random weights made from ``config`` (the dictionary of a config.json, or a
         typed configuration) and ``weight_seed``: no folder, no tokenizer, token ids in and out.
         The weights are those that ``write_random_model`` writes for the same seed (as float32)."""
@@ -73,7 +83,8 @@ class LLM:
         llm = cls.__new__(cls)
         llm.model = Model.from_random(typed, weight_seed, dtype=dtype, device=device, weight_copies=weight_copies)
         llm.engine = Engine(llm.model, block_size, num_blocks, seed, max_batch,
-                            max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk)
+                            max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk,
+                            fill_rows=cls._tuned_rows(tune_gemms, llm.model))
         llm.eos_id = eos_id
         llm._model_dir = None
         llm._tokenizer = None

@@ -21,10 +21,10 @@ from ..cache.storage import CacheLayout, CacheStorage
 from ..config.base import ModelConfig, read_config_json
 from ..models.registry import build_model_spec, parse_config
 from ..models.spec import ModelSpec
-from ..parts.base import HiddenState
+from ..parts.base import HiddenState, prepare_parts
 from ..weights.loader import fill_parts, load_weights
 from ..weights.random_init import random_tensor, expected_tensors
-from .context import PinnedStaging, StepContext, StepEntry, build_context, filler_entry, padded_tokens
+from .context import PinnedStaging, StepContext, StepEntry, build_context, filler_entry
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -127,18 +127,11 @@ class Model:
         return model
 
     def _prepare(self, weight_copies: bool = True) -> None:
-        from ..parts.base import Norm
-        from ..parts.linear import Linear
-
-        copy_from = Linear.streamed_copy_from
-        if not weight_copies:
-            Linear.streamed_copy_from = None  # while this model's parts are prepared
-        try:
-            for part in self.spec.all_parts():
-                part.prepare(self.device, self.dtype)
-        finally:
-            Linear.streamed_copy_from = copy_from
-        self.partial_sums_ok = all(p.adds_partial_sums for p in self.spec.all_parts() if isinstance(p, Norm))
+        self.options = {"weight_copies": bool(weight_copies)}
+        seen: set = set()
+        for part in self.spec.all_parts():
+            prepare_parts(part, self.device, self.dtype, self.options, seen)
+        self.partial_sums_ok = all(norm.adds_partial_sums for norm in self.spec.stream_norms())
 
     # ---------------------------------------------------------------- cache
     def make_cache(self, page_size: int, num_pages: int, max_requests: int):
@@ -173,8 +166,14 @@ class Runner:
     """The step function over one model and one cache."""
 
     def __init__(self, model: Model, page_size: int = 16, num_pages: int = 2048, max_requests: int = 256,
-                 use_graphs: bool = True):
+                 use_graphs: bool = True, fill_rows=None):
+        """``fill_rows``: optional policy ``tokens -> tokens`` of whoever made the runner: a step that
+        is not replayed from a graph is filled up to that many rows with the tokens of a request that
+        does not exist (``filler_entry``).  A caller that has the library's kernels timed for a few
+        row counts passes ``padded_tokens``.  Only for models whose parts all read a step through its
+        device tables (``graph_safe``): the filler's rows exist in those tables alone."""
         self.model = model
+        self.fill_rows = fill_rows if all(p.graph_safe for p in model.spec.all_parts()) else None
         self.manager, self.storage = model.make_cache(page_size, num_pages, max_requests)
         self._staging = PinnedStaging()
         self.vocab_size = model.spec.embedding.vocab_size
@@ -233,14 +232,9 @@ class Runner:
         else:
             n_tokens = sum(len(e.tokens) for e in entries)
             batch = list(entries)
-            if (self.model.dtype == torch.bfloat16 and ops.library_tuning_enabled()
-                    and self.graphs is not None and self.graphs.enabled):
-                # with the library's kernels chosen by timing, a step is filled up to one of the few
-                # row counts that are timed, with the tokens of a request that does not exist (only
-                # for models whose parts all read the step through its device tables, as for graphs)
-                extra = padded_tokens(n_tokens) - n_tokens
-                if extra > 0:
-                    batch.append(filler_entry(self.storage, extra, self.manager.page_size))
+            extra = self.fill_rows(n_tokens) - n_tokens if self.fill_rows is not None else 0
+            if extra > 0:
+                batch.append(filler_entry(self.storage, extra))
             ctx, _ = build_context(batch, self.manager, self.model.planners, self._staging, self.model.dtype,
                                    self.model.device)
             if feed is not None:

@@ -127,7 +127,7 @@ class Scheduler:
         need = self.manager.max_pages_held(total, self.prefill_chunk)
         for g, pages in enumerate(need):
             if pages > self.manager.allocators[g].num_pages:
-                raise ValueError(f"Engine: the request needs {pages} pages of {self.manager.page_size} tokens, "
+                raise ValueError(f"Engine: the request needs {pages} pages of {self.manager.tokens_per_page(g)} tokens, "
                                  f"the pool has {self.manager.allocators[g].num_pages}: it can never run")
         sid = self._next_id
         self._next_id += 1
@@ -172,7 +172,8 @@ class Scheduler:
             # cut back to the last page boundary below n (what is free in the last held page
             # always fits), then page by page
             filled = seq.computed + n
-            n = ((filled - 1) // self.manager.page_size) * self.manager.page_size - seq.computed
+            step = self.manager.smallest_page_tokens
+            n = ((filled - 1) // step) * step - seq.computed
         return max(n, 0)
 
     def _build(self) -> List[ScheduledItem]:

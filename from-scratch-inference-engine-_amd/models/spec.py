@@ -37,12 +37,27 @@ class ModelSpec:
     ignore_unexpected: Sequence[str] = ()
 
     def all_parts(self) -> List[Part]:
-        out: List[Part] = [self.embedding]
-        for block in self.layers:
-            out.append(block)
-            out.extend(block.sub_parts().values())
-        out += [self.final_norm, self.lm_head]
+        """Every part of the model once, parts before the parts they are made of."""
+        out: List[Part] = []
+        seen = set()
+
+        def add(part: Part) -> None:
+            if id(part) in seen:
+                return
+            seen.add(id(part))
+            out.append(part)
+            for sub in part.sub_parts().values():
+                add(sub)
+
+        for part in (self.embedding, *self.layers, self.final_norm, self.lm_head):
+            add(part)
         return out
+
+    def stream_norms(self) -> List[Norm]:
+        """The norms that read the residual stream and fold its pending delta in: those a block
+        names among its own parts, and the final one."""
+        norms = [p for block in self.layers for p in block.sub_parts().values() if isinstance(p, Norm)]
+        return norms + [self.final_norm]
 
 
 def bind(bindings: List[ParamBinding], owner: Part, attr: str, sources: Sequence[TensorSpec]) -> None:

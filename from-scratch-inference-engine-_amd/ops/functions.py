@@ -192,7 +192,8 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
     copy k and v to the cache slots ``slots`` (int32 [T], negative = not stored) of the pools: keys
     [pages, n_kv, page_size, head_dim], values [pages, n_kv, head_dim, page_size].  ``cos_sin``
     (``rope_table`` of these positions and frequencies): where the whole head is rotated and
-    head_dim is a multiple of 8, the kernel reads the angles' cosines and sines there.
+    head_dim is a multiple of 8, the kernel reads the angles' cosines and sines there; the table
+    alone, without ``inv_freq``, says that the whole head is rotated by it.
     ``parts`` (float32 [S, T, width], only with ``cos_sin``): the projection as the partial sums of a
     product cut along its inner dimension; they are added in order, ``qkv`` is then only written: its
     q columns get the rotated q heads, k and v go to the pools alone."""
@@ -205,6 +206,10 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
     if inv_freq is not None:
         _need(inv_freq, "inv_freq", dtype=torch.float64, ndim=1)
         rotary_dim = 2 * inv_freq.shape[0]
+    elif cos_sin is not None:
+        if head_dim % 8:
+            raise KernelError("rope_kv_write: a table of cosines and sines alone needs a head of a multiple of 8 dimensions")
+        rotary_dim = head_dim
     if bias is not None:
         _need(bias, "qkv bias", dtype=torch.float32, shape=(qkv.shape[1],))
     pool_slots = 0
@@ -432,7 +437,7 @@ def gemm_mfma_skinny_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[
     heads over the whole head (``inv_freq``: float64 [head_dim / 2], ``None`` = none) and the
     write of k and v into the cache pools at ``slots``.  ``cos_sin``: what ``rope_table`` made of
     these positions and frequencies (the kernel then reads the cosines and sines instead of
-    computing them).  Returns [M, N] whose q columns are filled; the k and v columns are not
+    computing them; the table may come without ``inv_freq``).  Returns [M, N] whose q columns are filled; the k and v columns are not
     written."""
     _need(x, "gemm x", dtype=torch.bfloat16, ndim=2)
     _need(weight, "gemm weight", dtype=torch.bfloat16, ndim=2)
@@ -446,8 +451,6 @@ def gemm_mfma_skinny_rope(x: torch.Tensor, weight: torch.Tensor, bias: Optional[
     if inv_freq is not None:
         _need(inv_freq, "inv_freq", dtype=torch.float64, shape=(head_dim // 2,))
     if cos_sin is not None:
-        if inv_freq is None:
-            raise KernelError("gemm_mfma_skinny_rope: a table of cosines and sines without frequencies")
         _need(cos_sin, "cos_sin", dtype=torch.float32, shape=(m, head_dim // 2, 2))
     pool_slots = 0
     if k_pool is not None:

@@ -11,9 +11,9 @@ import torch
 from .. import ops
 from ..cache.manager import PagedNeed
 from ..ops.functions import ATTN_ITEM_INTS, ATTN_MERGE_INTS
-from .base import Mixer, ParamDecl, PositionEncoding, register_part
+from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M
+from .base import Mixer, Norm, ParamDecl, Part, PositionEncoding, register_part
 from .linear import Linear
-from .rope import KVStore
 
 
 class AttentionPlanner:
@@ -251,10 +251,21 @@ class AttentionPlanner:
 
 @register_part("mixer", "gqa_attention")
 class GQAttention(Mixer):
-    """q/k/v projections (one matrix, optional bias), position encoding, causal attention with
-    kv head = q head // (heads / kv heads) and scale 1/sqrt(head_dim), output projection without
-    bias (src/model/model.cpp:110-129, src/model/nn.cpp:151-226).  ``window`` = number of latest
-    positions a query reads (None: all)."""
+    """q/k/v projections (one matrix, optional bias), optional norms of every q and k head,
+    position encoding, causal attention with kv head = q head // (heads / kv heads) and scale
+    1/sqrt(head_dim), output projection without bias (src/model/model.cpp:110-129,
+    src/model/nn.cpp:151-226).  ``window`` = number of latest positions a query reads (None: all).
+
+    What happens between the projection and attention, in this order: bias, ``q_norm`` / ``k_norm``
+    (a norm as wide as a head, applied to every head through ``Norm.plain``; None: none), the
+    position encoding's ``rotate``, the write of k and v into the cache.  The mixer owns all of it;
+    the encoding only rotates.  Where nothing stands between the projection and a rotation that
+    the encoding can describe by a table of cosines and sines (``rotation_table``), the mixer's own
+    kernels do several of these steps at once: for steps of one token a request the attention
+    kernel itself finishes the projection's partial sums (bias, rotation, cache write); for up to 16
+    rows the projection's epilogue does; for 17 to 128 rows the kernel that writes the cache adds
+    the partial sums up.  With head norms, or an encoding without a table, the steps run one after
+    the other (projection, bias, norms, ``rotate``, cache write), which every combination can take."""
 
     share_keys = True  # long portions: four tiles of a request share each block of keys through LDS
     # steps of one token a request: the attention kernel adds up the q/k/v product's partial sums,
@@ -263,11 +274,12 @@ class GQAttention(Mixer):
 
     @property
     def graph_safe(self) -> bool:
-        """forward reads the step only through device tables; the position encoding must too."""
-        return self.position.graph_safe
+        """forward reads the step only through device tables; its sub-parts must too."""
+        return all(p.graph_safe for p in self.sub_parts().values())
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, qkv_bias: bool,
-                 position: PositionEncoding, window: Optional[int] = None):
+                 position: PositionEncoding, window: Optional[int] = None, q_norm: Optional[Norm] = None,
+                 k_norm: Optional[Norm] = None):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: heads {n_heads} must be a multiple of kv heads {n_kv_heads}")
         if head_dim > 256:
@@ -275,11 +287,20 @@ class GQAttention(Mixer):
         self.hidden_size, self.n_heads, self.n_kv, self.head_dim = hidden_size, n_heads, n_kv_heads, head_dim
         self.window = window
         self.position = position
+        self.q_norm, self.k_norm = q_norm, k_norm
         self.q_dim, self.kv_dim = n_heads * head_dim, n_kv_heads * head_dim
         self.qkv = Linear(hidden_size, self.q_dim + 2 * self.kv_dim, bias=qkv_bias)
         self.o = Linear(self.q_dim, hidden_size)
         self.scale = 1.0 / math.sqrt(head_dim)
         self._planner: Optional[AttentionPlanner] = None
+
+    def sub_parts(self) -> Dict[str, Part]:
+        parts: Dict[str, Part] = {"position": self.position}
+        if self.q_norm is not None:
+            parts["q_norm"] = self.q_norm
+        if self.k_norm is not None:
+            parts["k_norm"] = self.k_norm
+        return parts
 
     # parameters -------------------------------------------------------------------------
     def param_decls(self) -> Dict[str, ParamDecl]:
@@ -294,9 +315,9 @@ class GQAttention(Mixer):
     o_weight = property(lambda s: s.o.weight, lambda s, t: setattr(s.o, "weight", t))
 
     def prepare(self, device, compute_dtype) -> None:
-        self.position.prepare(device, compute_dtype)
-        self.o.prepare()
-        self.qkv.prepare()  # (read by the product of 17 to 64 rows; the few-rows product with the rotation reads rows)
+        copies = bool(self.options.get("weight_copies", True))
+        self.o.prepare(copies)
+        self.qkv.prepare(copies)  # (read by the product of 17 to 64 rows; the few-rows product with the rotation reads rows)
 
     # cache and plan ---------------------------------------------------------------------
     def cache_need(self) -> PagedNeed:
@@ -308,15 +329,20 @@ class GQAttention(Mixer):
         return self._planner
 
     # compute ----------------------------------------------------------------------------
-    def _from_sums(self, x: torch.Tensor, ctx, cache, plan) -> Optional[torch.Tensor]:
+    def _fused_table(self, ctx) -> Optional[torch.Tensor]:
+        """The rotation as a table, if the mixer's fused kernels may stand for bias + rotate + write:
+        nothing between the projection and the rotation, and an encoding that is such a rotation
+        (or none at all: then the kernels only add the bias and write)."""
+        if self.q_norm is not None or self.k_norm is not None or self.head_dim % 8:
+            return None
+        return self.position.rotation_table(self.head_dim, ctx)
+
+    def _from_sums(self, x: torch.Tensor, ctx, cache, plan, table) -> Optional[torch.Tensor]:
         """Attention of a step of one token a request straight from the q/k/v product's partial sums
         (None: not such a step, or the kernels do not take the sizes)."""
-        if not (self.finish_qkv_in_attention and cache.writes and plan.mfma and plan.single and plan.n_small
-                and not plan.n_large and not plan.n_long and x.dtype == torch.bfloat16
+        if not (self.finish_qkv_in_attention and table is not None and cache.writes and plan.mfma and plan.single
+                and plan.n_small and not plan.n_large and not plan.n_long and x.dtype == torch.bfloat16
                 and ops.attention_mfma_qkv_ok(self.head_dim, cache.page_size)):
-            return None
-        table = self.position.rotation_table(self.head_dim, ctx)
-        if table is None:
             return None
         sums = self.qkv.partial_sums(x, few_rows=True)
         if sums is None:
@@ -333,23 +359,53 @@ class GQAttention(Mixer):
             ops.attention_merge(partials, plan.merges, plan.n_merges, out, self.n_heads, self.head_dim)
         return out
 
-    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
-        plan = ctx.plan(self.planner())
-        out = self._from_sums(x, ctx, cache, plan)
-        if out is not None:
-            return self.o.for_residual(out, ctx)
-        store = KVStore(cache.k_pool, cache.v_pool, cache.slots, cache.page_size) if cache.writes else None
-        qkv = self.position.project(x, self.qkv.weight, self.qkv.bias, self.n_heads, self.n_kv, self.head_dim, ctx,
-                                    store)
-        if qkv is None:
-            # 17 to 64 rows: the engine's product in slices of K, added up by the kernel that rotates
+    def _project_rotate_store(self, x: torch.Tensor, ctx, cache, table) -> torch.Tensor:
+        """q/k/v [T, (heads + 2 kv heads) head_dim] of which attention reads the q columns: projected,
+        with the bias, the head norms and the rotation applied, and k and v written into the cache
+        (unless this call only reads another call's cache)."""
+        nh, nkv, hd = self.n_heads, self.n_kv, self.head_dim
+        store = dict(slots=cache.slots, k_pool=cache.k_pool, v_pool=cache.v_pool,
+                     page_size=cache.page_size) if cache.writes else {}
+        bias = self.qkv.bias
+        if table is not None:
+            if x.dtype == torch.bfloat16 and 0 < x.shape[0] <= GEMM_MFMA_SKINNY_BEST_M and x.shape[1] % 8 == 0 and hd % 16 == 0:
+                # a few rows of a step that is not one token a request: the projection's own epilogue
+                # adds the bias, rotates and stores
+                return ops.gemm_mfma_skinny_rope(x, self.qkv.weight, bias, ctx.positions, nh, nkv, hd, None,
+                                                 cos_sin=table, **store)
             sums = self.qkv.partial_sums(x)
             if sums is not None:
-                qkv = self.position.apply_sums(sums, self.n_heads, self.n_kv, self.head_dim, ctx, store,
-                                               bias=self.qkv.bias)
-        if qkv is None:
-            qkv = self.qkv(x, skip_bias=True)
-            self.position.apply(qkv, self.n_heads, self.n_kv, self.head_dim, ctx, store, bias=self.qkv.bias)
+                # 17 to 128 rows: the engine's product in slices of K, added up by the kernel that rotates
+                qkv = torch.empty(sums.shape[1:], dtype=ctx.compute_dtype, device=x.device)
+                return ops.rope_kv_write(qkv, ctx.positions, nh, nkv, hd, None, bias=bias, cos_sin=table,
+                                         parts=sums, **store)
+        qkv = self.qkv(x, skip_bias=True)
+        if table is not None:
+            return ops.rope_kv_write(qkv, ctx.positions, nh, nkv, hd, None, bias=bias, cos_sin=table, **store)
+        # one step after the other
+        plain_write = not self.position.rotates and self.q_norm is None and self.k_norm is None
+        if bias is not None and not plain_write:
+            ops.bias_add(qkv, bias)
+            bias = None
+        if self.q_norm is not None:
+            q = qkv[:, :self.q_dim]
+            self.q_norm.plain(q, out=q)
+        if self.k_norm is not None:
+            k = qkv[:, self.q_dim:self.q_dim + self.kv_dim]
+            self.k_norm.plain(k, out=k)
+        if self.position.rotates:
+            self.position.rotate(qkv, nh, nkv, hd, ctx)
+        if store or bias is not None:
+            ops.rope_kv_write(qkv, ctx.positions, nh, nkv, hd, None, bias=bias, **store)  # (no rotation: bias, write)
+        return qkv
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        plan = ctx.plan(self.planner())
+        table = self._fused_table(ctx)
+        out = self._from_sums(x, ctx, cache, plan, table)
+        if out is not None:
+            return self.o.for_residual(out, ctx)
+        qkv = self._project_rotate_store(x, ctx, cache, table)
         t = x.shape[0]
         out = torch.empty((t, self.q_dim), dtype=x.dtype, device=x.device)
         partials = None

@@ -15,8 +15,9 @@ Kinds and their interfaces (``ctx`` is the step's ``StepContext``):
                    request: a need of ``cache.needs`` (``PagedNeed``: keys and values per token,
                    ``StateNeed``: fixed size, or one of its own that owns its memory) or nothing; ``planner()`` may name per-step index tables it wants built on the host.
   FeedForward      ``y = ffn.forward(x, ctx)``.
-  PositionEncoding ``pos.apply(qkv, n_heads, n_kv, head_dim, ctx, store)`` rotates/marks q and k
-                   in place and hands k and v to the cache through ``store``.
+  PositionEncoding ``pos.rotate(qkv, n_heads, n_kv, head_dim, ctx)`` transforms the q and k heads
+                   in place by the step's positions.  It touches nothing else: bias, norms of q
+                   and k and the write into the cache are the mixer's.
   Block            the arrangement: ``block.forward(hidden, ctx, cache)``.
 """
 
@@ -63,12 +64,36 @@ class Part:
     # that captures a graph (the warm-up before a capture runs on rows of no request), so a part
     # whose cache is a running state may set it.
     graph_safe = False
+    # what the model was loaded with (``weight_copies``: whether large matrices may be kept a second
+    # time in another order); the model sets it on every part before ``prepare``
+    options: Dict[str, Any] = {}
 
     def param_decls(self) -> Dict[str, ParamDecl]:
         return {}
 
     def prepare(self, device, compute_dtype: torch.dtype) -> None:
         """Called once after the parameters are set (tables, constants on the device)."""
+
+    def sub_parts(self) -> Dict[str, "Part"]:
+        """The parts this one is made of (a block's norms, mixer and feed-forward; a mixer's
+        position encoding and the norms of its heads).  The model prepares them, asks them for
+        ``graph_safe`` and lists them with the rest; their parameters are bound like any part's."""
+        return {}
+
+
+def prepare_parts(part: "Part", device, compute_dtype: torch.dtype, options: Optional[Dict[str, Any]] = None,
+                  _seen: Optional[set] = None) -> None:
+    """``prepare`` for ``part`` and every part it is made of, each once, with ``options`` set on
+    them first.  The model calls it for its parts; whoever uses a part by itself calls it too."""
+    seen = set() if _seen is None else _seen
+    if id(part) in seen:
+        return
+    seen.add(id(part))
+    if options is not None:
+        part.options = options
+    part.prepare(device, compute_dtype)
+    for sub in part.sub_parts().values():
+        prepare_parts(sub, device, compute_dtype, options, seen)
 
 
 class Norm(Part):
@@ -82,10 +107,11 @@ class Norm(Part):
     def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
         raise NotImplementedError
 
-    def plain(self, x: torch.Tensor) -> torch.Tensor:
+    def plain(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """The norm of a plain tensor [T, W], away from the residual stream: a mixer's or a
         feed-forward's output before it is added (sandwich and post-norm arrangements), or the
-        heads of q and k (a norm as wide as a head normalises every head of a row)."""
+        heads of q and k (a norm as wide as a head normalises every head of a row; ``x`` may be
+        the q or k columns of a q/k/v row, and ``out`` may be ``x``)."""
         raise NotImplementedError
 
 
@@ -111,31 +137,22 @@ class FeedForward(Part):
 
 class PositionEncoding(Part):
     kind = "position"
+    # False for an encoding that leaves q and k as they are (the mixer then skips the call)
+    rotates = True
 
-    def apply(self, qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, ctx, store,
-              bias: Optional[torch.Tensor] = None) -> None:
+    def rotate(self, qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, ctx) -> None:
+        """Transform the q and k heads of ``qkv`` [T, (n_heads + 2 n_kv) head_dim] in place by the
+        step's positions (``ctx.positions``, int32 [T]).  The bias has been added and the heads
+        normalised, if the mixer does either; the values are not touched, and nothing is written
+        to the cache: that is the mixer's, after this call."""
         raise NotImplementedError
-
-    def project(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], n_heads: int,
-                n_kv: int, head_dim: int, ctx, store) -> Optional[torch.Tensor]:
-        """Optional: the fused q/k/v projection of ``x`` and ``apply`` in one kernel.  Returns
-        the [T, (n_heads + 2 n_kv) head_dim] result of which the mixer reads only the q columns,
-        or None if this encoding (or these sizes) has no such kernel: the mixer then projects
-        by itself and calls ``apply``."""
-        return None
-
-    def apply_sums(self, parts: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, ctx, store,
-                   bias: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-        """Optional: ``apply`` on a projection that comes as float32 partial sums [S, T, width] of a
-        product cut along its inner dimension (added in order).  Returns [T, width] in the compute
-        dtype, of which the mixer reads only the q columns, or None if this encoding cannot: the
-        mixer then projects whole and calls ``apply``."""
-        return None
 
     def rotation_table(self, head_dim: int, ctx) -> Optional[torch.Tensor]:
         """Optional: if this encoding is the rotation of the pairs (i, i + head_dim / 2) of every
         q and k head by an angle per token and pair, the step's float32 table [T, head_dim / 2, 2]
-        of their cosines and sines, for a mixer whose own kernel rotates; else None."""
+        of their cosines and sines.  A mixer whose own kernels rotate (in the epilogue of the q/k/v
+        product, in the kernel that writes the cache, inside attention) takes the table instead of
+        calling ``rotate``; None, the default: the mixer calls ``rotate``."""
         return None
 
 
@@ -144,9 +161,6 @@ class Block(Part):
 
     def forward(self, hidden: HiddenState, ctx, cache) -> None:
         raise NotImplementedError
-
-    def sub_parts(self) -> Dict[str, Part]:
-        return {}
 
 
 # ------------------------------------------------------------------------------ registries

@@ -16,6 +16,7 @@ class TokenEmbedding(Part):
     residual stream."""
 
     kind = "embedding"
+    graph_safe = True  # reads the step's token ids from the device
 
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
@@ -33,6 +34,7 @@ class LMHead(Part):
     its weight is bound to the embedding table."""
 
     kind = "lm_head"
+    graph_safe = True
 
     def __init__(self, hidden_size: int, vocab_size: int):
         self.linear = Linear(hidden_size, vocab_size)
@@ -50,7 +52,7 @@ class LMHead(Part):
         self.linear.weight = t
 
     def prepare(self, device, compute_dtype) -> None:
-        self.linear.prepare()
+        self.linear.prepare(bool(self.options.get("weight_copies", True)))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.linear(x, out_dtype=torch.float32)

@@ -61,11 +61,11 @@ class Linear:
         self.streamed = None  # a copy of the weight that was here says nothing about this one
         self._wide_takes = {}
 
-    def prepare(self) -> None:
-        """Called by the owning part once the weight is set."""
+    def prepare(self, copies: bool = True) -> None:
+        """Called by the owning part once the weight is set.  ``copies=False``: no second copy."""
         w = self.weight
         self.streamed = None
-        if (self.streamed_copy_from is not None and w is not None and w.dtype == torch.bfloat16 and w.is_cuda
+        if (copies and self.streamed_copy_from is not None and w is not None and w.dtype == torch.bfloat16 and w.is_cuda
                 and w.numel() * 2 >= self.streamed_copy_from and ops.gemm_mfma_wide_splits_ok(self.in_features, 1)):
             free, total = torch.cuda.mem_get_info(w.device)
             if free - w.numel() * 2 >= self.streamed_copy_reserve * total:
@@ -184,7 +184,8 @@ class Linear:
         groups = -(-self.out_features // 16)
         shortest = 512 if m <= GEMM_MFMA_SKINNY_BEST_M else 1024
         splits = 1
-        while splits < 8 and groups * splits < 896 and self.in_features // (2 * splits) >= shortest:
+        # (about three and a half workgroups a compute unit)
+        while splits < 8 and 2 * groups * splits < 7 * ops.compute_units() and self.in_features // (2 * splits) >= shortest:
             splits *= 2
         if m > GEMM_MFMA_SKINNY_BEST_M and splits < 4:
             return 1

@@ -48,8 +48,9 @@ class SwiGLU(FeedForward):
         self.down.weight = t
 
     def prepare(self, device, compute_dtype) -> None:
-        self.gate_up.prepare()
-        self.down.prepare()
+        copies = bool(self.options.get("weight_copies", True))
+        self.gate_up.prepare(copies)
+        self.down.prepare(copies)
 
     # rows up to which silu(gate) * up comes from the product that shares x through LDS when the weight
     # has a fragment-ordered copy (beyond: the library's product and a kernel for SiLU*up)

@@ -36,5 +36,5 @@ class RMSNorm(Norm):
     def rows(self, hidden: HiddenState, rows: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
         return ops.rmsnorm(hidden.residual, self.weight, self.eps, out_dtype, delta=hidden.delta, rows=rows)
 
-    def plain(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.rmsnorm_plain(x, self.weight, self.eps)
+    def plain(self, x: torch.Tensor, out=None) -> torch.Tensor:
+        return ops.rmsnorm_plain(x, self.weight, self.eps, out=out)

@@ -8,25 +8,15 @@ import numpy as np
 import torch
 
 from .. import ops
-from ..ops.functions import GEMM_MFMA_SKINNY_BEST_M
 from .base import PositionEncoding, register_part
-
-
-class KVStore:
-    """Where a position encoding hands keys and values: the pools of one layer and, per token,
-    the slot to write (negative = not stored)."""
-
-    __slots__ = ("k_pool", "v_pool", "slots", "page_size")
-
-    def __init__(self, k_pool, v_pool, slots, page_size):
-        self.k_pool, self.v_pool, self.slots, self.page_size = k_pool, v_pool, slots, page_size
 
 
 @register_part("position", "rope")
 class RotaryEncoding(PositionEncoding):
     """Rotate-half RoPE over ``rotary_dim`` (default: the whole head): pair (i, i + rotary_dim/2),
     frequency theta^(-2i/rotary_dim), angle = position * frequency in float64
-    (src/model/nn.cpp:110-149).  Fused with the q/k/v bias and the write into the cache."""
+    (src/model/nn.cpp:110-149).  Where the whole head rotates it also offers the step's table of
+    cosines and sines, from which a mixer's own kernels rotate."""
 
     graph_safe = True
 
@@ -55,50 +45,20 @@ class RotaryEncoding(PositionEncoding):
     def rotation_table(self, head_dim, ctx):
         return self.table(ctx) if self.rotary_dim == head_dim else None
 
-    def apply(self, qkv, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore], bias=None) -> None:
+    def rotate(self, qkv, n_heads, n_kv, head_dim, ctx) -> None:
         cos_sin = self.table(ctx) if self.rotary_dim == head_dim and head_dim % 8 == 0 else None
-        if store is None:
-            ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, bias=bias, cos_sin=cos_sin)
-        else:
-            ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, slots=store.slots,
-                              k_pool=store.k_pool, v_pool=store.v_pool, page_size=store.page_size, bias=bias,
-                              cos_sin=cos_sin)
-
-    def apply_sums(self, parts, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore], bias=None):
-        if self.rotary_dim != head_dim or head_dim % 8:
-            return None
-        qkv = torch.empty(parts.shape[1:], dtype=ctx.compute_dtype, device=parts.device)
-        kw = {} if store is None else dict(slots=store.slots, k_pool=store.k_pool, v_pool=store.v_pool,
-                                           page_size=store.page_size)
-        return ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, bias=bias,
-                                 cos_sin=self.table(ctx), parts=parts, **kw)
-
-    def project(self, x, weight, bias, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore]):
-        """For a few rows of bfloat16 (decoding) the projection's own epilogue rotates and stores."""
-        if (x.dtype != torch.bfloat16 or not 0 < x.shape[0] <= GEMM_MFMA_SKINNY_BEST_M or x.shape[1] % 8
-                or head_dim % 16 or self.rotary_dim != head_dim):
-            return None
-        table = self.table(ctx)
-        if store is None:
-            return ops.gemm_mfma_skinny_rope(x, weight, bias, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq,
-                                             cos_sin=table)
-        return ops.gemm_mfma_skinny_rope(x, weight, bias, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq,
-                                         slots=store.slots, k_pool=store.k_pool, v_pool=store.v_pool,
-                                         page_size=store.page_size, cos_sin=table)
+        ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, self.inv_freq, cos_sin=cos_sin)
 
 
 @register_part("position", "none")
 class NoPositionEncoding(PositionEncoding):
-    """No rotation: only the bias and the write into the cache."""
+    """No rotation: q and k stay as they are."""
 
     graph_safe = True
+    rotates = False
 
     def __init__(self, head_dim: int = 0):
         self.head_dim = head_dim
 
-    def apply(self, qkv, n_heads, n_kv, head_dim, ctx, store: Optional[KVStore], bias=None) -> None:
-        if store is None:
-            ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, None, bias=bias)
-        else:
-            ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, None, slots=store.slots,
-                              k_pool=store.k_pool, v_pool=store.v_pool, page_size=store.page_size, bias=bias)
+    def rotate(self, qkv, n_heads, n_kv, head_dim, ctx) -> None:
+        return None

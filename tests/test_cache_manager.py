@@ -134,3 +134,35 @@ def test_random_orders_keep_every_page_accounted(seed):
         m.close(rc)
     m.check_invariants()
     assert all(a.num_free == a.num_pages for a in m.allocators) and m.free_slots == 4 and events > 50
+
+
+def test_groups_with_page_geometries_of_their_own():
+    """A need may say how many positions one of its entries holds and how many entries a page of
+    its group has; the manager then counts that group's pages, and hands back a window's pages, by
+    those numbers, beside a group that uses the cache's page size."""
+    from dataclasses import dataclass
+    from from_scratch_inference_engine_amd.cache.needs import CacheNeed
+
+    @dataclass(frozen=True)
+    class Blocks(CacheNeed):
+        tokens_per_entry: int = 4
+        page_entries: int = 2
+        window: object = None
+
+    m = CacheManager([PagedNeed(2, 8), Blocks(), Blocks(window=10)], page_size=4, num_pages=[16, 5, 5], max_requests=2)
+    assert [m.tokens_per_page(g) for g in range(3)] == [4, 8, 8] and m.smallest_page_tokens == 4
+    assert [m.pages_for(17, g) for g in range(3)] == [5, 3, 3]
+    rc = m.open("r")
+    assert m.new_pages_needed(rc, 17) == [5, 3, 3]
+    assert m.max_pages_held(100, 6) == [25, 13, 4]      # the windowed group: 10 + 6 + 8 positions and one page
+    m.reserve(rc, 17)
+    m.commit(rc, 17)
+    assert [len(t) for t in rc.tables] == [5, 3, 3]
+    assert rc.tables[2][0] == -1 and rc.tables[2][1] >= 0  # positions before 17 - 10 + 1 = 8 are past the window: page 0 is back
+    assert m.new_pages_needed(rc, 7) == [1, 0, 0] and m.new_pages_needed(rc, 8) == [2, 1, 1]
+    with pytest.raises(RuntimeError, match="beyond the reserved"):
+        m.commit(rc, 8)                                   # 25 positions do not fit five pages of four
+    assert not m.can_reserve([(rc, 17 * 8)])
+    m.check_invariants()
+    m.close(rc)
+    assert [a.num_free for a in m.allocators] == [16, 5, 5]

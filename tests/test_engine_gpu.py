@@ -647,7 +647,8 @@ def test_prefill_with_the_library_kernel_selection(model_dirs):
         # that does not exist: what the real requests get does not change, nor what they decode next
         from from_scratch_inference_engine_amd.engine.context import padded_tokens
         assert padded_tokens(70 + 37) == 128
-        runner = Runner(load_model(model_dirs["B"], dtype="bfloat16"), page_size=8, num_pages=40, max_requests=3)
+        runner = Runner(load_model(model_dirs["B"], dtype="bfloat16"), page_size=8, num_pages=40, max_requests=3,
+                        fill_rows=padded_tokens)
         pair = [helpers.token_ids(vocab, 71, 870), helpers.token_ids(vocab, 38, 871)]
         pair_ref = [plain.forward_dir(model_dirs["B"], s_).numpy() for s_ in pair]
         pc = [runner.manager.open(i) for i in range(2)]
@@ -954,7 +955,8 @@ def test_steps_filled_up_to_the_timed_row_counts_of_256_and_more(tmp_path):
     real_mm = ops.library_mm
     ops.enable_library_tuning(max_ms_per_candidate=5, iterations=2)
     try:
-        runner = Runner(load_model(d, dtype="bfloat16"), page_size=16, num_pages=80, max_requests=4)
+        runner = Runner(load_model(d, dtype="bfloat16"), page_size=16, num_pages=80, max_requests=4,
+                        fill_rows=padded_tokens)
         import from_scratch_inference_engine_amd.parts.linear as linear_module
         saved = linear_module.library_mm
         linear_module.library_mm = lambda x, w, **k: (rows_seen.append(x.shape[0]), saved(x, w, **k))[1]

@@ -91,8 +91,9 @@ def mixer_harness(mixer, dtype, page_size, num_pages, n_requests=3):
     from from_scratch_inference_engine_amd.cache import CacheManager
     from from_scratch_inference_engine_amd.cache.storage import CacheLayout, CacheStorage
     from from_scratch_inference_engine_amd.engine.context import PinnedStaging, StepEntry, build_context
+    from from_scratch_inference_engine_amd.parts import prepare_parts
 
-    mixer.prepare("cuda", dtype)
+    prepare_parts(mixer, "cuda", dtype)
     manager = CacheManager([mixer.cache_need()], page_size, num_pages, n_requests)
     storage = CacheStorage(CacheLayout([mixer.cache_need()], [[0]], {}), manager, "cuda", dtype)
     staging = PinnedStaging()

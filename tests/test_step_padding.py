@@ -26,10 +26,11 @@ def test_rows_of_a_decode_graph():
 
 
 def test_the_filler_reads_and_writes_spare_places_only():
-    storage = SimpleNamespace(spare_slot=5, spare_pages=[40, 17])   # two groups of layers
-    e = filler_entry(storage, 37, page_size=8)
+    # two groups of layers; a page of the second holds 16 positions (a need with a geometry of its own)
+    storage = SimpleNamespace(spare_slot=5, spare_pages=[40, 17], tokens_per_page=[8, 16])
+    e = filler_entry(storage, 37)
     assert len(e.tokens) == 37 and set(e.tokens) == {0} and tuple(e.want) == ()
     assert e.cache.length == 0 and e.cache.slot == 5
-    assert e.cache.tables == [[40] * 5, [17] * 5]          # every page of its table is the spare one
+    assert e.cache.tables == [[40] * 5, [17] * 3]          # every page of its table is the spare one
     host = HostBatch([e], page_size=8)
     assert host.n_tokens == 37 and host.positions.tolist() == list(range(37)) and host.want_rows.size == 0

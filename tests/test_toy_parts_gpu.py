@@ -58,15 +58,15 @@ def define_toys():
     @register_part("position", "toy_interleaved_rope")
     class InterleavedRope(PositionEncoding):
         """Rotation of the pairs (2i, 2i + 1) of every q and k head (the engine's own encoding
-        pairs i with i + head_dim / 2).  The toy adds the bias and rotates with torch, then hands
-        q, k and v to the engine's kernel for the write into the cache (no rotation there)."""
+        pairs i with i + head_dim / 2).  The toy rotates with torch; the bias before it and the
+        write into the cache after it are the mixer's."""
 
         def __init__(self, head_dim: int, theta: float):
             self.head_dim, self.theta = head_dim, theta
 
-        def apply(self, qkv, n_heads, n_kv, head_dim, ctx, store, bias=None):
+        def rotate(self, qkv, n_heads, n_kv, head_dim, ctx):
             t = qkv.shape[0]
-            full = qkv.float() + (bias if bias is not None else 0.0)
+            full = qkv.float()
             rot = (n_heads + n_kv) * head_dim
             heads = full[:, :rot].reshape(t, n_heads + n_kv, head_dim // 2, 2)
             inv = self.theta ** (-2.0 * torch.arange(head_dim // 2, dtype=torch.float64, device=qkv.device) / head_dim)
@@ -75,10 +75,6 @@ def define_toys():
             a, b = heads[..., 0], heads[..., 1]
             full[:, :rot] = torch.stack((a * c - b * s, b * c + a * s), dim=-1).reshape(t, rot)
             qkv.copy_(full.to(qkv.dtype))
-            if store is None:
-                return
-            ops.rope_kv_write(qkv, ctx.positions, n_heads, n_kv, head_dim, None, slots=store.slots, k_pool=store.k_pool,
-                              v_pool=store.v_pool, page_size=store.page_size)
 
     @dataclass(frozen=True)
     class ToyConfig(ModelConfig):

@@ -53,18 +53,30 @@ LENGTHS = [330, 301, 77]
 PORTIONS = [7, 2, 16, 3, 2, 33, 5, 2, 64, 9, 130]
 
 
-def _rounded_plain(cfg, w, ids, rows=None):
+def _rounded_plain(cfg, w, ids, rows=None, many_rows=False):
     """The plain model with its activations rounded to bfloat16 where the bfloat16 engine rounds
-    them: the inputs of every product, q and k after the rotation, the gated activation."""
+    them: the inputs of every product, q and k after the rotation, the gated activation.
+    ``many_rows``: also what a step of many rows rounds (its products come from the library as
+    bfloat16, where steps of up to 128 rows keep float32 partial sums): the result of every product
+    but the head's, and the values as the cache keeps them."""
     r16 = lambda t: t.to(torch.bfloat16).float()
-    lin, rope, silu = plain.linear, plain.rope, plain.silu_mul
-    plain.linear = lambda x, wt, b=None: lin(r16(x), wt, b)
+    lin, rope, silu, att = plain.linear, plain.rope, plain.silu_mul, plain.attention
+
+    def linear(x, wt, b=None):
+        y = lin(r16(x), wt)
+        if many_rows and wt.shape[0] != cfg["vocab_size"]:
+            y = r16(y)
+        return y if b is None else y + b
+
+    plain.linear = linear
     plain.rope = lambda *a, **k: r16(rope(*a, **k))
     plain.silu_mul = lambda g, u: r16(silu(r16(g), r16(u)))
+    if many_rows:
+        plain.attention = lambda q, k, v, *a, **kw: att(q, k, r16(v), *a, **kw)
     try:
         return plain.forward(cfg, w, ids, rows=rows)
     finally:
-        plain.linear, plain.rope, plain.silu_mul = lin, rope, silu
+        plain.linear, plain.rope, plain.silu_mul, plain.attention = lin, rope, silu, att
 
 
 def _write_model(folder, raw, seed):
@@ -108,7 +120,7 @@ def wide(tmp_path_factory):
     long_ids = helpers.token_ids(WIDE["vocab_size"], 2048, 6000)
     rows = sorted({0, 1, 15, 16, 17, 255, 256, 1023, 1024, 2046, 2047} | set(range(100, 2048, 150)))
     long_ref = plain.forward(cfg, w, long_ids, rows=rows)
-    moved = _rounded_plain(cfg, w, long_ids, rows=rows) - long_ref
+    moved = _rounded_plain(cfg, w, long_ids, rows=rows, many_rows=True) - long_ref
     out["long"] = {"ids": long_ids, "rows": rows, "ref": long_ref,
                    "noise": (moved.abs().max().item(), moved.pow(2).mean().sqrt().item())}
     print("plain logits of the 2,048-token prompt done", flush=True)
