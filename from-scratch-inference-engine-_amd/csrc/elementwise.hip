@@ -7,6 +7,7 @@
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kWideNormRows = 8;  // up to so many rows, RMSNorm runs in workgroups of 1,024 threads
 
 // out[t, :] = table[ids[t], :] as float32.  An id outside the table gives a row of zeros; the
 // host refuses such ids before the launch.
@@ -105,8 +106,8 @@ __global__ void embedding_vec_kernel(const T* __restrict__ table, const int32_t*
 // DELTA: 0 = none, 1 = one array of T, 2 to 9 = that many float32 partial sums, added in
 // order (every load of the row goes out before anything waits); -1 = `n_parts` of them (any other
 // number: a loop, four loads ahead).
-template <typename T, int ITERS, int DELTA, bool WRITE_BACK>
-__global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+template <typename T, int ITERS, int DELTA, bool WRITE_BACK, int THREADS>
+__global__ __launch_bounds__(THREADS) void rmsnorm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta,
                                                                const float* __restrict__ weight, T* __restrict__ out,
                                                                const int32_t* __restrict__ rows, int hidden, float eps,
                                                                int64_t part_stride, int n_parts) {
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict
     float4 v[ITERS], d[ITERS], w[ITERS];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-        const int j = min((it * kThreads + static_cast<int>(threadIdx.x)) * 4, hidden - 4);
+        const int j = min((it * THREADS + static_cast<int>(threadIdx.x)) * 4, hidden - 4);
         v[it] = Pack4<float>::load(res + j);
         if (DELTA == 1) d[it] = Pack4<T>::load(del + j);
         if (DELTA > 1) {
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict
     float sum_sq = 0.f;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-        const int j = (it * kThreads + threadIdx.x) * 4;
+        const int j = (it * THREADS + threadIdx.x) * 4;
         if (HAS_DELTA) {
             v[it].x += d[it].x;
             v[it].y += d[it].y;
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_vec_kernel(float* __restrict
     T* dst = out + static_cast<int64_t>(r) * hidden;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-        const int j = (it * kThreads + threadIdx.x) * 4;
+        const int j = (it * THREADS + threadIdx.x) * 4;
         if (j < hidden) {
             Pack4<T>::store(dst + j, float4{(v[it].x * scale) * w[it].x, (v[it].y * scale) * w[it].y,
                                             (v[it].z * scale) * w[it].z, (v[it].w * scale) * w[it].w});
@@ -194,33 +195,33 @@ struct NormCall {
     hipStream_t stream;
 };
 
-template <typename T, int ITERS, int DELTA>
+template <typename T, int ITERS, int DELTA, int THREADS>
 void launch_rmsnorm_delta(const NormCall& c) {
     const T* d = static_cast<const T*>(c.delta);
     T* o = static_cast<T*>(c.out);
     if (c.write_back) {
-        rmsnorm_vec_kernel<T, ITERS, DELTA, DELTA != 0><<<c.n_rows, kThreads, 0, c.stream>>>(
+        rmsnorm_vec_kernel<T, ITERS, DELTA, DELTA != 0, THREADS><<<c.n_rows, THREADS, 0, c.stream>>>(
             c.residual, d, c.weight, o, c.rows, c.hidden, c.eps, c.part_stride, c.n_parts);
     } else {
-        rmsnorm_vec_kernel<T, ITERS, DELTA, false><<<c.n_rows, kThreads, 0, c.stream>>>(
+        rmsnorm_vec_kernel<T, ITERS, DELTA, false, THREADS><<<c.n_rows, THREADS, 0, c.stream>>>(
             c.residual, d, c.weight, o, c.rows, c.hidden, c.eps, c.part_stride, c.n_parts);
     }
 }
 
-template <typename T, int ITERS>
+template <typename T, int ITERS, int THREADS = kThreads>
 void launch_rmsnorm_vec(const NormCall& c) {
-    if (!c.delta) return launch_rmsnorm_delta<T, ITERS, 0>(c);
+    if (!c.delta) return launch_rmsnorm_delta<T, ITERS, 0, THREADS>(c);
     switch (c.n_parts) {
-        case 0: return launch_rmsnorm_delta<T, ITERS, 1>(c);
-        case 2: return launch_rmsnorm_delta<T, ITERS, 2>(c);
-        case 3: return launch_rmsnorm_delta<T, ITERS, 3>(c);
-        case 4: return launch_rmsnorm_delta<T, ITERS, 4>(c);
-        case 5: return launch_rmsnorm_delta<T, ITERS, 5>(c);
-        case 6: return launch_rmsnorm_delta<T, ITERS, 6>(c);
-        case 7: return launch_rmsnorm_delta<T, ITERS, 7>(c);
-        case 8: return launch_rmsnorm_delta<T, ITERS, 8>(c);
-        case 9: return launch_rmsnorm_delta<T, ITERS, 9>(c);
-        default: return launch_rmsnorm_delta<T, ITERS, -1>(c);
+        case 0: return launch_rmsnorm_delta<T, ITERS, 1, THREADS>(c);
+        case 2: return launch_rmsnorm_delta<T, ITERS, 2, THREADS>(c);
+        case 3: return launch_rmsnorm_delta<T, ITERS, 3, THREADS>(c);
+        case 4: return launch_rmsnorm_delta<T, ITERS, 4, THREADS>(c);
+        case 5: return launch_rmsnorm_delta<T, ITERS, 5, THREADS>(c);
+        case 6: return launch_rmsnorm_delta<T, ITERS, 6, THREADS>(c);
+        case 7: return launch_rmsnorm_delta<T, ITERS, 7, THREADS>(c);
+        case 8: return launch_rmsnorm_delta<T, ITERS, 8, THREADS>(c);
+        case 9: return launch_rmsnorm_delta<T, ITERS, 9, THREADS>(c);
+        default: return launch_rmsnorm_delta<T, ITERS, -1, THREADS>(c);
     }
 }
 
@@ -233,6 +234,14 @@ void launch_rmsnorm(const NormCall& c) {
     // values asks for five quads a thread and not for eight of which three repeat the last one
     const int per_iter = kThreads * 4;
     const int iters = (c.hidden + per_iter - 1) / per_iter;
+    // A few rows (decoding): a row and its partial sums (nine of them at hidden 3584 are 129 KB) come
+    // through one compute unit, which draws the more the more waves ask (some 50 GB/s with four waves,
+    // 125 with sixteen): workgroups of 1,024 threads, one or two quads a thread.
+    if (aligned && c.n_rows <= kWideNormRows && c.hidden >= 2048 && c.hidden <= 8192) {
+        if (c.hidden <= 4096) launch_rmsnorm_vec<T, 1, 1024>(c);
+        else launch_rmsnorm_vec<T, 2, 1024>(c);
+        return;
+    }
     if (aligned && c.hidden >= 4 && iters <= 8) {
         switch (iters) {
             case 1: launch_rmsnorm_vec<T, 1>(c); break;

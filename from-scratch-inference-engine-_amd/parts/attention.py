@@ -102,6 +102,10 @@ class AttentionPlanner:
         rows, shortest, room = (ops.attention_mfma_rows(self.head_dim, False), 128, 1) if mfma else (16, 64, 2)
         per_item = self.n_kv * -(-group // min(group, rows))  # workgroups of one item
         split = longest
+        if mfma and keys and len(keys) <= self.whole_requests and max(keys) <= longest:
+            # one or two requests whose keys fit one item: the item stays whole and the step has no
+            # merge at all; the waves of its workgroup deal the keys and combine through LDS
+            return longest
         # halved while the halves' workgroups still number at most the compute units: beyond that a
         # split only adds a merge (48 requests of 600 keys, 192 workgroups whole: 4.59 ms a step;
         # 384 of 512 keys each: 4.86).  The float32-arithmetic kernel's workgroups are slower and
@@ -142,6 +146,12 @@ class AttentionPlanner:
         return split
 
     long_items = True  # items beyond the longest of `geometry` where they still fill the device
+    # Steps of up to so many requests keep items that fit the longest whole (no merge launch).  0: never.
+    # MI355X, 28/4 heads of 128, 640 keys a request, a decode step at batch 1 / 2 / 4: 3.10 / 3.11 / 3.12 ms
+    # whole against 3.04 / 3.06 / 3.07 in items of 128 keys with a merge: a wave of the many-wave
+    # workgroup walks its keys two blocks at a time (a trip to memory each), the one-wave item asks
+    # for all four blocks at once, which the registers of eight waves a workgroup do not allow.
+    whole_requests = 0
 
     @staticmethod
     def _items_of(keys: int, split_keys: int, longest: int) -> int:
