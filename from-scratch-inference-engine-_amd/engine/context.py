@@ -43,10 +43,8 @@ def padded_tokens(n: int) -> int:
     """Rows of a step that is not a decode step, once filled up (done while the library's kernels
     are chosen by timing): up to 64 as they are, then 128, then the next multiple of 256 where that
     adds at most a fifth (or 64 rows).  Only these counts are timed (a count costs seconds the first
-    time it comes), and a timed choice is up to a fifth faster than the library's own (28 layers of
-    3584 / 18944 on MI355X, ms as they are / filled up: 100 tokens 6.9 / 6.0, 200 8.6 / 7.2, 448 12.7 / 10.5,
-    1,000 18.9 / 17.1, 3,000 45.5 / 37.4; 300 tokens, 8.7 ms, would take 10.4 as 512 and stay as they
-    are).  Without the timing the filled-up step is no faster than the step as it is."""
+    time it comes), and a timed choice is up to a fifth faster than the library's own; without the
+    timing the filled-up step is no faster than the step as it is."""
     if n <= 64:
         return n
     if n <= 128:

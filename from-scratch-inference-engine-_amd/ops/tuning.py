@@ -2,8 +2,7 @@
 
 For many rows (prefill) the engine hands x . W^T to the vendor library through ``torch.mm`` (the
 reference's engine calls cuBLAS there).  The library picks one of its kernels by a heuristic; its
-other kernels are sometimes a good deal faster (measured on MI355X at 2,048 rows: 462 against
-568 us for N = 37888, K = 3584, and 261 against 357 us for N = 3584, K = 18944).  With tuning on,
+other kernels are sometimes a fifth or a quarter faster.  With tuning on,
 torch's TunableOp times the library's candidates the first time a shape is seen and keeps the
 best (in the process, and in a file under the temporary folder for later ones).  Each new shape
 costs seconds (at 16,384 rows, minutes), so only two kinds of row counts are tuned: multiples of 256

@@ -37,9 +37,8 @@ class AttentionPlanner:
     a multiple of 4) and the float32-arithmetic kernel for everything else; which one a step
     uses follows from the step's dtype and page size."""
 
-    # Keys above which a large tile is given four waves that split its keys.  Off: on MI355X a
-    # 2,048-token prefill at 28/4 heads of 128 took 235 us per layer with 512 against 176 us
-    # without (idle waves in the four-wave workgroups cost more than the balance gains).
+    # Keys above which a large tile is given four waves that split its keys.  Off: idle waves in
+    # the four-wave workgroups cost more than the balance gains.
     long_keys: Optional[int] = None
     # Compute units to fill with the workgroups of small items; None: those of the device.
     compute_units: Optional[int] = None
@@ -87,12 +86,9 @@ class AttentionPlanner:
         return keys
 
     def split_keys(self, host, mfma: bool) -> int:
-        """Keys per small item in this step.  A workgroup draws only some 50 GB/s from memory, so a
-        step with few requests is faster with more, shorter items, although they cost a merge
-        (MI355X, 28/4 heads of 128, per layer: 8 requests of 640 keys 10.7 us with 256 keys an
-        item against 12.2 with 1,024; one request of 3,550 keys 11.3 against 18.2; 64 requests of
-        640 keys 24.8 against 18.3, which is why a full device keeps the long items; items of 128
-        keys, one wave each, gain another per cent of a decode step of one to eight requests)."""
+        """Keys per small item in this step.  A workgroup draws only so much from memory, so a step
+        with few requests is faster with more, shorter items although they cost a merge, and a full
+        device keeps the long ones."""
         small_tokens, _, longest = self.geometry(mfma)
         units = self.compute_units if self.compute_units is not None else ops.compute_units()
         keys = self._small_keys(host, small_tokens)
@@ -107,26 +103,19 @@ class AttentionPlanner:
             # merge at all; the waves of its workgroup deal the keys and combine through LDS
             return longest
         # halved while the halves' workgroups still number at most the compute units: beyond that a
-        # split only adds a merge (48 requests of 600 keys, 192 workgroups whole: 4.59 ms a step;
-        # 384 of 512 keys each: 4.86).  The float32-arithmetic kernel's workgroups are slower and
-        # several share a unit: twice the units (8 requests of 640 keys, 28 layers of the 32-bit
-        # path: 8.5 ms a step with 64 keys an item, 9.1 with 128)
+        # split only adds a merge.  The float32-arithmetic kernel's workgroups are slower and several
+        # share a unit: twice the units.
         while split > shortest and sum(-(-k // (split // 2)) for k in keys) * per_item < units * room:
             split //= 2
         # requests that fit one item each need no merge at all while they stay whole: cutting them in
-        # two is not worth one (32 requests of 600 keys: 4.04 ms a step whole, 4.14 in halves; 24:
-        # 4.17 against 4.27), in three or more it is (8 requests in five: 3.55 against 3.60)
+        # two is not worth one, in three or more it is
         if keys and split < longest and max(keys) <= longest and -(-max(keys) // split) <= 2:
             return longest
         # Items of the matrix-core kernel may be longer: the waves of a workgroup deal an item's keys
         # among themselves, and an item more for a request costs the work before the walk again and
         # a merge.  Where the requests alone give every compute unit a workgroup they stay whole,
-        # however long (MI355X, a step of 64 requests at 28/4 heads of 128: 2,000 keys each 4.92 ms
-        # whole against 5.52 in items of 1,024, 3,500 keys 5.76 against 6.34; 64 requests of 1,040
-        # keys at 40/8 heads 15.8 against 17.6, where the second item had 16 keys).  Fewer requests
-        # take the longest items of which the full ones still number the units (8 requests of 16,000
-        # keys at 40/8 heads: 16.6 ms in items of 2,048 against 17.2 in items of 1,024); fewer workgroups than units lose
-        # (48 requests of 2,000 keys whole: 6.1 ms against 4.8).
+        # however long.  Fewer requests take the longest items of which the full ones still number the
+        # units; fewer workgroups than units lose.
         if self.long_items and mfma and keys and split == longest and units > 0 and max(keys) > longest:
             long = longest
             while long < max(keys):
@@ -146,11 +135,9 @@ class AttentionPlanner:
         return split
 
     long_items = True  # items beyond the longest of `geometry` where they still fill the device
-    # Steps of up to so many requests keep items that fit the longest whole (no merge launch).  0: never.
-    # MI355X, 28/4 heads of 128, 640 keys a request, a decode step at batch 1 / 2 / 4: 3.10 / 3.11 / 3.12 ms
-    # whole against 3.04 / 3.06 / 3.07 in items of 128 keys with a merge: a wave of the many-wave
-    # workgroup walks its keys two blocks at a time (a trip to memory each), the one-wave item asks
-    # for all four blocks at once, which the registers of eight waves a workgroup do not allow.
+    # Steps of up to so many requests keep items that fit the longest whole (no merge launch).  0:
+    # never, which is faster: the one-wave item asks for all its blocks of keys at once, a wave of the
+    # many-wave workgroup for two at a time.
     whole_requests = 0
 
     @staticmethod

@@ -60,17 +60,13 @@ class SwiGLU(FeedForward):
         m = x.shape[0]
         if (x.dtype == torch.bfloat16 and self.gate_up.streamed is not None and 0 < m <= self.streamed_swiglu_max_rows
                 and self.gate_up.wide_takes(m, 1, gate_up=True)):
-            # from the fragment-ordered copy at any number of rows up to 64, and up to 128 where the kernel
-            # has the launch shape for it (MI355X, N = 37888, K = 3584: 44 us for 1 to 16 rows, where the
-            # few-rows kernel takes 49 to 55 on rows; 49 at 64 rows, 52 at 96, 54 at 112, where the library
-            # and a SiLU*up kernel take 66, 69 and 75)
+            # from the fragment-ordered copy at any number of rows up to 64, and up to 128 where the
+            # kernel has the launch shape for it: SiLU*up in the product's epilogue
             act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.streamed)
         elif (x.dtype == torch.bfloat16 and 3 <= m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 128 == 0
                 and self.gate_up.out_features % 4 == 0 and self.gate_up.out_features // 64 >= ops.compute_units()):
             # three rows and more of a matrix that gives every compute unit a workgroup: the kernel that
-            # shares x through LDS (MI355X, 8 rows: N = 37888, K = 3584 49.3 against 51.2 us; N = 27648,
-            # K = 5120 57.2 against 62.4; N = 55296, K = 5120 110.5 against 118.7, at 16 rows 106 against
-            # 129; one or two rows, and N = 9728, K = 896, are faster in the other)
+            # shares x through LDS (one or two rows, and small matrices, are faster in the other)
             act = ops.gemm_mfma_wide_swiglu(x, self.gate_up.weight)
         elif x.dtype == torch.bfloat16 and m <= GEMM_MFMA_SKINNY_BEST_M and self.hidden_size % 8 == 0:
             act = ops.gemm_mfma_skinny(x, self.gate_up.weight, epilogue="swiglu")
