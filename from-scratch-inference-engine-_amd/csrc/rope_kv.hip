@@ -188,7 +188,7 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
     if (TOK == 8 && run) {
         const int64_t page = slot[0] / page_size;
         const int off = slot[0] % page_size;
-        for (int idx = threadIdx.x; idx < kv_dim; idx += kThreads) {  // lanes over the dimensions: rows read whole
+        for (int idx = first; idx < kv_dim; idx += stride) {  // lanes over the dimensions: rows read whole
             const int kvh = idx / head_dim;
             const int d = idx - kvh * head_dim;
             const float b = HAS_BIAS ? bias[q_dim + kv_dim + idx] : 0.f;
@@ -223,10 +223,14 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
         }
     }
 
-    // ---- q and k heads: unit u of a token = four pairs of one head; the tokens of the block in turn
+    // ---- q and k heads: unit u of a token = four pairs of one head.  The block's (token, unit) pairs are
+    // dealt to the threads of its gridDim.y blocks token by token, so that neighbouring threads take
+    // neighbouring units of one token's row
     const int quads = half / 4;
     const int n_units = (n_heads + n_kv) * quads;
-    for (int u = first; u < n_units; u += stride) {
+    for (int w = first; w < n_units * n_here; w += stride) {
+        const int j = TOK == 1 ? 0 : w / n_units;
+        const int u = TOK == 1 ? w : w - j * n_units;
         const int h = u / quads;
         const int i = (u - h * quads) * 4;
         float4 b1{0.f, 0.f, 0.f, 0.f}, b2{0.f, 0.f, 0.f, 0.f};
@@ -234,31 +238,30 @@ __global__ __launch_bounds__(kThreads) void rope_kv_write_table_kernel(
             b1 = *reinterpret_cast<const float4*>(bias + h * head_dim + i);
             b2 = *reinterpret_cast<const float4*>(bias + h * head_dim + i + half);
         }
+        const int t = t0 + j;
+        T* head = qkv + static_cast<int64_t>(t) * width + h * head_dim;
+        float4 a1 = load4(t, h * head_dim + i), a2 = load4(t, h * head_dim + i + half);
+        a1 = float4{a1.x + b1.x, a1.y + b1.y, a1.z + b1.z, a1.w + b1.w};
+        a2 = float4{a2.x + b2.x, a2.y + b2.y, a2.z + b2.z, a2.w + b2.w};
+        const float4* cs = reinterpret_cast<const float4*>(cos_sin + static_cast<int64_t>(t) * head_dim);
+        const float4 c01 = cs[i / 2], c23 = cs[i / 2 + 1];  // (cos, sin) of pairs i, i + 1 and i + 2, i + 3
+        const float4 r1{a1.x * c01.x - a2.x * c01.y, a1.y * c01.z - a2.y * c01.w, a1.z * c23.x - a2.z * c23.y,
+                        a1.w * c23.z - a2.w * c23.w};
+        const float4 r2{a2.x * c01.x + a1.x * c01.y, a2.y * c01.z + a1.y * c01.w, a2.z * c23.x + a1.z * c23.y,
+                        a2.w * c23.z + a1.w * c23.w};
+        if (!PARTS || h < n_heads) {
+            Quad<T>::store(head + i, r1);
+            Quad<T>::store(head + i + half, r2);
+        }
+        int sl = slot[0];
 #pragma unroll
-        for (int j = 0; j < TOK; ++j) {
-            if (j >= n_here) break;
-            const int t = t0 + j;
-            T* head = qkv + static_cast<int64_t>(t) * width + h * head_dim;
-            float4 a1 = load4(t, h * head_dim + i), a2 = load4(t, h * head_dim + i + half);
-            a1 = float4{a1.x + b1.x, a1.y + b1.y, a1.z + b1.z, a1.w + b1.w};
-            a2 = float4{a2.x + b2.x, a2.y + b2.y, a2.z + b2.z, a2.w + b2.w};
-            const float4* cs = reinterpret_cast<const float4*>(cos_sin + static_cast<int64_t>(t) * head_dim);
-            const float4 c01 = cs[i / 2], c23 = cs[i / 2 + 1];  // (cos, sin) of pairs i, i + 1 and i + 2, i + 3
-            const float4 r1{a1.x * c01.x - a2.x * c01.y, a1.y * c01.z - a2.y * c01.w, a1.z * c23.x - a2.z * c23.y,
-                            a1.w * c23.z - a2.w * c23.w};
-            const float4 r2{a2.x * c01.x + a1.x * c01.y, a2.y * c01.z + a1.y * c01.w, a2.z * c23.x + a1.z * c23.y,
-                            a2.w * c23.z + a1.w * c23.w};
-            if (!PARTS || h < n_heads) {
-                Quad<T>::store(head + i, r1);
-                Quad<T>::store(head + i + half, r2);
-            }
-            if (h >= n_heads && slot[j] >= 0) {
-                const int64_t page = slot[j] / page_size;
-                const int off = slot[j] % page_size;
-                T* dst = k_pool + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
-                Quad<T>::store(dst + i, r1);
-                Quad<T>::store(dst + i + half, r2);
-            }
+        for (int q = 1; q < TOK; ++q) sl = j == q ? slot[q] : sl;
+        if (h >= n_heads && sl >= 0) {
+            const int64_t page = sl / page_size;
+            const int off = sl % page_size;
+            T* dst = k_pool + ((page * n_kv + (h - n_heads)) * page_size + off) * head_dim;
+            Quad<T>::store(dst + i, r1);
+            Quad<T>::store(dst + i + half, r2);
         }
     }
 }
@@ -338,7 +341,8 @@ extern "C" int fsie_rope_kv_write_table(void* qkv, const float* cos_sin, const i
     const int write_kv = (k_pool && v_pool && slots) ? 1 : 0;
     FSIE_REQUIRE(!write_kv || (page_size > 0 && pool_slots > 0), "rope_kv_write_table: bad page geometry");
     if (n_tokens == 0) return 0;
-    // eight tokens a block where there are enough blocks left to fill the device
+    // eight tokens a block where there are enough blocks left to fill the device, four blocks a run of eight
+    // tokens: the kernel is made of loads that wait for memory, so it wants many waves on every unit
     // blocks a token: so many that the device's units all have one (64 tokens of 4,608 columns in 7 partial
     // sums on MI355X: 9.0 us with one block a token)
     const int units = fsie_compute_units();
@@ -361,7 +365,7 @@ extern "C" int fsie_rope_kv_write_table(void* qkv, const float* cos_sin, const i
 #define FSIE_ROPE_LAUNCH(T, B)                                                                                    \
     do {                                                                                                          \
         if (n_tokens >= 1024)                                                                                     \
-            rope_kv_write_table_kernel<T, B, 8><<<(n_tokens + 7) / 8, kThreads, 0, stream>>>(                     \
+            rope_kv_write_table_kernel<T, B, 8><<<dim3((n_tokens + 7) / 8, 4), kThreads, 0, stream>>>(            \
                 static_cast<T*>(qkv), cos_sin, slots, bias, static_cast<T*>(k_pool), static_cast<T*>(v_pool),     \
                 n_tokens, n_heads, n_kv, head_dim, page_size, write_kv, pool_slots);                              \
         else                                                                                                      \

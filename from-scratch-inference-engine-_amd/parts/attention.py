@@ -201,7 +201,10 @@ class AttentionPlanner:
                     nq = min(large_tokens, n - t0)
                     pos0 = p + t0
                     kb = max(0, pos0 - self.window + 1) if self.window else 0
-                    (small if nq <= small_tokens else large).append((s, row0 + t0, nq, pos0, kb, pos0 + nq, -1, 0))
+                    # (the short tile that a long portion may end with stays with the portion's other tiles:
+                    # as a small item it would walk all the portion's keys in one workgroup a kv head, alone
+                    # on the device, while as the last of a group of four it shares their blocks of keys)
+                    large.append((s, row0 + t0, nq, pos0, kb, pos0 + nq, -1, 0))
         waves = 1
         if mfma and small:
             waves = self._waves_for(max(it[5] - it[4] for it in small), ops.attention_mfma_max_waves(self.head_dim))

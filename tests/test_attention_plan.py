@@ -185,3 +185,23 @@ def test_graph_bucket_pads_plans_of_decode_steps():
             assert plan["n_merges"] == len(lens)  # every row gets a merge entry, empty where none is needed
     # a step with a portion is no decode step
     assert planner.graph_bucket(Host([(10, 1), (0, 40)], 16, torch.bfloat16)) is None
+
+
+def test_the_short_tile_at_the_end_of_a_long_portion_stays_with_its_group():
+    """40 query heads on 8 kv heads give tiles of six tokens: a portion of 2,048 tokens ends with a tile
+    of two.  That tile is the last of its group of four, not a small item of its own (which would
+    walk thousands of keys in one workgroup a kv head while the device idles)."""
+    planner = AttentionPlanner(40, 8, 128, None)
+    host = Host([(4096, 2048), (0, 1)], 16, torch.bfloat16)
+    plan = planner.plan(host)
+    check_plan(planner, host, plan)
+    small, large, most = planner.geometry(True)
+    assert large == 6 and 2048 % large == 2
+    items, groups = plan["items"], plan["groups"]
+    assert plan["n_small"] == 1 and int(items[0][SEQ]) == 1          # the decoded token of the other request
+    tiles = items[plan["n_small"]:]
+    assert len(tiles) == -(-2048 // large) and int(tiles[-1][NQ]) == 2
+    covered = sorted(i for g in groups for i in range(int(g[0]), int(g[0]) + int(g[1])))
+    assert covered == list(range(len(tiles))), "every tile, the short one too, is in a group"
+    last = max(groups, key=lambda g: int(g[0]) + int(g[1]))
+    assert int(last[0]) + int(last[1]) == len(tiles) and int(last[1]) >= 2
