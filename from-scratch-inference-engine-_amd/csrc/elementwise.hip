@@ -7,7 +7,7 @@
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kWideNormRows = 8;  // up to so many rows, RMSNorm runs in workgroups of 1,024 threads
+constexpr int kWideNormRows = 128;  // up to so many rows (half the device's units), RMSNorm runs in workgroups of 1,024 threads
 
 // out[t, :] = table[ids[t], :] as float32.  An id outside the table gives a row of zeros; the
 // host refuses such ids before the launch.
@@ -234,7 +234,7 @@ void launch_rmsnorm(const NormCall& c) {
     // values asks for five quads a thread and not for eight of which three repeat the last one
     const int per_iter = kThreads * 4;
     const int iters = (c.hidden + per_iter - 1) / per_iter;
-    // A few rows (decoding): a row and its partial sums (nine of them at hidden 3584 are 129 KB) come
+    // Decoding (up to 128 rows): a row and its partial sums (nine of them at hidden 3584 are 129 KB) come
     // through one compute unit, which draws the more the more waves ask (some 50 GB/s with four waves,
     // 125 with sixteen): workgroups of 1,024 threads, one or two quads a thread.
     if (aligned && c.n_rows <= kWideNormRows && c.hidden >= 2048 && c.hidden <= 8192) {

@@ -30,11 +30,13 @@ class Linear:
     float32_on_matrix_cores = True  # up to 64 rows of float32: v_mfma_f32_16x16x4_f32 instead of vector FMAs
     # A bfloat16 weight of at least this many bytes is kept a second time, in the order of the matrix
     # instruction's fragments, for the engine's own products (decoding): a wave then loads 1 KB in one
-    # piece with streaming loads, where rows give it 16 pieces of 64 bytes.  Matrices below some 48 MB
-    # gain nothing from it.  The rows stay for the library's products of many rows.  None: no copies.
+    # piece with streaming loads, where rows give it 16 pieces of 64 bytes (a compute unit draws about
+    # half as much when a wave's load is pieces of rows).  From 16 MB on: the q/k/v and output
+    # projections of a 7B model (33 and 26 MB) gain by it.  The rows stay for the library's products of
+    # many rows.  None: no copies.
     # A copy that would leave less than ``streamed_copy_reserve`` of the device's memory free is not
     # made: a model that large keeps copies of its first layers only and runs the rest from rows.
-    streamed_copy_from = 48 << 20
+    streamed_copy_from = 16 << 20
     streamed_copy_reserve = 0.25
 
     def __init__(self, in_features: int, out_features: int, bias: bool = False):
