@@ -461,6 +461,11 @@ __global__ __launch_bounds__(QKV && MAXW == 1 ? 256 : 64 * MAXW) __attribute__((
     // QKV: the new key and value, from the sums: a block of their own whose first key they are (the
     // mask hides the rest), and into the pools for the steps to come.  An idle wave does it, or the
     // first one before its walk, while its first keys from the cache are under way.
+    // The stores into the pools (2 bytes a dimension for the value) are not ordered against the loads of
+    // other waves and workgroups that read the 16 bytes around that slot: those lanes are masked
+    // (probability zero), so the result does not depend on which bytes they see, provided they are
+    // finite either way.  That is the pools' invariant: a slot at or after a request's length holds a
+    // finite value (a page is zeroed by the step that takes it; the null page is never written).
     auto score_new_key = [&]() {
         if (!(owner && wave == new_key_wave)) return;
         key_end = pos0 + 1;

@@ -135,8 +135,22 @@ class Model:
 
     # ---------------------------------------------------------------- cache
     def make_cache(self, page_size: int, num_pages: int, max_requests: int):
+        """The cache's host and device side.  The second copies of the large weights were made before
+        the cache's size was known: if the pools do not fit beside them, the copies go (decode steps
+        then read rows, some 8 % slower) and the pools are asked for once more."""
         manager = CacheManager(self.cache_layout.paged_groups, page_size, num_pages, max_requests)
-        storage = CacheStorage(self.cache_layout, manager, self.device, self.dtype)
+        try:
+            storage = CacheStorage(self.cache_layout, manager, self.device, self.dtype)
+        except torch.cuda.OutOfMemoryError:
+            freed = sum(part.release_optional_memory() for part in self.spec.all_parts())
+            if not freed:
+                raise
+            torch.cuda.empty_cache()
+            import warnings
+
+            warnings.warn(f"the cache of {num_pages} pages did not fit beside the second copies of the large weights: "
+                          f"{freed / 2 ** 30:.1f} GiB of copies dropped (as with weight_copies=False)")
+            storage = CacheStorage(self.cache_layout, manager, self.device, self.dtype)
         return manager, storage
 
     def cache_bytes_per_token(self) -> int:

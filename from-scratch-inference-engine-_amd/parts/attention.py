@@ -319,6 +319,9 @@ class GQAttention(Mixer):
         self.o.prepare(copies)
         self.qkv.prepare(copies)  # (read by the product of 17 to 64 rows; the few-rows product with the rotation reads rows)
 
+    def release_optional_memory(self) -> int:
+        return self.qkv.drop_copy() + self.o.drop_copy()
+
     # cache and plan ---------------------------------------------------------------------
     def cache_need(self) -> PagedNeed:
         return PagedNeed(self.n_kv, self.head_dim, self.window)

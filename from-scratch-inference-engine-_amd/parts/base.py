@@ -74,6 +74,11 @@ class Part:
     def prepare(self, device, compute_dtype: torch.dtype) -> None:
         """Called once after the parameters are set (tables, constants on the device)."""
 
+    def release_optional_memory(self) -> int:
+        """Give back device memory that the part can work without (second copies of weights in
+        another order); returns the bytes.  Called when the cache does not fit beside them."""
+        return 0
+
     def sub_parts(self) -> Dict[str, "Part"]:
         """The parts this one is made of (a block's norms, mixer and feed-forward; a mixer's
         position encoding and the norms of its heads).  The model prepares them, asks them for

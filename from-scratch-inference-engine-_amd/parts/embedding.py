@@ -54,5 +54,8 @@ class LMHead(Part):
     def prepare(self, device, compute_dtype) -> None:
         self.linear.prepare(bool(self.options.get("weight_copies", True)))
 
+    def release_optional_memory(self) -> int:
+        return self.linear.drop_copy()
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.linear(x, out_dtype=torch.float32)

@@ -69,6 +69,15 @@ class Linear:
             if free - w.numel() * 2 >= self.streamed_copy_reserve * total:
                 self.streamed = ops.fragment_order(w)
 
+    def drop_copy(self) -> int:
+        """Forget the fragment-ordered copy (the products then read rows); returns its bytes."""
+        if self.streamed is None:
+            return 0
+        freed = self.streamed.data.numel() * self.streamed.data.element_size()
+        self.streamed = None
+        self._wide_takes = {}
+        return freed
+
     @property
     def wide_weight(self):
         """What the products that share x through LDS read: the fragment-ordered copy if there is one."""

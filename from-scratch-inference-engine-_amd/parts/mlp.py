@@ -52,6 +52,9 @@ class SwiGLU(FeedForward):
         self.gate_up.prepare(copies)
         self.down.prepare(copies)
 
+    def release_optional_memory(self) -> int:
+        return self.gate_up.drop_copy() + self.down.drop_copy()
+
     # rows up to which silu(gate) * up comes from the product that shares x through LDS when the weight
     # has a fragment-ordered copy (beyond: the library's product and a kernel for SiLU*up)
     streamed_swiglu_max_rows = 128

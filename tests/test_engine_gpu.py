@@ -616,6 +616,48 @@ def test_decoding_from_fragment_ordered_copies(tmp_path, monkeypatch):
     assert lin.streamed is None
 
 
+def test_a_cache_that_does_not_fit_beside_the_weight_copies_drops_them(tmp_path, monkeypatch):
+    """The second copies of the large weights are made when the model is loaded, before anybody
+    knows how large the cache will be.  If the pools then do not fit, the copies go and the pools
+    are asked for again; the model decodes from rows and gives the same tokens.  (The first request
+    for the pools is made to fail from the host: no memory is exhausted here.)"""
+    import warnings
+
+    from from_scratch_inference_engine_amd import LLM, Engine, GenerationConfig, SamplingParams
+    from from_scratch_inference_engine_amd.cache import storage as storage_module
+    from from_scratch_inference_engine_amd.parts.linear import Linear
+
+    monkeypatch.setattr(Linear, "streamed_copy_from", 0)  # every matrix of the tiny model has a copy
+    cfg = dict(helpers.TINY_B, hidden_size=256, num_attention_heads=8, head_dim=32, intermediate_size=384)
+    d = helpers.make_model_dir(tmp_path / "m", cfg, seed=5)
+    llm = LLM(d, dtype="bfloat16", block_size=8, num_blocks=32, max_batch=4, eos_id=-1)
+    mixer = llm.model.spec.layers[0].mixer
+    assert mixer.o.streamed is not None and llm.model.spec.lm_head.linear.streamed is not None
+    prompts = [helpers.token_ids(509, n, 1600 + n) for n in (5, 19)]
+    gen = GenerationConfig(max_tokens=10, temperature=0.0)
+    with_copies = llm.generate_ids_batch(prompts, gen)
+
+    real_init = storage_module.CacheStorage.__init__
+    failed = []
+
+    def init(self, *a, **k):
+        if not failed:
+            failed.append(1)
+            raise torch.cuda.OutOfMemoryError("(the test says so)")
+        real_init(self, *a, **k)
+
+    monkeypatch.setattr(storage_module.CacheStorage, "__init__", init)
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        engine = Engine(llm.model, block_size=8, num_blocks=32, max_batch=4)
+    assert failed and any("copies dropped" in str(w.message) for w in caught)
+    assert all(lin.streamed is None for block in llm.model.spec.layers
+               for lin in (block.mixer.qkv, block.mixer.o, block.ffn.gate_up, block.ffn.down))
+    assert llm.model.spec.lm_head.linear.streamed is None
+    without = engine.generate_batch(prompts, SamplingParams(temperature=0.0), max_tokens=10)
+    assert without == with_copies  # (the products on the copy and on rows give the same bits)
+
+
 def test_prefill_with_the_library_kernel_selection(model_dirs):
     """With tuning on, a prompt portion of a multiple of 256 rows, and a decode batch of a multiple
     of 16, let torch time the library's candidates for their products; whatever it picks, the
@@ -838,8 +880,9 @@ def test_more_requests_than_a_step_has_tokens_for(llms, model_dirs):
     assert engine.free_blocks() == 64
 
 
-def _model_with_one_loud_key(tmp_path, special):
-    """The second tiny configuration with its first layer arranged so that every query gives
+def _model_with_one_loud_key(tmp_path, special, layer=0):
+    """The second tiny configuration with one layer (the first, or a later one, whose input still
+    carries the token's embedding beside the small sums of the layers before) arranged so that every query gives
     nearly all of its attention to the keys of one token, wherever it stands: dimension 15 of the
     key (the slowest-turning rotary pair: the rotation leaves it alone over thousands of positions)
     reads how much the normed input looks like that token's, and every query head carries a
@@ -847,27 +890,29 @@ def _model_with_one_loud_key(tmp_path, special):
     that is missed or taken from the wrong page; here the logits move by a whole unit."""
     cfg = dict(helpers.TINY_B, max_position_embeddings=2048)
     t = {k: v.float() for k, v in helpers.random_tensors(cfg, 1).items()}
-    n = plain.rms_norm(t["model.embed_tokens.weight"][special][None], t["model.layers.0.input_layernorm.weight"], 1e-5)[0]
-    t["model.layers.0.self_attn.k_proj.weight"][15] = 8.0 * n / (n @ n)
-    t["model.layers.0.self_attn.k_proj.bias"][15] = 0.0
+    p = f"model.layers.{layer}."
+    n = plain.rms_norm(t["model.embed_tokens.weight"][special][None], t[p + "input_layernorm.weight"], 1e-5)[0]
+    t[p + "self_attn.k_proj.weight"][15] = 8.0 * n / (n @ n)
+    t[p + "self_attn.k_proj.bias"][15] = 0.0
     for h in range(6):
-        t["model.layers.0.self_attn.q_proj.weight"][h * 32 + 15] = 0.0
-        t["model.layers.0.self_attn.q_proj.bias"][h * 32 + 15] = 40.0
+        t[p + "self_attn.q_proj.weight"][h * 32 + 15] = 0.0
+        t[p + "self_attn.q_proj.bias"][h * 32 + 15] = 40.0
     return helpers.make_model_dir(tmp_path / "loud", cfg, 1, tensors={k: v.to(torch.bfloat16).contiguous() for k, v in t.items()})
 
 
-@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
-def test_the_model_finds_one_far_key_through_its_own_tables(tmp_path, dtype):
+@pytest.mark.parametrize("dtype, layer", [("bfloat16", 0), ("float32", 0), ("bfloat16", 2)])
+def test_the_model_finds_one_far_key_through_its_own_tables(tmp_path, dtype, layer):
     """Three requests whose loud token stands at position 2, at the last slot of a page and 1,200
     tokens back: prefilled in portions beside each other's decoded tokens, then decoded together
     (eagerly and through graphs).  What the step function's tables and the attention plan hand
-    to the kernels decides the logits here."""
+    to the kernels decides the logits here.  With the last layer made loud instead of the first, a
+    key taken from another layer's plane of the pool shows in bfloat16 too."""
     from from_scratch_inference_engine_amd import load_model
     from from_scratch_inference_engine_amd.engine.context import StepEntry
     from from_scratch_inference_engine_amd.engine.model import Runner
 
     special = 100
-    d = _model_with_one_loud_key(tmp_path, special)
+    d = _model_with_one_loud_key(tmp_path, special, layer)
     seqs = []
     for n, where, seed in ((700, 2, 1), (420, 335, 2), (1500, 287, 3)):
         ids = [t if t != special else special + 1 for t in helpers.token_ids(509, n, 880 + seed)]
@@ -935,6 +980,69 @@ def test_what_an_earlier_request_left_in_its_pages_does_not_reach_the_next(model
                 fed[i] += n
         assert fed == [len(s_) for s_ in seqs]
         assert not torch.isnan(k[:, 0]).any() and (k[:, 0] == 0).all() and (v[:, 0] == 0).all()  # the null page stays empty
+
+
+def test_nan_in_the_pools_and_the_attention_that_finishes_qkv_itself(tmp_path):
+    """The same for the kernel of steps of one token a request, which writes the new key and value
+    into the pools while other waves of its workgroup read the 16 bytes around that place (masked
+    by a probability of zero): what lies in the slots at and after a request's length must be
+    finite, and it is, because a page is zeroed by the step that takes it, whatever an earlier
+    request left there.  A configuration that this kernel takes (head size 32, pages of 8, a hidden
+    size of 1,024 that the sliced product takes); requests decode across the edges of their pages, in pages
+    that another request, closed meanwhile, had filled."""
+    from from_scratch_inference_engine_amd import load_model, ops
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    cfg = dict(WIDE, head_dim=32, num_attention_heads=8, max_position_embeddings=256)  # hidden 1,024: two slices of K
+    d = helpers.make_model_dir(tmp_path / "m", cfg, seed=77)
+    model = load_model(d, dtype="bfloat16")
+    seqs = [helpers.token_ids(331, n, 1500 + n) for n in (29, 14, 21)]
+    refs = [plain.forward_dir(d, ids).numpy() for ids in seqs]
+    calls = []
+    real = ops.attention_mfma_qkv
+    ops.attention_mfma_qkv = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+    try:
+        for graphs in (False, True):
+            runner = Runner(model, page_size=8, num_pages=9, max_requests=3, use_graphs=graphs)
+            k, v, _ = runner.storage.group_stores[0]
+            k[:, 1:] = float("nan")
+            v[:, 1:] = float("nan")
+            calls.clear()
+            a, b = runner.manager.open("a"), runner.manager.open("b")
+            fed = {"a": 0, "b": 0, "c": 0}
+            which = {"a": 0, "b": 1, "c": 2}
+            caches = {"a": a, "b": b}
+
+            def step(items):
+                entries = [StepEntry(caches[r], seqs[which[r]][fed[r]:fed[r] + n], list(range(n))) for r, n in items]
+                out = runner.step(entries).float().cpu().numpy()
+                row = 0
+                for r, n in items:
+                    helpers.assert_close_to_plain(out[row:row + n], refs[which[r]][fed[r]:fed[r] + n], "bfloat16",
+                                                  f"graphs={graphs} request {r} at {fed[r]}")
+                    row += n
+                    fed[r] += n
+
+            step([("a", 5), ("b", 6)])
+            for _ in range(8):                     # both decode over the edge of their first page (8)
+                step([("a", 1), ("b", 1)])
+            runner.manager.close(caches.pop("b"))  # b's two pages, filled with its keys, go back ...
+            k[:, 1:][torch.isfinite(k[:, 1:])] = float("nan")  # ... and whatever they held is made worse
+            v[:, 1:][torch.isfinite(v[:, 1:])] = float("nan")
+            caches["c"] = runner.manager.open("c")
+            # a's keys are gone with that (they were finite): it starts again in pages of its own
+            runner.manager.close(caches.pop("a"))
+            caches["a"] = runner.manager.open("a")
+            fed["a"] = 0
+            step([("a", 9), ("c", 3)])
+            for _ in range(18):                    # c runs into b's old pages, one token a step, a beside it
+                step([("a", 1), ("c", 1)])
+            assert fed == {"a": 27, "b": 14, "c": 21}
+            assert len(calls) >= (26 * 2 if not graphs else 2), "the kernel that finishes q/k/v ran"
+            assert (k[:, 0] == 0).all() and (v[:, 0] == 0).all()
+    finally:
+        ops.attention_mfma_qkv = real
 
 
 def test_steps_filled_up_to_the_timed_row_counts_of_256_and_more(tmp_path):
