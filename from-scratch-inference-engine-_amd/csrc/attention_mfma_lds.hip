@@ -154,12 +154,18 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
 #pragma unroll
         for (int s = 0; s < S32; ++s) qf[nt][s].raw = ld16(qp + s * 32 + 8 * G);
     }
-    float m_run[NT], l_run[NT];
+    // the running sums of the probabilities come from the matrix cores too: a row of ones beside
+    // the values, so that every lane holds its row's whole sum (32 additions a block less for the
+    // vector unit, which is as busy as the matrix cores here; 1 to 2 % at long portions)
+    float m_run[NT];
+    floatx4 l_acc[NT];
+    F16B ones;
+    ones.raw = uint4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     floatx4 acc[NT][HDT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         m_run[nt] = -INFINITY;
-        l_run[nt] = 0.f;
+        l_acc[nt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dt = 0; dt < HDT; ++dt) acc[nt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
@@ -327,7 +333,11 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
         }
         if (__any(moved)) {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt) {
+                l_acc[nt][0] *= corr[nt];
+                l_acc[nt][1] *= corr[nt];
+                l_acc[nt][2] *= corr[nt];
+                l_acc[nt][3] *= corr[nt];
 #pragma unroll
                 for (int dt = 0; dt < HDT; ++dt) {
                     acc[nt][dt][0] *= corr[nt];
@@ -335,25 +345,21 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
                     acc[nt][dt][2] *= corr[nt];
                     acc[nt][dt][3] *= corr[nt];
                 }
+            }
         }
         // probabilities
         F16B pb[2][NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            float p_sum = 0.f;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 if (!use[h]) continue;
                 float p[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    p[i] = __builtin_amdgcn_exp2f(fmaf(sv[h][nt][i], scale2, shift[nt]));
-                    p_sum += p[i];
-                }
+                for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_exp2f(fmaf(sv[h][nt][i], scale2, shift[nt]));
                 pb[h][nt].raw = uint4{pack2_bf16(p[0], p[1]), pack2_bf16(p[2], p[3]), pack2_bf16(p[4], p[5]),
                                       pack2_bf16(p[6], p[7])};
             }
-            l_run[nt] = l_run[nt] * corr[nt] + p_sum;  // this lane's keys only; the lane groups are summed at the end
         }
         // O^T += V^T P^T
 #pragma unroll
@@ -364,10 +370,12 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
             for (int dt = 0; dt < HDT; ++dt)
                 vf[dt].raw = *reinterpret_cast<const uint4*>(vbuf + (dt * 16 + c) * VS + 32 * h + 8 * G);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt) {
+                l_acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pb[h][nt].v, l_acc[nt], 0, 0, 0);
 #pragma unroll
                 for (int dt = 0; dt < HDT; ++dt)
                     acc[nt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pb[h][nt].v, acc[nt][dt], 0, 0, 0);
+            }
         }
     };
 
@@ -394,8 +402,7 @@ __global__ __launch_bounds__(kLdsThreads) __attribute__((amdgpu_waves_per_eu(HDT
     if (!active) return;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        float l_tot = l_run[nt];
-        l_tot = sum_xor32(sum_xor16(l_tot));
+        const float l_tot = l_acc[nt][0];
         if (!rvalid[nt]) continue;
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         bf16_t* o = out + (static_cast<int64_t>(q_row0 + rtok[nt]) * n_heads + rhead[nt]) * HD + 4 * G;
