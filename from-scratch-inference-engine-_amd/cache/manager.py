@@ -205,3 +205,14 @@ class CacheManager:
         slots = [rc.slot for rc in self._live.values()]
         if len(slots) != len(set(slots)) or len(slots) + len(self._free_slots) != self.max_requests:
             raise AssertionError("state slots lost or held twice")
+
+
+def pages_that_fit(free_bytes: int, bytes_per_token: int, page_size: int, fraction: float = 0.9,
+                   reserve_bytes: int = 2 << 30) -> int:
+    """Pages a pool can have when it may take ``fraction`` of ``free_bytes`` less ``reserve_bytes``
+    (what a step's activations, the captured graphs and the library's workspaces need beside it);
+    ``bytes_per_token`` is what one token holds in all groups and layers together.  At least one."""
+    if bytes_per_token <= 0 or page_size <= 0:
+        raise ValueError("pages_that_fit: bytes_per_token and page_size must be positive")
+    room = int(free_bytes * fraction) - int(reserve_bytes)
+    return max(1, room // (bytes_per_token * page_size))

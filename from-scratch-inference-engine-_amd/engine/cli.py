@@ -22,7 +22,8 @@ def _common(p: argparse.ArgumentParser) -> None:
                    help="with --config: random weights made on the device from this seed")
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     p.add_argument("--block-size", type=int, default=16)
-    p.add_argument("--num-blocks", type=int, default=2048)
+    p.add_argument("--num-blocks", type=int, default=2048,
+                   help="pages in the cache pool (0: as many as the free device memory holds)")
     p.add_argument("--max-batch", type=int, default=256)
     p.add_argument("--max-tokens-per-step", type=int, default=2048)
     p.add_argument("--prefill-chunk", type=int, default=None,

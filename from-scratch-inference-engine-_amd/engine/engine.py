@@ -32,13 +32,16 @@ class Engine:
     ``step``, ``has_work``, ``output``, ``status``, ``preemptions`` and ``generate`` as in the
     reference (bindings/module.cpp:103-147, include/engine/engine.hpp:36-89).  Added:
     ``max_tokens_per_step`` (token budget of a step), ``prefill_chunk`` (longest portion of a
-    prompt in one step) and ``fill_rows`` (see ``Runner``).  ``enable_prefix_cache`` is accepted for compatibility; prefix caching
+    prompt in one step) and ``fill_rows`` (see ``Runner``); ``num_blocks=0`` makes the pool as large
+    as the device's free memory allows (``Model.pages_that_fit``).  ``enable_prefix_cache`` is accepted for compatibility; prefix caching
     is not part of this engine and the flag changes nothing."""
 
     def __init__(self, model: Model, block_size: int = 16, num_blocks: int = 2048, seed: int = 0,
                  max_batch: int = 256, enable_prefix_cache: bool = False, *, max_tokens_per_step: int = 2048,
                  prefill_chunk: Optional[int] = None, fill_rows=None):
         self.model = model
+        if num_blocks <= 0:
+            num_blocks = model.pages_that_fit(block_size)
         self.runner = Runner(model, page_size=block_size, num_pages=num_blocks, max_requests=max_batch,
                              fill_rows=fill_rows)
         self.scheduler = Scheduler(self.runner.manager, max_batch=max_batch,

@@ -25,7 +25,7 @@ class LLM:
     """Load a model folder and generate through the engine.
 
     Options of the reference keep their names and meanings: ``block_size`` (tokens per cache
-    page), ``num_blocks`` (pages in the pool), ``seed`` (sampling), ``max_batch`` (most requests
+    page), ``num_blocks`` (pages in the pool; 0: as many as the free device memory holds), ``seed`` (sampling), ``max_batch`` (most requests
     running at once), ``eos_id`` (default: read from the folder).  ``dtype`` ('bfloat16' or
     'float32'), ``max_tokens_per_step``, ``prefill_chunk``, ``tune_gemms`` and ``weight_copies`` (keep
     the large matrices a second time in the order the decode kernels read them: twice the memory,

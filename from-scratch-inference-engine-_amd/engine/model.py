@@ -157,6 +157,22 @@ class Model:
         return sum(need.bytes_per_token(self.dtype) * len(ids)
                    for need, ids in zip(self.cache_layout.paged_groups, self.cache_layout.group_caches))
 
+    def pages_that_fit(self, page_size: int) -> int:
+        """Pages of ``page_size`` tokens that the device's free memory holds beside what is loaded
+        (nine tenths of it, less 2 GiB for a step's activations, graphs and workspaces), and no
+        more than keep every layer's pools below 2^31 elements (pools beyond that can be asked for
+        by their number of pages; none has been run)."""
+        from ..cache.manager import pages_that_fit
+
+        per_token = self.cache_bytes_per_token()
+        if per_token <= 0:
+            raise ValueError("the cache's needs do not say how many bytes a token takes: give the number of pages")
+        free, _ = torch.cuda.mem_get_info(self.device)
+        pages = pages_that_fit(free, per_token, page_size)
+        itemsize = torch.empty((), dtype=self.dtype).element_size()
+        per_layer = max(need.bytes_per_token(self.dtype) for need in self.cache_layout.paged_groups) // itemsize
+        return max(1, min(pages, (2 ** 31 - 1) // max(1, per_layer * page_size)))
+
     # ---------------------------------------------------------------- compute
     def forward(self, ctx: StepContext, storage: CacheStorage) -> torch.Tensor:
         """float32 logits [wanted, vocab] for the step described by ``ctx``."""

@@ -166,3 +166,15 @@ def test_groups_with_page_geometries_of_their_own():
     m.check_invariants()
     m.close(rc)
     assert [a.num_free for a in m.allocators] == [16, 5, 5]
+
+
+def test_pages_that_fit_the_free_memory():
+    from from_scratch_inference_engine_amd.cache.manager import pages_that_fit
+
+    gib = 1 << 30
+    # nine tenths of 100 GiB less the reserve of 2 GiB, in pages of 16 tokens of 57,344 bytes
+    assert pages_that_fit(100 * gib, 57344, 16) == (int(100 * gib * 0.9) - 2 * gib) // (57344 * 16)
+    assert pages_that_fit(100 * gib, 57344, 16, fraction=0.5, reserve_bytes=0) == 50 * gib // (57344 * 16)
+    assert pages_that_fit(gib, 57344, 16) == 1  # nothing left beside the reserve: one page, and the pool will say so
+    with pytest.raises(ValueError):
+        pages_that_fit(gib, 0, 16)

@@ -78,6 +78,27 @@ def test_llm_from_a_configuration_alone(tmp_path):
     assert load_config(d).to_dict()["vocab_size"] == raw["vocab_size"]
 
 
+def test_a_pool_as_large_as_the_free_memory(model_dirs, monkeypatch):
+    """``num_blocks=0``: the pool takes nine tenths of the device's free memory less 2 GiB (here of a
+    free memory that the test states), and generation from it is what a small pool gives."""
+    from from_scratch_inference_engine_amd import LLM, GenerationConfig
+
+    gib = 1 << 30
+    monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (3 * gib, 288 * gib))
+    llm = LLM(model_dirs["A"], dtype="float32", block_size=16, num_blocks=0)
+    per_token = llm.model.cache_bytes_per_token()
+    cfg = helpers.TINY_A
+    layers, kv, hd = cfg["num_hidden_layers"], cfg["num_key_value_heads"], cfg["hidden_size"] // cfg["num_attention_heads"]
+    assert per_token == layers * 2 * kv * hd * 4
+    pages = llm.engine.runner.manager.allocators[0].num_pages
+    assert pages == (int(3 * gib * 0.9) - 2 * gib) // (per_token * 16)
+    monkeypatch.undo()
+    prompt = helpers.token_ids(cfg["vocab_size"], 11, 5)
+    small = LLM(model_dirs["A"], dtype="float32", block_size=16, num_blocks=8)
+    gen = GenerationConfig(max_tokens=10, temperature=0.0)
+    assert llm.generate_ids(prompt, gen) == small.generate_ids(prompt, gen) == plain_greedy(model_dirs["A"], prompt, 10)
+
+
 def test_eos_from_the_folder_stops_generation(llms, model_dirs):
     from from_scratch_inference_engine_amd import GenerationConfig
 
