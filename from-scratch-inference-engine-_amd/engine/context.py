@@ -70,8 +70,8 @@ class HostBatch:
         self.seq_slots = [e.cache.slot for e in entries]
         # the slots of the requests that start in this step (their per-request memory is reset), -1 for the others
         self.reset_slots = [e.cache.slot if e.cache.length == 0 else -1 for e in entries]
-        self.token_ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64,
-                                     count=self.n_tokens)
+        self.token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64).reshape(-1) for e in entries]
+                                        ) if entries else np.zeros(0, np.int64)
         self.positions = np.concatenate(
             [np.arange(p, p + n, dtype=np.int32) for p, n in zip(self.past_lens, self.q_lens)]
         ) if entries else np.zeros(0, np.int32)

@@ -179,7 +179,8 @@ class AttentionPlanner:
         small_tokens, large_tokens, most = self.geometry(mfma)
         padded = getattr(host, "pad", None) is not None
         split_keys = host.pad[self.key][2] if padded else self.split_keys(host, mfma)
-        small, large, merges = [], [], []
+        small, merges = [], []
+        large_runs = []  # per long portion: its tiles as rows of an array (a prompt of thousands of tokens has hundreds)
         n_partial = 0
         for s in range(host.n_seqs):
             n, p, row0 = host.q_lens[s], host.past_lens[s], host.q_starts[s]
@@ -197,21 +198,29 @@ class AttentionPlanner:
             elif n <= small_tokens:
                 small.append((s, row0, n, p, first_key, total, -1, 0))
             else:
-                for t0 in range(0, n, large_tokens):
-                    nq = min(large_tokens, n - t0)
-                    pos0 = p + t0
-                    kb = max(0, pos0 - self.window + 1) if self.window else 0
-                    # (the short tile that a long portion may end with stays with the portion's other tiles:
-                    # as a small item it would walk all the portion's keys in one workgroup a kv head, alone
-                    # on the device, while as the last of a group of four it shares their blocks of keys)
-                    large.append((s, row0 + t0, nq, pos0, kb, pos0 + nq, -1, 0))
+                # (the short tile that a long portion may end with stays with the portion's other tiles:
+                # as a small item it would walk all the portion's keys in one workgroup a kv head, alone
+                # on the device, while as the last of a group of four it shares their blocks of keys)
+                t0 = np.arange(0, n, large_tokens, dtype=np.int64)
+                run = np.empty((t0.shape[0], ATTN_ITEM_INTS), dtype=np.int64)
+                pos0 = p + t0
+                run[:, 0] = s
+                run[:, 1] = row0 + t0
+                run[:, 2] = np.minimum(large_tokens, n - t0)
+                run[:, 3] = pos0
+                run[:, 4] = np.maximum(0, pos0 - self.window + 1) if self.window else 0
+                run[:, 5] = pos0 + run[:, 2]
+                run[:, 6] = -1
+                run[:, 7] = 0
+                large_runs.append(run)
+        large = np.concatenate(large_runs) if large_runs else np.zeros((0, ATTN_ITEM_INTS), dtype=np.int64)
         waves = 1
         if mfma and small:
             waves = self._waves_for(max(it[5] - it[4] for it in small), ops.attention_mfma_max_waves(self.head_dim))
         if padded:
             # a captured graph launches fixed grids: pad with items and merges that do nothing
             n_items, waves, _ = host.pad[self.key]
-            if large or len(small) > n_items:
+            if len(large) or len(small) > n_items:
                 raise RuntimeError("attention plan does not fit the captured graph")
             small += [(0, 0, 0, 0, 0, 0, -1, 0)] * (n_items - len(small))
             if n_items > host.n_seqs:
@@ -222,27 +231,31 @@ class AttentionPlanner:
                 n_partial = n_items * small_tokens
         # consecutive large tiles of one request, four at a time, for the kernel that shares the
         # keys of a block among four waves
-        groups = []
-        if mfma:
-            for i, it in enumerate(large):
-                if groups and groups[-1][1] < 4 and large[i - 1][0] == it[0] and large[i - 1][3] < it[3]:
-                    groups[-1][1] += 1
-                else:
-                    groups.append([i, 1])
+        groups = np.zeros((0, 2), dtype=np.int64)
+        if mfma and large_runs:
+            firsts, counts, at = [], [], 0
+            for run in large_runs:
+                f = np.arange(0, run.shape[0], 4, dtype=np.int64)
+                firsts.append(at + f)
+                counts.append(np.minimum(4, run.shape[0] - f))
+                at += run.shape[0]
+            firsts, counts = np.concatenate(firsts), np.concatenate(counts)
             # by the number of keys a group goes through, ascending: the kernel starts its workgroups
             # from the back of this list, the longest first (with several requests in a step the
             # order of the requests would otherwise decide)
-            groups.sort(key=lambda g: large[g[0] + g[1] - 1][5] - large[g[0]][4])
+            order = np.argsort(large[firsts + counts - 1, 5] - large[firsts, 4], kind="stable")
+            groups = np.stack([firsts[order], counts[order]], axis=1)
         n_long = 0
         if mfma and self.long_keys is not None:
             # large tiles that read more than ``long_keys`` keys go to workgroups of four waves
-            long_ones = [it for it in large if it[5] - it[4] > self.long_keys]
-            large = [it for it in large if it[5] - it[4] <= self.long_keys] + long_ones
-            n_long = len(long_ones)
+            is_long = large[:, 5] - large[:, 4] > self.long_keys
+            large = np.concatenate([large[~is_long], large[is_long]])
+            n_long = int(is_long.sum())
+        small_items = np.asarray(small, dtype=np.int64).reshape(-1, ATTN_ITEM_INTS)
         return {
-            "items": np.asarray(small + large, dtype=np.int32).reshape(-1, ATTN_ITEM_INTS),
+            "items": np.concatenate([small_items, large]).astype(np.int32),
             "merges": np.asarray(merges, dtype=np.int32).reshape(-1, ATTN_MERGE_INTS),
-            "groups": np.asarray(groups, dtype=np.int32).reshape(-1, 2), "n_groups": len(groups),
+            "groups": groups.astype(np.int32), "n_groups": len(groups),
             "n_small": len(small), "n_large": len(large) - n_long, "n_long": n_long, "n_merges": len(merges),
             "n_partial": n_partial, "mfma": mfma, "waves": waves,
             "single": all(host.q_lens[s] == 1 for s in range(host.n_seqs)),  # one token a request
