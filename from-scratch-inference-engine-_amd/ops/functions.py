@@ -28,7 +28,14 @@ def dtype_code(dtype: torch.dtype) -> int:
     raise KernelError(f"kernels take float32 or bfloat16, not {dtype}")
 
 
+# the current stream's handle straight from the runtime where torch offers it: the Stream object that
+# torch.cuda.current_stream() builds costs some 10 us, and every kernel launch asks for it
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
