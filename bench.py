@@ -239,6 +239,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (named in config)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="7b", help="layer sizes (default: 28 layers of 3584 / 18944)")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
+    ap.add_argument("--max-positions", type=int, default=None,
+                    help="position limit of the model (default: the shape's; raise it for prompts beyond that)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-kernels", action="store_true", help="skip the time of each class of kernels of a decode step")
     ap.add_argument("--no-tune", action="store_true", help="leave the library's kernel choice for prefill to its heuristic")
@@ -279,6 +281,8 @@ def main() -> int:
     full_layers = raw["num_hidden_layers"]
     layers = args.layers or full_layers
     raw["num_hidden_layers"] = layers
+    if args.max_positions:
+        raw["max_position_embeddings"] = args.max_positions
     cfg = parse_config(raw)
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     itemsize = 2 if args.dtype == "bf16" else 4

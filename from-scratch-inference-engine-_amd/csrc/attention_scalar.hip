@@ -239,19 +239,27 @@ __global__ __launch_bounds__(256) void attention_scalar_kernel(
 
 // Combine the partial records of one query token in the fixed order of its splits.
 // merge item: {out_row, first_slot, n_splits, slot_stride}
-// One wave per (token, head).  The maxima and denominators of up to 64 splits are read by one
-// lane each, and the sums of a dimension are loaded several splits ahead of their use: a loop
-// that waits for each record in turn costs a memory latency per split (28 splits took longer
-// than the attention itself).
+// One workgroup per (token, head).  Up to kMergeWideFrom splits are one wave's work (the other
+// three leave at once): the maxima and denominators of up to 64 splits are read by one lane each,
+// and the sums of a dimension are loaded several splits ahead of their use: a loop that waits for
+// each record in turn costs a memory latency per split (28 splits took longer than the attention
+// itself).  More splits (one request of 100,000 keys is cut into more than a hundred items) are
+// dealt to the four waves in runs, which add their sums up through LDS in the order of the waves.
+constexpr int kMergeWideFrom = 32;
+
 template <typename T, int DIMS>
-__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ partials,
-                                                             const int32_t* __restrict__ merges, T* __restrict__ out,
-                                                             int n_heads, int hd) {
+__global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ partials,
+                                                              const int32_t* __restrict__ merges, T* __restrict__ out,
+                                                              int n_heads, int hd) {
+    __shared__ float handed[3][DIMS * 64 + 1];  // of waves 1 to 3: the sums, then the denominator
     const int32_t* mi = merges + static_cast<int64_t>(blockIdx.x) * FSIE_ATTN_MERGE_INTS;
     const int out_row = mi[0], first = mi[1], n_splits = mi[2], stride = mi[3];
     if (n_splits <= 0) return;
     const int hq = blockIdx.y;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const bool wide = n_splits > kMergeWideFrom;  // the same for the whole workgroup
+    if (!wide && wave > 0) return;
     const int64_t rec_size = hd + 2;
     const float* rec0 = partials + (static_cast<int64_t>(first) * n_heads + hq) * rec_size;
     const int64_t rec_step = static_cast<int64_t>(stride) * n_heads * rec_size;
@@ -287,21 +295,28 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __rest
             }
         }
     } else {
-        float m = -INFINITY;
+        float m = -INFINITY;  // over all splits, in every wave
         for (int base = 0; base < n_splits; base += 64) {
             const int s = base + lane;
             m = fmaxf(m, s < n_splits ? rec0[s * rec_step + hd] : -INFINITY);
         }
         m = wave_max(m);
-        for (int base = 0; base < n_splits; base += 64) {
+        // this wave's run of the splits: all of them, or a quarter
+        int s_begin = 0, s_end = n_splits;
+        if (wide) {
+            const int run = (n_splits + 3) / 4;
+            s_begin = wave * run;
+            s_end = min(n_splits, s_begin + run);
+        }
+        for (int base = s_begin; base < s_end; base += 64) {
             const int s = base + lane;
             float w = 0.f, l = 0.f;
-            if (s < n_splits) {
+            if (s < s_end) {
                 const float ms = rec0[s * rec_step + hd];
                 l = rec0[s * rec_step + hd + 1];
                 w = ms == -INFINITY ? 0.f : expf(ms - m);
             }
-            const int here = min(64, n_splits - base);
+            const int here = min(64, s_end - base);
             const float* rec = rec0 + base * rec_step;
             for (int j0 = 0; j0 < here; j0 += AHEAD) {
                 float v[AHEAD][DIMS];
@@ -325,6 +340,21 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __rest
             }
         }
     }
+    if (wide) {
+        if (wave > 0) {
+#pragma unroll
+            for (int i = 0; i < DIMS; ++i) handed[wave - 1][i * 64 + lane] = a[i];
+            if (lane == 0) handed[wave - 1][DIMS * 64] = denom;
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < 3; ++w) {
+            denom += handed[w][DIMS * 64];
+#pragma unroll
+            for (int i = 0; i < DIMS; ++i) a[i] += handed[w][i * 64 + lane];
+        }
+    }
     const float inv = denom > 0.f ? 1.0f / denom : 0.f;
 #pragma unroll
     for (int i = 0; i < DIMS; ++i) {
@@ -337,9 +367,9 @@ template <typename T>
 void launch_merge(const float* partials, const int32_t* merges, int n_merges, T* out, int n_heads, int hd,
                   hipStream_t stream) {
     const dim3 grid(n_merges, n_heads);
-    if (hd <= 64) attention_merge_kernel<T, 1><<<grid, 64, 0, stream>>>(partials, merges, out, n_heads, hd);
-    else if (hd <= 128) attention_merge_kernel<T, 2><<<grid, 64, 0, stream>>>(partials, merges, out, n_heads, hd);
-    else attention_merge_kernel<T, 4><<<grid, 64, 0, stream>>>(partials, merges, out, n_heads, hd);
+    if (hd <= 64) attention_merge_kernel<T, 1><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd);
+    else if (hd <= 128) attention_merge_kernel<T, 2><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd);
+    else attention_merge_kernel<T, 4><<<grid, 256, 0, stream>>>(partials, merges, out, n_heads, hd);
 }
 
 }  // namespace

@@ -132,6 +132,24 @@ class AttentionPlanner:
                 while long > longest and sum(max(1, k // long) for k in keys) * per_item < units:
                     long //= 2
             split = long
+        # More workgroups than units run in rounds, and a last round that is mostly empty costs as
+        # much as a full one (one request of 100,000 keys in items of 1,024: 392 workgroups on 256
+        # units, two rounds of which the second is half empty).  The items then shorten, in steps of
+        # 32 keys and to no less than half, as far as the same number of rounds still holds all their
+        # workgroups (800 keys there: 504 workgroups, and each a fifth shorter).
+        if self.fill_rounds and mfma and keys and units > 0:
+            def groups_of(length):
+                return sum(-(-k // length) for k in keys) * per_item
+            now = groups_of(split)
+            rounds = -(-now // units)
+            if now > units and now * 10 < rounds * units * 9:
+                shorter = split
+                for length in range(split - 32, split // 2 - 1, -32):
+                    if groups_of(length) > rounds * units:
+                        break
+                    shorter = length
+                if groups_of(shorter) > now:  # (shorter items that are no more items gain nothing)
+                    split = shorter
         return split
 
     long_items = True  # items beyond the longest of `geometry` where they still fill the device
@@ -139,6 +157,8 @@ class AttentionPlanner:
     # never, which is faster: the one-wave item asks for all its blocks of keys at once, a wave of the
     # many-wave workgroup for two at a time.
     whole_requests = 0
+    # items shorten so that the last round of their workgroups is a full one (see split_keys)
+    fill_rounds = True
 
     @staticmethod
     def _items_of(keys: int, split_keys: int, longest: int) -> int:

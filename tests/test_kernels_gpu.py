@@ -843,10 +843,11 @@ def test_attention_finds_one_far_key_and_respects_edges(ops, dtype, scalar):
 @pytest.mark.parametrize("heads, hd, dtype", [(3, 32, torch.float32), (5, 80, torch.bfloat16), (28, 128, torch.bfloat16),
                                              (2, 256, torch.float32)])
 def test_attention_merge_alone(ops, heads, hd, dtype):
-    """Records of 1 to 130 splits (more than the 64 that one pass of the wave reads), some of them
-    empty (maximum -inf), one token's records a stride apart, against the sums written out."""
+    """Records of 1 to 257 splits (up to 32 are one wave's work, more are dealt to four waves in runs,
+    a run of more than 64 takes a wave two passes), some of them empty (maximum -inf), one token's
+    records a stride apart, against the sums written out."""
     g = torch.Generator().manual_seed(hd)
-    splits = [1, 2, 3, 9, 64, 65, 130]
+    splits = [1, 2, 3, 9, 32, 33, 64, 65, 130, 257]
     stride = 2  # two tokens of a portion lie side by side in every split
     slots = sum(n * stride for n in splits)
     rec = torch.randn(slots, heads, hd + 2, generator=g)
