@@ -105,7 +105,10 @@ class AttentionPlanner:
         # halved while the halves' workgroups still number at most the compute units: beyond that a
         # split only adds a merge.  The float32-arithmetic kernel's workgroups are slower and several
         # share a unit: twice the units.
-        while split > shortest and sum(-(-k // (split // 2)) for k in keys) * per_item < units * room:
+        # (the matrix-core kernel: up to exactly one workgroup a unit; four requests of 8,000 keys in 64 items of
+        # 512, 19.1 us, and not in 32 of 1,024, 23.3)
+        most_groups = units * room + (1 if mfma else 0)
+        while split > shortest and sum(-(-k // (split // 2)) for k in keys) * per_item < most_groups:
             split //= 2
         # requests that fit one item each need no merge at all while they stay whole: cutting them in
         # two is not worth one, in three or more it is
@@ -132,23 +135,41 @@ class AttentionPlanner:
                 while long > longest and sum(max(1, k // long) for k in keys) * per_item < units:
                     long //= 2
             split = long
-        # More workgroups than units run in rounds, and a last round that is mostly empty costs as
-        # much as a full one (one request of 100,000 keys in items of 1,024: 392 workgroups on 256
-        # units, two rounds of which the second is half empty).  The items then shorten, in steps of
-        # 32 keys and to no less than half, as far as the same number of rounds still holds all their
-        # workgroups (800 keys there: 504 workgroups, and each a fifth shorter).
+        # Two cases in which shorter items are faster, found by measuring (28/4 and 40/8 heads of 128):
+        # * more workgroups than units, in rounds of which the last is mostly empty (one request of
+        #   100,000 keys in items of 1,024: 392 workgroups on 256 units; 24 requests of 3,000 keys: 288).
+        #   The items shorten as far as the same number of rounds still holds all their workgroups.  Items
+        #   of less than a quarter of the length (the one key by which a request has passed a multiple)
+        #   do not count as workgroups here: they are over at once.
+        # * long items (twice the usual longest and more) whose workgroups leave the units half empty: a
+        #   unit holds two such workgroups, and 512 of 1,056 keys read faster than 256 of 2,048 (8 requests
+        #   of 16,500 keys).  The items shorten as far as two workgroups a unit allow.  Not where no
+        #   request is cut at all: 64 whole requests of 3,550 keys read at the memory's rate as they are, and
+        #   cut in two they only gain a merge (79.5 against 72.5 us).
+        # Both in steps of a 64th of the length (at least 32 keys) and to no less than half of it.
         if self.fill_rounds and mfma and keys and units > 0:
-            def groups_of(length):
-                return sum(-(-k // length) for k in keys) * per_item
-            now = groups_of(split)
-            rounds = -(-now // units)
-            if now > units and now * 10 < rounds * units * 9:
-                shorter = split
-                for length in range(split - 32, split // 2 - 1, -32):
-                    if groups_of(length) > rounds * units:
-                        break
-                    shorter = length
-                if groups_of(shorter) > now:  # (shorter items that are no more items gain nothing)
+            def groups_of(length, least=0):
+                return sum(k // length + (1 if k % length > least else 0) for k in keys) * per_item
+            everyone, large_ones = groups_of(split), groups_of(split, split // 4)
+            rounds = -(-large_ones // units)
+            room_for = 0
+            if large_ones > units and large_ones * 10 < rounds * units * 9:
+                room_for = rounds * units
+            elif split >= 2 * longest and everyone * 2 <= units * 3 and max(keys) > split:
+                room_for = 2 * units
+            if room_for:
+                step = max(32, split // 64 // 32 * 32)
+                # the shortest length on the grid whose workgroups still fit (their number only grows as
+                # the items shorten): by halving the range
+                lo, hi = 0, (split - split // 2) // step  # steps below `split`: lo fits, hi is the most
+                while lo < hi:
+                    mid = (lo + hi + 1) // 2
+                    if groups_of(split - mid * step) <= room_for:
+                        lo = mid
+                    else:
+                        hi = mid - 1
+                shorter = split - lo * step
+                if groups_of(shorter, shorter // 4) > large_ones:  # (shorter items that are no more items gain nothing)
                     split = shorter
         return split
 

@@ -136,12 +136,13 @@ def test_decode_items_shorten_while_compute_units_are_idle():
     # requests that by themselves give every unit a workgroup stay whole, however long: no item of 16 keys and no
     # merge for requests that have just passed 1,024; fewer long requests take the longest items of which the
     # full ones still number the units
-    # (where the workgroups of such items would leave the last of their rounds over the units mostly empty, the
-    # items shorten, in steps of 32 keys, until that round is full: 16 requests of 9,000 keys in 8 items of 1,152
-    # and not in 4 of 2,048 and one of 808; one request of 100,000 keys in 126 items of 800, not 98 of 1,024)
+    # (where the workgroups of such items would leave the last of their rounds over the units mostly empty, or
+    # long items leave the units half empty, the items shorten: 16 requests of 9,000 keys in 8 items of 1,152 and
+    # not in 4 of 2,048 and one of 808; one request of 100,000 keys in 125 items of 800, not 98 of 1,024; the four
+    # keys by which 48 requests have passed 4,096 do not count as workgroups, and whole requests stay whole)
     for n_requests, keys, split, items in ((64, 1040, 2048, 1), (64, 3500, 4096, 1), (80, 2000, 2048, 1), (64, 16000, 16384, 1),
-                                           (48, 2000, 1024, 2), (48, 4100, 1056, 4), (32, 3500, 1024, 4), (16, 9000, 1152, 8),
-                                           (8, 33000, 2080, 16), (1, 100000, 800, 125)):
+                                           (48, 2000, 1024, 2), (48, 4100, 2048, 3), (32, 3500, 1024, 4), (16, 9000, 1152, 8),
+                                           (8, 33000, 2112, 16), (1, 100000, 800, 125)):
         host = Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16)
         assert planner.split_keys(host, True) == split
         plan = planner.plan(host)
@@ -161,7 +162,7 @@ def test_decode_items_shorten_while_compute_units_are_idle():
     planner.fill_rounds = True
     wide = AttentionPlanner(40, 8, 128, None)
     wide.compute_units = 256
-    for n_requests, keys, split in ((8, 16000, 2048), (8, 16500, 2080), (32, 2300, 4096), (16, 4000, 1024), (8, 640, 256)):
+    for n_requests, keys, split in ((8, 16000, 2048), (8, 16500, 2112), (32, 2300, 4096), (16, 4000, 1024), (8, 640, 256)):
         assert wide.split_keys(Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16), True) == split
     planner.long_items = False
     assert planner.split_keys(Host([(3499, 1)] * 64, 16, torch.bfloat16), True) == 1024
