@@ -30,7 +30,7 @@ import torch
 
 from .context import HostBatch, StepEntry, build_context, filler_entry
 
-PAGE_BUCKET = 32  # block-table widths are rounded up to this many pages
+PAGE_BUCKET = 32  # block-table widths are at least this many pages (and powers of two)
 CAPTURE_AFTER = 3  # a shape is captured the n-th time it is asked for (read when a runner is made)
 
 
@@ -85,7 +85,9 @@ class DecodeGraphs:
         entries = self.filled_up(entries)
         host = HostBatch(entries, runner.manager.page_size, runner.model.dtype)
         pages = max(len(t) for e in entries for t in e.cache.tables) if runner.manager.groups else 1
-        pad = {"pages": -(-pages // PAGE_BUCKET) * PAGE_BUCKET}
+        # the width of the block tables: a power of two (at least PAGE_BUCKET pages), so that a batch whose
+        # requests grow changes graphs once per doubling and not every few hundred tokens
+        pad = {"pages": max(PAGE_BUCKET, 1 << (max(pages, 1) - 1).bit_length())}
         for planner in runner.model.planners:
             bucket = planner.graph_bucket(host)
             if bucket is None:

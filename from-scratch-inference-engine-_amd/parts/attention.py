@@ -67,8 +67,7 @@ class AttentionPlanner:
         return (compute_dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.head_dim <= 256
                 and page_size % 4 == 0)
 
-    @staticmethod
-    def _waves_for(keys: int, max_waves: int) -> int:
+    def _waves_for(self, keys: int, max_waves: int) -> int:
         """Waves of a workgroup for an item of ``keys`` keys: one per 128 keys, a power of two."""
         need = max(1, -(-keys // 128))
         w = 1
@@ -110,6 +109,16 @@ class AttentionPlanner:
         most_groups = units * room + (1 if mfma else 0)
         while split > shortest and sum(-(-k // (split // 2)) for k in keys) * per_item < most_groups:
             split //= 2
+        if self.fine_items and mfma and keys and split > shortest:
+            # between that length and its half: the shortest multiple of 32 whose workgroups still number at most the units
+            lo, hi = 0, (split - split // 2) // 32 - 1
+            while lo < hi:
+                mid = (lo + hi + 1) // 2
+                if sum(-(-k // (split - 32 * mid)) for k in keys) * per_item < most_groups:
+                    lo = mid
+                else:
+                    hi = mid - 1
+            split -= 32 * lo
         # requests that fit one item each need no merge at all while they stay whole: cutting them in
         # two is not worth one, in three or more it is
         if keys and split < longest and max(keys) <= longest and -(-max(keys) // split) <= 2:
@@ -180,6 +189,8 @@ class AttentionPlanner:
     whole_requests = 0
     # items shorten so that the last round of their workgroups is a full one (see split_keys)
     fill_rounds = True
+    # between a power of two and its half, the shortest items whose workgroups still number at most the units
+    fine_items = True
 
     @staticmethod
     def _items_of(keys: int, split_keys: int, longest: int) -> int:
@@ -206,12 +217,16 @@ class AttentionPlanner:
                 longest = max(longest, split_keys)
             n += mine
         if mfma:
-            # items: a multiple of the number of requests, and of what 1,024 keys of each need, so
-            # that a graph serves as many steps with short items as with long ones (the captured
-            # graph pads with empty items, whose workgroups leave at once)
-            step = host.n_seqs * max(1, 1024 // split_keys)
+            # items: a multiple of the number of requests and of a quarter of what gives every unit a
+            # workgroup, so that one graph serves a batch while its requests grow: their items grow
+            # longer, not more (the captured graph pads with empty items, whose workgroups leave at
+            # once).  The length of the items is data of the step, not of the graph.
+            units = self.compute_units if self.compute_units is not None else ops.compute_units()
+            group = self.n_heads // self.n_kv
+            per_item = self.n_kv * -(-group // min(group, ops.attention_mfma_rows(self.head_dim, False)))
+            step = max(host.n_seqs, units // per_item // 4, 1)
             return (-(-n // step) * step,
-                    self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)), split_keys)
+                    self._waves_for(longest, ops.attention_mfma_max_waves(self.head_dim)), 0)
         step = host.n_seqs * max(1, 1024 // split_keys)
         return (-(-n // step) * step, 1, split_keys)
 
@@ -219,7 +234,7 @@ class AttentionPlanner:
         mfma = self.uses_mfma(host.compute_dtype, host.page_size)
         small_tokens, large_tokens, most = self.geometry(mfma)
         padded = getattr(host, "pad", None) is not None
-        split_keys = host.pad[self.key][2] if padded else self.split_keys(host, mfma)
+        split_keys = self.split_keys(host, mfma)
         small, merges = [], []
         large_runs = []  # per long portion: its tiles as rows of an array (a prompt of thousands of tokens has hundreds)
         n_partial = 0

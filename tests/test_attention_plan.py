@@ -124,14 +124,17 @@ def test_plans_cover_every_key_once(dtype, page_size, heads, kv, hd, window):
 def test_decode_items_shorten_while_compute_units_are_idle():
     planner = AttentionPlanner(28, 4, 128, None)
     planner.compute_units = 256
-    for n_requests, keys, split in ((8, 640, 128), (1, 3550, 128), (64, 640, 1024), (8, 16000, 1024), (20, 3000, 1024), (12, 1500, 512),
-                                   (48, 600, 1024), (8, 3550, 512), (32, 600, 1024), (24, 600, 1024), (16, 640, 256)):
+    # (items halve while the halves' workgroups number at most the units, and between that length and its half
+    # they take the shortest multiple of 32 keys that still does: 12 requests of 1,500 keys in 5 items of 320)
+    for n_requests, keys, split, waves in ((8, 640, 128, 1), (1, 3550, 128, 1), (64, 640, 1024, 8), (8, 16000, 1024, 8),
+                                           (20, 3000, 1024, 8), (12, 1500, 320, 4), (48, 600, 1024, 8), (8, 3550, 448, 4),
+                                           (32, 600, 1024, 8), (24, 600, 1024, 8), (16, 640, 160, 2)):
         host = Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16)
         assert planner.split_keys(host, True) == split
         plan = planner.plan(host)
         check_plan(planner, host, plan)
         assert plan["n_small"] == n_requests * -(-keys // split)
-        assert plan["waves"] == {128: 1, 256: 2, 512: 4, 1024: 8}[split]  # one wave per 128 keys
+        assert plan["waves"] == waves  # one wave per 128 keys of the longest item, a power of two
         assert plan["n_merges"] == (n_requests if keys > split else 0)
     # requests that by themselves give every unit a workgroup stay whole, however long: no item of 16 keys and no
     # merge for requests that have just passed 1,024; fewer long requests take the longest items of which the
@@ -150,7 +153,7 @@ def test_decode_items_shorten_while_compute_units_are_idle():
         assert plan["n_small"] == n_requests * items and plan["waves"] == 8
         assert plan["n_merges"] == (n_requests if items > 1 else 0)
         bucket = planner.graph_bucket(host)
-        assert bucket[0] >= plan["n_small"] and bucket[1] == 8 and bucket[2] == split
+        assert bucket[0] >= plan["n_small"] and bucket[1] == 8
     # one very long request among short ones is cut, the short ones stay whole
     host = Host([(599, 1)] * 63 + [(99999, 1)], 16, torch.bfloat16)
     assert planner.split_keys(host, True) == 2048
@@ -162,7 +165,7 @@ def test_decode_items_shorten_while_compute_units_are_idle():
     planner.fill_rounds = True
     wide = AttentionPlanner(40, 8, 128, None)
     wide.compute_units = 256
-    for n_requests, keys, split in ((8, 16000, 2048), (8, 16500, 2112), (32, 2300, 4096), (16, 4000, 1024), (8, 640, 256)):
+    for n_requests, keys, split in ((8, 16000, 2048), (8, 16500, 2112), (32, 2300, 4096), (16, 4000, 1024), (8, 640, 160)):
         assert wide.split_keys(Host([(keys - 1, 1)] * n_requests, 16, torch.bfloat16), True) == split
     planner.long_items = False
     assert planner.split_keys(Host([(3499, 1)] * 64, 16, torch.bfloat16), True) == 1024
@@ -182,11 +185,12 @@ def test_graph_bucket_pads_plans_of_decode_steps():
     for lens in ([640] * 8, [5, 900, 1500, 3000], [2047, 2048, 2049]):
         host = Host([(p, 1) for p in lens], 16, torch.bfloat16)
         bucket = planner.graph_bucket(host)
-        assert bucket is not None and bucket[0] % len(lens) == 0
+        assert bucket is not None and bucket[0] >= len(lens)
         host.pad = {planner.key: bucket}
         plan = planner.plan(host)
         assert plan["n_small"] == bucket[0] and plan["n_large"] == 0 and plan["waves"] == bucket[1]
-        assert bucket[2] == planner.split_keys(host, True)
+        # (the length of the items is no part of what the graph fixes: a batch keeps its graph while its requests grow)
+        assert sum(1 for it in plan["items"] if it[NQ] > 0) <= bucket[0]
         real = [it for it in plan["items"] if it[NQ] > 0]
         assert sum(int(it[KE]) - int(it[KB]) for it in real) == sum(p + 1 for p in lens)
         if bucket[0] > len(lens):
