@@ -800,6 +800,47 @@ def test_decoding_against_contexts_that_are_split_and_merged(tmp_path, dtype):
         assert model.planners[0].split_keys(host, True) == 128
 
 
+def test_a_growing_batch_keeps_its_graph_while_its_items_grow_longer(tmp_path, monkeypatch):
+    """Three requests decode 260 tokens each through graphs on a device that the planner takes to
+    have six compute units, so that the rules for the length of attention items (halving, the
+    lengths between the powers of two, the shortening that fills the last round of workgroups) all
+    come into play at these small sizes: the items change their length many times, the graph of the
+    batch changes only when the tables or the waves of an item double, and every 20th token's logits
+    are those of the plain implementation."""
+    from from_scratch_inference_engine_amd import load_model
+    from from_scratch_inference_engine_amd.engine import graphs
+    from from_scratch_inference_engine_amd.engine.context import StepEntry
+    from from_scratch_inference_engine_amd.engine.model import Runner
+
+    monkeypatch.setattr(graphs, "CAPTURE_AFTER", 1)
+    cfg = dict(helpers.TINY_B, max_position_embeddings=2048)
+    d = helpers.make_model_dir(tmp_path / "grow", cfg, seed=23)
+    model = load_model(d, dtype="bfloat16")
+    planner = model.planners[0]
+    planner.compute_units = 6
+    n_decoded = 260
+    seqs = [helpers.token_ids(cfg["vocab_size"], n + n_decoded, 900 + n) for n in (200, 520, 1100)]
+    refs = [plain.forward_dir(d, ids).numpy() for ids in seqs]
+    runner = Runner(model, page_size=16, num_pages=176, max_requests=4)
+    assert runner.graphs.enabled
+    caches = [runner.manager.open(i) for i in range(len(seqs))]
+    runner.step([StepEntry(c, ids[:-n_decoded], []) for c, ids in zip(caches, seqs)])
+    lengths = set()
+    from types import SimpleNamespace
+    for t in range(n_decoded, 0, -1):
+        host = SimpleNamespace(n_seqs=3, q_lens=[1, 1, 1], past_lens=[len(ids) - t for ids in seqs])
+        lengths.add(planner.split_keys(host, True))
+        out = runner.step([StepEntry(c, [ids[-t]], [0]) for c, ids in zip(caches, seqs)])
+        if t % 20 == 1:
+            got = out.float().cpu().numpy()
+            for i, ref in enumerate(refs):
+                helpers.assert_close_to_plain(got[i:i + 1], ref[len(ref) - t:len(ref) - t + 1], "bfloat16",
+                                              f"request of {len(seqs[i])} tokens, {t} from its end")
+    print(f"item lengths {sorted(lengths)}, {runner.graphs.captures} graphs, {runner.graphs.replays} replays")
+    assert len(lengths) >= 3, f"the items were {sorted(lengths)} keys long"
+    assert runner.graphs.captures <= 4 and runner.graphs.replays >= n_decoded - 4
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("page_size", [3, 8])
 def test_sizes_the_fast_kernels_do_not_take_still_give_right_results(tmp_path, dtype, page_size):
