@@ -104,8 +104,7 @@ class AttentionPlanner:
         # halved while the halves' workgroups still number at most the compute units: beyond that a
         # split only adds a merge.  The float32-arithmetic kernel's workgroups are slower and several
         # share a unit: twice the units.
-        # (the matrix-core kernel: up to exactly one workgroup a unit; four requests of 8,000 keys in 64 items of
-        # 512, 19.1 us, and not in 32 of 1,024, 23.3)
+        # (the matrix-core kernel: up to exactly one workgroup a unit)
         most_groups = units * room + (1 if mfma else 0)
         while split > shortest and sum(-(-k // (split // 2)) for k in keys) * per_item < most_groups:
             split //= 2
@@ -144,17 +143,15 @@ class AttentionPlanner:
                 while long > longest and sum(max(1, k // long) for k in keys) * per_item < units:
                     long //= 2
             split = long
-        # Two cases in which shorter items are faster, found by measuring (28/4 and 40/8 heads of 128):
-        # * more workgroups than units, in rounds of which the last is mostly empty (one request of
-        #   100,000 keys in items of 1,024: 392 workgroups on 256 units; 24 requests of 3,000 keys: 288).
-        #   The items shorten as far as the same number of rounds still holds all their workgroups.  Items
-        #   of less than a quarter of the length (the one key by which a request has passed a multiple)
-        #   do not count as workgroups here: they are over at once.
+        # Two cases in which shorter items are faster (measured at 28/4 and 40/8 heads of 128):
+        # * more workgroups than units, in rounds of which the last is mostly empty: the items shorten
+        #   as far as the same number of rounds still holds all their workgroups.  Items of less than a
+        #   quarter of the length (the one key by which a request has passed a multiple) do not count
+        #   as workgroups here: they are over at once.
         # * long items (twice the usual longest and more) whose workgroups leave the units half empty: a
-        #   unit holds two such workgroups, and 512 of 1,056 keys read faster than 256 of 2,048 (8 requests
-        #   of 16,500 keys).  The items shorten as far as two workgroups a unit allow.  Not where no
-        #   request is cut at all: 64 whole requests of 3,550 keys read at the memory's rate as they are, and
-        #   cut in two they only gain a merge (79.5 against 72.5 us).
+        #   unit holds two such workgroups, so the items shorten as far as two a unit allow.  Not where
+        #   no request is cut at all: whole requests that fill the units read at the memory's rate as
+        #   they are, and cut in two they only gain a merge.
         # Both in steps of a 64th of the length (at least 32 keys) and to no less than half of it.
         if self.fill_rounds and mfma and keys and units > 0:
             def groups_of(length, least=0):
