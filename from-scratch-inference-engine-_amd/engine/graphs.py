@@ -3,10 +3,12 @@
 A decode step launches some ten kernels per layer, each a few microseconds long; queued one by
 one from Python they cost more host time than GPU time.  A step whose every request brings one
 token and wants its logits has a shape that depends only on the number of requests and, through
-the width of the block tables and the number of attention work items, on rounded-up context
-lengths.  For each such shape the whole forward is captured once into a graph that reads all
-its index tables from one fixed device buffer; a later step of the same shape copies its tables
-there and replays the graph.
+the width of the block tables (a power of two of pages) and the number of attention work items
+and their waves, on coarsely rounded context lengths: how long the items are is data of a step,
+so a batch keeps its graph while its requests grow, until the tables or the items double.  For
+each such shape the whole forward is captured once into a graph that reads all its index tables
+from one fixed device buffer; a later step of the same shape copies its tables there and replays
+the graph.
 
 The number of requests is rounded up as well (``padded_rows``): a batch that shrinks request by
 request as they finish would otherwise want a new graph, some tens of milliseconds of capture,
